@@ -1,0 +1,2 @@
+"""MI355X-native Muon / Dion optimizer step (drop-in for the `dion` package's single-GPU path)."""
+from .newton_schulz import zeropower_via_newtonschulz5  # noqa: F401

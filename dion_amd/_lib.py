@@ -1,0 +1,118 @@
+"""ctypes binding of `libdion_amd.so` (the C ABI declared in `include/dion_amd.h`).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdion_amd.so")
+
+BF16, F32, F64 = 0, 1, 2
+EPI_STORE, EPI_AXPBY = 0, 1
+
+_DTYPE_CODE = {torch.bfloat16: BF16, torch.float32: F32, torch.float64: F64}
+
+_ERRORS = {
+    -1: "bad argument (null pointer or non-positive size)",
+    -2: "alignment: dimensions/pitches must be multiples of 8 (bf16) or 4 (fp32) elements, pointers 16-byte aligned",
+    -3: "workspace too small",
+    -4: "unsupported dtype",
+    -5: "size beyond a documented limit",
+}
+
+_c = ctypes
+_vp, _i, _ll, _f, _sz = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float, _c.c_size_t
+_fp = _c.POINTER(_c.c_float)
+_vpp = _c.POINTER(_c.c_void_p)
+
+_SIGNATURES = {
+    "dion_amd_version": (_c.c_char_p, []),
+    "dion_amd_ns_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "dion_amd_newton_schulz": (_i, [_vp, _i, _ll, _i, _vp, _ll, _i, _i, _i, _i, _fp, _i, _f, _i, _i, _vp, _sz, _vp]),
+    "dion_amd_syrk": (_i, [_vp, _ll, _i, _vp, _ll, _i, _i, _i, _i, _i, _vp]),
+    "dion_amd_sym_poly": (_i, [_vp, _ll, _i, _vp, _ll, _i, _i, _i, _f, _f, _i, _i, _vp]),
+    "dion_amd_gemm": (_i, [_vp, _ll, _i, _i, _vp, _ll, _i, _i, _vp, _ll, _i, _vp, _ll, _i,
+                           _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _vp]),
+    "dion_amd_muon_workspace_bytes": (_sz, [_i, _i, _i]),
+    "dion_amd_muon_step": (_i, [_vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _f, _i, _f, _f, _fp, _i, _f, _i, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+class DionAmdError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library (once) and declare every prototype."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise DionAmdError(
+            f"{LIB_PATH} not found: the HIP extension is not built. Run `python -m dion_amd.build` "
+            "(there is no CPU or PyTorch fallback)."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def exported_symbols():
+    return list(_SIGNATURES)
+
+
+def check(rc, what):
+    if rc == 0:
+        return
+    if rc < 0:
+        raise DionAmdError(f"{what}: {_ERRORS.get(rc, 'error')} (code {rc})")
+    raise DionAmdError(f"{what}: HIP error {rc}")
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise DionAmdError(f"unsupported dtype {dtype}") from None
+
+
+def require_gpu(t, what):
+    if not t.is_cuda:
+        raise DionAmdError(
+            f"{what}: tensor is on {t.device}; the MI355X kernels need a GPU tensor (no CPU fallback)"
+        )
+
+
+def stream_ptr(device=None):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def float_array(values):
+    arr = (ctypes.c_float * len(values))(*values)
+    return arr
+
+
+def ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+class Workspace:
+    """A grow-only byte buffer taken from PyTorch's caching allocator (stream-ordered lifetime)."""
+
+    def __init__(self):
+        self._buf = None
+
+    def get(self, nbytes, device):
+        if self._buf is None or self._buf.numel() < nbytes or self._buf.device != device:
+            self._buf = None
+            self._buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        return self._buf

@@ -1,0 +1,255 @@
+// C ABI entry points (declared in include/dion_amd.h) and the host-side drivers that chain
+// the kernels of one Newton-Schulz / Muon bucket on a stream.
+#include "../../include/dion_amd.h"
+#include "common.h"
+#include "elementwise.h"
+
+namespace {
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Workspace carve-up for one chunk of `cb` wide matrices (mw x nw).
+struct NsLayout {
+  int mw, nw, tiles;
+  size_t esz;
+  size_t x_bytes, a_bytes, part_bytes;  // per matrix
+  size_t per_matrix;
+  NsLayout(int m, int n, int dtype) {
+    mw = m < n ? m : n;
+    nw = m < n ? n : m;
+    tiles = da_stage_tiles(m, n);
+    esz = dtype == DA_BF16 ? 2 : 4;
+    x_bytes = align_up((size_t)mw * nw * esz, 256);
+    a_bytes = align_up((size_t)mw * mw * esz, 256);
+    part_bytes = align_up((size_t)tiles * sizeof(float) + sizeof(float), 256);
+    per_matrix = 2 * x_bytes + 2 * a_bytes + part_bytes;
+  }
+  int chunk(int batch, size_t ws_bytes) const {
+    size_t c = ws_bytes / per_matrix;
+    if (c > (size_t)batch) c = batch;
+    if (c > DA_MAX_PTRS) c = DA_MAX_PTRS;
+    return (int)c;
+  }
+  size_t recommended(int batch) const {
+    size_t c = ((size_t)4 << 30) / per_matrix;
+    if (c < 1) c = 1;
+    if (c > (size_t)batch) c = batch;
+    if (c > DA_MAX_PTRS) c = DA_MAX_PTRS;
+    return c * per_matrix;
+  }
+};
+
+struct NsBuffers {
+  char *x0, *x1, *a, *b;
+  float *partials, *divisor;
+  NsBuffers(const NsLayout& L, void* ws, int cb) {
+    char* p = static_cast<char*>(ws);
+    x0 = p; p += L.x_bytes * cb;
+    x1 = p; p += L.x_bytes * cb;
+    a = p; p += L.a_bytes * cb;
+    b = p; p += L.a_bytes * cb;
+    partials = reinterpret_cast<float*>(p);
+    divisor = partials + (size_t)L.tiles * cb;
+  }
+};
+
+int gemm_any(const GemmDesc& d, int dtype, hipStream_t s) {
+  return dtype == DA_BF16 ? da_gemm_bf16(d, s) : da_gemm_f32(d, s);
+}
+
+// steps x { A = X X^T ; B = b A + c A A ; X' = a X + B X } on cb wide matrices.
+// Returns in *result which of x0 / x1 holds the final iterate.
+int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const float* coeffs, int steps,
+               int faithful, hipStream_t s, char** result) {
+  char* x = W.x0;
+  char* y = W.x1;
+  const long long sx = (long long)(L.x_bytes / L.esz), sa = (long long)(L.a_bytes / L.esz);
+  for (int it = 0; it < steps; ++it) {
+    const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
+    GemmDesc g{};
+    g.batch = cb; g.c_dtype = dtype; g.faithful = faithful;
+    // A = X X^T   (symmetric output, k = nw)
+    g.A = x; g.B = x; g.C = W.a; g.E = nullptr;
+    g.sA = sx; g.sB = sx; g.sC = sa; g.sE = 0;
+    g.lda = L.nw; g.ldb = L.nw; g.ldc = L.mw; g.lde = 0;
+    g.M = L.mw; g.N = L.mw; g.K = L.nw;
+    g.a_kstrided = 0; g.b_kstrided = 0; g.symmetric = 1;
+    g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
+    int rc = gemm_any(g, dtype, s);
+    if (rc) return rc;
+    // B = b A + c A A^T   (A symmetric, so A A = A A^T: both operands k-contiguous)
+    g.A = W.a; g.B = W.a; g.C = W.b; g.E = W.a;
+    g.sA = sa; g.sB = sa; g.sC = sa; g.sE = sa;
+    g.lda = L.mw; g.ldb = L.mw; g.ldc = L.mw; g.lde = L.mw;
+    g.M = L.mw; g.N = L.mw; g.K = L.mw;
+    g.epilogue = DA_EPI_AXPBY; g.s0 = b; g.s1 = c;
+    rc = gemm_any(g, dtype, s);
+    if (rc) return rc;
+    // X' = a X + B X   (B symmetric: k-contiguous; X is the k-strided operand)
+    g.A = W.b; g.B = x; g.C = y; g.E = x;
+    g.sA = sa; g.sB = sx; g.sC = sx; g.sE = sx;
+    g.lda = L.mw; g.ldb = L.nw; g.ldc = L.nw; g.lde = L.nw;
+    g.M = L.mw; g.N = L.nw; g.K = L.mw;
+    g.a_kstrided = 0; g.b_kstrided = 1; g.symmetric = 0;
+    g.epilogue = DA_EPI_AXPBY; g.s0 = a; g.s1 = 1.f;
+    rc = gemm_any(g, dtype, s);
+    if (rc) return rc;
+    char* t = x; x = y; y = t;
+  }
+  *result = x;
+  return DA_OK;
+}
+
+int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
+  int rc = da_norm_finish(W.partials, L.tiles, cb, eps, dtype == DA_BF16, W.divisor, s);
+  if (rc) return rc;
+  // x_bytes is padded per matrix; the pad is never read by the GEMMs, normalising it is harmless.
+  return da_normalize(W.x0, dtype, (long long)(L.x_bytes / L.esz), cb, W.divisor, s);
+}
+
+bool dtype_ok(int d) { return d == DA_BF16 || d == DA_F32; }
+
+}  // namespace
+
+extern "C" {
+
+const char* dion_amd_version(void) { return "dion_amd 0.1 (gfx950)"; }
+
+size_t dion_amd_ns_workspace_bytes(int batch, int m, int n, int compute_dtype) {
+  if (batch <= 0 || m <= 0 || n <= 0 || !dtype_ok(compute_dtype)) return 0;
+  return NsLayout(m, n, compute_dtype).recommended(batch);
+}
+
+int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int ldg, void* out, long long out_stride,
+                           int ldo, int batch, int m, int n, const float* coeffs, int steps, float eps,
+                           int compute_dtype, int faithful, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!G || !out || !coeffs || !workspace || batch <= 0 || m <= 0 || n <= 0 || steps < 0) return DA_ERR_ARG;
+  if (!dtype_ok(g_dtype) || !dtype_ok(compute_dtype)) return DA_ERR_DTYPE;
+  if ((m | n | ldg | ldo) & 7) return DA_ERR_ALIGN;
+  if ((g_stride | out_stride) & 7) return DA_ERR_ALIGN;
+  if (((uintptr_t)G | (uintptr_t)out | (uintptr_t)workspace) & 255) return DA_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const NsLayout L(m, n, compute_dtype);
+  const int chunk = L.chunk(batch, workspace_bytes);
+  if (chunk < 1) return DA_ERR_WORKSPACE;
+  const size_t gsz = g_dtype == DA_BF16 ? 2 : 4;
+  for (int b0 = 0; b0 < batch; b0 += chunk) {
+    const int cb = batch - b0 < chunk ? batch - b0 : chunk;
+    const NsBuffers W(L, workspace, cb);
+    DaStage st{};
+    for (int i = 0; i < cb; ++i)
+      st.g.p[i] = const_cast<char*>(static_cast<const char*>(G)) + (size_t)(b0 + i) * g_stride * gsz;
+    st.wide = W.x0; st.partials = W.partials;
+    st.batch = cb; st.rows = m; st.cols = n; st.ld = ldg;
+    st.g_dtype = g_dtype; st.m_dtype = g_dtype; st.w_dtype = compute_dtype;
+    st.mu = 0.f; st.nesterov = 0; st.muon = 0;
+    int rc = da_stage_wide(st, s);
+    if (rc) return rc;
+    rc = ns_normalize_chunk(L, W, cb, compute_dtype, eps, s);
+    if (rc) return rc;
+    char* res = nullptr;
+    rc = ns_iterate(L, W, cb, compute_dtype, coeffs, steps, faithful, s, &res);
+    if (rc) return rc;
+    DaUnstage us{};
+    for (int i = 0; i < cb; ++i) us.x.p[i] = static_cast<char*>(out) + (size_t)(b0 + i) * out_stride * L.esz;
+    us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = ldo;
+    us.x_dtype = compute_dtype; us.w_dtype = compute_dtype;
+    us.decay = 1.f; us.step = 1.f; us.muon = 0;
+    rc = da_unstage(us, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+int dion_amd_syrk(const void* A, long long a_stride, int lda, void* C, long long c_stride, int ldc, int batch, int m,
+                  int k, int dtype, void* stream) {
+  if (!dtype_ok(dtype)) return DA_ERR_DTYPE;
+  GemmDesc g{};
+  g.A = A; g.B = A; g.C = C; g.E = nullptr;
+  g.sA = a_stride; g.sB = a_stride; g.sC = c_stride;
+  g.lda = lda; g.ldb = lda; g.ldc = ldc;
+  g.M = m; g.N = m; g.K = k; g.batch = batch;
+  g.symmetric = 1; g.epilogue = DA_EPI_STORE; g.s1 = 1.f; g.faithful = 0; g.c_dtype = dtype;
+  return gemm_any(g, dtype, static_cast<hipStream_t>(stream));
+}
+
+int dion_amd_sym_poly(const void* A, long long a_stride, int lda, void* C, long long c_stride, int ldc, int batch,
+                      int m, float alpha, float beta, int dtype, int faithful, void* stream) {
+  if (!dtype_ok(dtype)) return DA_ERR_DTYPE;
+  if (A == C) return DA_ERR_ARG;  // mirrored stores would race with operand loads
+  GemmDesc g{};
+  g.A = A; g.B = A; g.C = C; g.E = A;
+  g.sA = a_stride; g.sB = a_stride; g.sC = c_stride; g.sE = a_stride;
+  g.lda = lda; g.ldb = lda; g.ldc = ldc; g.lde = lda;
+  g.M = m; g.N = m; g.K = m; g.batch = batch;
+  g.symmetric = 1; g.epilogue = DA_EPI_AXPBY; g.s0 = beta; g.s1 = alpha; g.faithful = faithful; g.c_dtype = dtype;
+  return gemm_any(g, dtype, static_cast<hipStream_t>(stream));
+}
+
+int dion_amd_gemm(const void* A, long long a_stride, int lda, int a_kstrided, const void* B, long long b_stride,
+                  int ldb, int b_kstrided, void* C, long long c_stride, int ldc, const void* E, long long e_stride,
+                  int lde, int batch, int M, int N, int K, int in_dtype, int c_dtype, int epilogue, float s0,
+                  float s1, int faithful, void* stream) {
+  if (!dtype_ok(in_dtype) || !dtype_ok(c_dtype)) return DA_ERR_DTYPE;
+  if (epilogue != DA_EPI_STORE && epilogue != DA_EPI_AXPBY) return DA_ERR_ARG;
+  GemmDesc g{};
+  g.A = A; g.B = B; g.C = C; g.E = epilogue == DA_EPI_AXPBY ? E : nullptr;
+  g.sA = a_stride; g.sB = b_stride; g.sC = c_stride; g.sE = e_stride;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.lde = lde;
+  g.M = M; g.N = N; g.K = K; g.batch = batch;
+  g.a_kstrided = a_kstrided != 0; g.b_kstrided = b_kstrided != 0; g.symmetric = 0;
+  g.epilogue = epilogue; g.s0 = s0; g.s1 = s1; g.faithful = faithful; g.c_dtype = c_dtype;
+  return gemm_any(g, in_dtype, static_cast<hipStream_t>(stream));
+}
+
+size_t dion_amd_muon_workspace_bytes(int batch, int m, int n) {
+  if (batch <= 0 || m <= 0 || n <= 0) return 0;
+  return NsLayout(m, n, DA_BF16).recommended(batch);
+}
+
+int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int batch, int m, int n, int x_dtype,
+                       int g_dtype, float mu, int nesterov, float decay, float adjusted_lr, const float* coeffs,
+                       int steps, float eps, int faithful, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!X || !G || !M || !coeffs || !workspace || batch <= 0 || m <= 0 || n <= 0 || steps < 0) return DA_ERR_ARG;
+  if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype)) return DA_ERR_DTYPE;
+  if ((m | n) & 7) return DA_ERR_ALIGN;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
+  for (int i = 0; i < batch; ++i) {
+    if (!X[i] || !G[i] || !M[i]) return DA_ERR_ARG;
+    if (((uintptr_t)X[i] | (uintptr_t)G[i] | (uintptr_t)M[i]) & 15) return DA_ERR_ALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const NsLayout L(m, n, DA_BF16);
+  const int chunk = L.chunk(batch, workspace_bytes);
+  if (chunk < 1) return DA_ERR_WORKSPACE;
+  for (int b0 = 0; b0 < batch; b0 += chunk) {
+    const int cb = batch - b0 < chunk ? batch - b0 : chunk;
+    const NsBuffers W(L, workspace, cb);
+    DaStage st{};
+    for (int i = 0; i < cb; ++i) {
+      st.g.p[i] = const_cast<void*>(G[b0 + i]);
+      st.mom.p[i] = M[b0 + i];
+    }
+    st.wide = W.x0; st.partials = W.partials;
+    st.batch = cb; st.rows = m; st.cols = n; st.ld = n;
+    st.g_dtype = g_dtype; st.m_dtype = x_dtype; st.w_dtype = DA_BF16;
+    st.mu = mu; st.nesterov = nesterov; st.muon = 1;
+    int rc = da_stage_wide(st, s);
+    if (rc) return rc;
+    rc = ns_normalize_chunk(L, W, cb, DA_BF16, eps, s);
+    if (rc) return rc;
+    char* res = nullptr;
+    rc = ns_iterate(L, W, cb, DA_BF16, coeffs, steps, faithful, s, &res);
+    if (rc) return rc;
+    DaUnstage us{};
+    for (int i = 0; i < cb; ++i) us.x.p[i] = X[b0 + i];
+    us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = n;
+    us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
+    us.decay = decay; us.step = adjusted_lr; us.muon = 1;
+    rc = da_unstage(us, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+}  // extern "C"

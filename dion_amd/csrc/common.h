@@ -1,0 +1,91 @@
+// Shared declarations for the gfx950 kernels of the Muon / Dion optimizer step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+// ---- error codes of the C ABI (0 ok, <0 bad argument, >0 hipError_t) -------------
+#define DA_OK 0
+#define DA_ERR_ARG (-1)        // null pointer / non-positive size
+#define DA_ERR_ALIGN (-2)      // a dimension or leading dimension breaks an alignment rule
+#define DA_ERR_WORKSPACE (-3)  // workspace too small
+#define DA_ERR_DTYPE (-4)      // unsupported dtype code
+#define DA_ERR_LIMIT (-5)      // size beyond a documented maximum
+
+// ---- dtype codes -------------------------------------------------------------------
+#define DA_BF16 0
+#define DA_F32 1
+#define DA_F64 2
+
+typedef uint16_t bf16_t;  // storage type; arithmetic always goes through float
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+
+#define DA_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// Round-to-nearest-even float -> bf16 storage bits, and back.
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  __bf16 h = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, h);
+}
+__device__ __forceinline__ float bf2f(bf16_t h) {
+  return __builtin_bit_cast(float, ((uint32_t)h) << 16);
+}
+// Round a float to bf16 precision and keep it as float (one rounding point of the
+// reference's op-by-op bf16 arithmetic).
+__device__ __forceinline__ float rbf(float f) { return bf2f(f2bf(f)); }
+
+template <typename T> __device__ __forceinline__ float ld_as_float(const T* p);
+template <> __device__ __forceinline__ float ld_as_float<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ld_as_float<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void st_from_float(T* p, float v);
+template <> __device__ __forceinline__ void st_from_float<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void st_from_float<float>(float* p, float v) { *p = v; }
+
+#define DA_HIP_CHECK(expr)                       \
+  do {                                           \
+    hipError_t e__ = (expr);                     \
+    if (e__ != hipSuccess) return (int)e__;      \
+  } while (0)
+
+static inline int da_launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? DA_OK : (int)e;
+}
+
+// ---- GEMM descriptor shared by the bf16 / f32 / f64 kernels -------------------------
+// C[b] (M x N) = epilogue( sum_k Aop[b](i,k) * Bop[b](j,k) ).
+// An operand is either "k-contiguous" (stored rows x K, ld = row pitch) or
+// "k-strided" (stored K x rows, ld = k pitch).  All pitches / strides in elements.
+struct GemmDesc {
+  const void* A;
+  const void* B;
+  void* C;
+  const void* E;      // epilogue operand (same shape / layout as C), may be null
+  long long sA, sB, sC, sE;  // batch strides
+  int lda, ldb, ldc, lde;
+  int M, N, K;
+  int batch;
+  int a_kstrided, b_kstrided;
+  int symmetric;      // 1: C is symmetric (M == N); compute upper tiles and mirror
+  int epilogue;       // DA_EPI_*
+  int faithful;       // 1: reproduce every bf16 rounding of the op-by-op reference
+  float s0, s1;       // epilogue scalars
+  int c_dtype;        // dtype of C / E for the f32 and f64 kernels' mixed outputs
+};
+
+// Epilogues.  With `faithful` set the rounding points of the reference's separate
+// tensor ops are reproduced: t = r_in(acc); t = r_in(s1 * t) (skipped when s1 == 1);
+// e = r_c(s0 * E); C = r_c(e + t), where r_in rounds to the GEMM's input dtype (the
+// dtype a library matmul would have returned) and r_c to C's dtype.  Otherwise
+// C = r_c(s0 * E + s1 * acc) with a single rounding.
+#define DA_EPI_STORE 0  // C = s1 * acc
+#define DA_EPI_AXPBY 1  // C = s0 * E + s1 * acc; E may alias C (in-place update)
+
+int da_gemm_bf16(const GemmDesc& d, hipStream_t stream);
+int da_gemm_f32(const GemmDesc& d, hipStream_t stream);

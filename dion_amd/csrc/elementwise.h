@@ -1,0 +1,37 @@
+// Host-side launch descriptors for the HBM-bound passes (see elementwise.hip).
+#pragma once
+#include "common.h"
+
+#define DA_MAX_PTRS 64  // matrices per launch: pointer tables travel as kernel arguments
+
+struct DaPtrTable {
+  void* p[DA_MAX_PTRS];
+};
+
+struct DaStage {
+  DaPtrTable g;      // source matrices (rows x cols, row pitch ld)
+  DaPtrTable mom;    // momentum buffers (contiguous rows x cols), Muon mode only
+  void* wide;        // [batch][min(rows,cols)][max(rows,cols)] working matrices
+  float* partials;   // [batch][da_stage_tiles(rows, cols)]
+  int batch, rows, cols, ld;
+  int g_dtype, m_dtype, w_dtype;
+  float mu;
+  int nesterov;
+  int muon;
+};
+
+struct DaUnstage {
+  DaPtrTable x;      // destinations (rows x cols, row pitch ld)
+  const void* wide;
+  int batch, rows, cols, ld;
+  int x_dtype, w_dtype;
+  float decay, step;
+  int muon;
+};
+
+int da_stage_tiles(int rows, int cols);
+int da_stage_wide(const DaStage& d, hipStream_t s);
+int da_norm_finish(const float* partials, int tiles, int batch, float eps, int bf16_mode, float* divisor,
+                   hipStream_t s);
+int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor, hipStream_t s);
+int da_unstage(const DaUnstage& d, hipStream_t s);

@@ -1,0 +1,339 @@
+// HBM-bound passes around the Newton-Schulz iteration (all single-pass, 16-byte accesses):
+//
+//   stage_wide  : source matrix -> bf16/f32 working matrix in *wide* orientation
+//                 (rows <= cols; tall sources are transposed through an LDS tile), fused
+//                 with either a plain dtype cast (stand-alone Newton-Schulz) or Muon's
+//                 momentum / Nesterov update, plus per-tile partial sums of squares for
+//                 the Frobenius norm.
+//   norm_finish : fixed-order reduction of the partial sums -> divisor per matrix.
+//   normalize   : X <- X / (||X||_F + eps) with the reference's rounding points.
+//   unstage     : wide working matrix -> destination orientation; either a plain store
+//                 (stand-alone Newton-Schulz) or Muon's weight-decay + scaled update.
+//
+// Rounding follows the reference op by op (reference dion/muon.py:536-550, 569-573,
+// 633-638); the translation unit must be compiled with -ffp-contract=off.
+#include "common.h"
+#include "elementwise.h"
+
+namespace {
+
+constexpr int TS = 64;  // tile edge; 256 threads, 16 elements (two 8-wide chunks) per thread
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = bf2f((bf16_t)(w[i] & 0xffffu));
+      v[2 * i + 1] = bf2f((bf16_t)(w[i] >> 16));
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(v[2 * i]) | ((uint32_t)f2bf(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  static __device__ __forceinline__ float round(float x) { return rbf(x); }
+};
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+  static __device__ __forceinline__ float round(float x) { return x; }
+};
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+  if (threadIdx.x == 0) s = (red[0] + red[1]) + (red[2] + red[3]);
+  return s;  // valid in thread 0
+}
+
+// ---------------------------------------------------------------------------------------
+// stage_wide
+// ---------------------------------------------------------------------------------------
+// Source element access, in the source's own (rows x cols, row-major) orientation.
+template <typename TG, typename TM, typename TW>
+struct StageArgs {
+  DaPtrTable g;       // sources (gradients), one pointer per matrix
+  DaPtrTable mom;     // momentum buffers (Muon mode), modified in place; unused for plain
+  TW* wide;           // [batch][mw][nw]
+  float* partials;    // [batch][tiles]
+  int rows, cols;     // source shape
+  int ld;             // source row pitch (elements)
+  float mu;
+  int nesterov;
+  int muon;           // 1: momentum update, 0: plain cast
+};
+
+template <typename TG, typename TM, typename TW, bool TALL>
+__global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a) {
+  // Tile coordinates are in the source orientation: tile (ti, tj) covers source rows
+  // ti*64.., cols tj*64...  The wide matrix is the source (TALL = false) or its transpose.
+  __shared__ float red[4];
+  __shared__ float tile[TALL ? TS : 1][TS + 1];
+  const int b = blockIdx.y;
+  const int tiles_c = (a.cols + TS - 1) / TS;
+  const int ti = blockIdx.x / tiles_c, tj = blockIdx.x % tiles_c;
+  const int tid = threadIdx.x;
+  const TG* G = static_cast<const TG*>(a.g.p[b]);
+  TM* M = a.muon ? static_cast<TM*>(a.mom.p[b]) : nullptr;
+  const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
+  TW* W = a.wide + (long long)b * mw * nw;
+
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int c = tid + 256 * it;        // chunk id within tile: 64 rows x 8 chunks
+    const int r = c >> 3, cc = (c & 7) * 8;
+    const int i = ti * TS + r, j = tj * TS + cc;
+    float u[8];
+    const bool ok = i < a.rows && j < a.cols;  // cols is a multiple of 8
+    if (ok) {
+      float g[8];
+      Vec8<TG>::load(G + (long long)i * a.ld + j, g);
+      if (a.muon) {
+        float m[8];
+        Vec8<TM>::load(M + (long long)i * a.cols + j, m);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float ge = Vec8<TM>::round(g[e]);                 // G.to(M.dtype)
+          float me = Vec8<TM>::round(m[e] * a.mu);                // M *= mu
+          me = Vec8<TM>::round(me + ge);                          // M += G
+          m[e] = me;
+          float ue = me;
+          if (a.nesterov) ue = Vec8<TM>::round(Vec8<TM>::round(me * a.mu) + ge);  // U = M*mu; U += G
+          u[e] = Vec8<TW>::round(ue);                             // U.to(bf16)
+        }
+        Vec8<TM>::store(M + (long long)i * a.cols + j, m);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = Vec8<TW>::round(g[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += u[e] * u[e];
+      if (!TALL) Vec8<TW>::store(W + (long long)i * nw + j, u);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = 0.f;
+    }
+    if (TALL) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[cc + e][r] = u[e];  // tile[source col][source row]
+    }
+  }
+  if (TALL) {
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int c = tid + 256 * it;
+      const int p = c >> 3, qq = (c & 7) * 8;   // wide row p = source col, wide cols = source rows
+      const int wi = tj * TS + p, wj = ti * TS + qq;
+      if (wi < mw && wj < nw) {                 // rows is a multiple of 8
+        float u[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = tile[p][qq + e];
+        Vec8<TW>::store(W + (long long)wi * nw + wj, u);
+      }
+    }
+  }
+  const float s = block_sum(ss, red);
+  if (tid == 0) a.partials[(long long)b * gridDim.x + blockIdx.x] = s;
+}
+
+// ---------------------------------------------------------------------------------------
+// norm_finish: divisor[b] = round(round(sqrt(sum)) + eps)   (bf16 working dtype)
+//              divisor[b] = sqrt(sum) + eps                 (f32 working dtype)
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void norm_finish_kernel(const float* partials, int n, float eps, int bf16_mode,
+                                                          float* divisor) {
+  __shared__ double red[256];
+  const float* p = partials + (long long)blockIdx.x * n;
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256) s += (double)p[i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    float nrm = sqrtf((float)red[0]);
+    float d;
+    if (bf16_mode) d = rbf(rbf(nrm) + eps);
+    else d = nrm + eps;
+    divisor[blockIdx.x] = d;
+  }
+}
+
+template <typename TW>
+__global__ __launch_bounds__(256) void normalize_kernel(TW* W, long long per_matrix, const float* divisor) {
+  const int b = blockIdx.y;
+  const float d = divisor[b];
+  TW* p = W + (long long)b * per_matrix;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < per_matrix;
+       i += (long long)gridDim.x * 256 * 8) {
+    float v[8];
+    Vec8<TW>::load(p + i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = v[e] / d;
+    Vec8<TW>::store(p + i, v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// unstage
+// ---------------------------------------------------------------------------------------
+template <typename TX, typename TW>
+struct UnstageArgs {
+  DaPtrTable x;       // destinations, one pointer per matrix (rows x cols, row-major, pitch ld)
+  const TW* wide;     // [batch][mw][nw]
+  int rows, cols, ld;
+  float decay;        // 1 - lr * weight_decay
+  float step;         // adjusted learning rate
+  int muon;           // 1: X <- X*decay - wide*step ; 0: X <- wide
+};
+
+template <typename TX, typename TW, bool TALL>
+__global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
+  __shared__ float tile[TALL ? TS : 1][TS + 1];
+  const int b = blockIdx.y;
+  const int tiles_c = (a.cols + TS - 1) / TS;
+  const int ti = blockIdx.x / tiles_c, tj = blockIdx.x % tiles_c;
+  const int tid = threadIdx.x;
+  TX* X = static_cast<TX*>(a.x.p[b]);
+  const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
+  const TW* W = a.wide + (long long)b * mw * nw;
+
+  if (TALL) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int c = tid + 256 * it;
+      const int p = c >> 3, qq = (c & 7) * 8;
+      const int wi = tj * TS + p, wj = ti * TS + qq;
+      float u[8];
+      if (wi < mw && wj < nw) Vec8<TW>::load(W + (long long)wi * nw + wj, u);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[qq + e][p] = u[e];  // tile[source row][source col]
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int c = tid + 256 * it;
+    const int r = c >> 3, cc = (c & 7) * 8;
+    const int i = ti * TS + r, j = tj * TS + cc;
+    if (i >= a.rows || j >= a.cols) continue;
+    float u[8];
+    if (TALL) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = tile[r][cc + e];
+    } else {
+      Vec8<TW>::load(W + (long long)i * nw + j, u);
+    }
+    TX* xp = X + (long long)i * a.ld + j;
+    if (a.muon) {
+      float x[8];
+      Vec8<TX>::load(xp, x);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xd = Vec8<TX>::round(x[e] * a.decay);    // X *= 1 - lr*wd
+        const float t = Vec8<TW>::round(u[e] * a.step);      // U * adjusted_lr (U's dtype)
+        x[e] = xd - t;                                       // X -= U ; rounded by the store
+      }
+      Vec8<TX>::store(xp, x);
+    } else {
+      Vec8<TX>::store(xp, u);
+    }
+  }
+}
+
+template <typename TG, typename TM, typename TW>
+int stage_launch(const StageArgs<TG, TM, TW>& a, int batch, bool tall, hipStream_t s) {
+  const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
+  dim3 grid(tiles, batch);
+  if (tall) hipLaunchKernelGGL((stage_wide_kernel<TG, TM, TW, true>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((stage_wide_kernel<TG, TM, TW, false>), grid, dim3(256), 0, s, a);
+  return da_launch_status();
+}
+
+template <typename TG, typename TM>
+int stage_dispatch_w(const DaStage& d, hipStream_t s) {
+  if (d.w_dtype == DA_BF16) {
+    StageArgs<TG, TM, bf16_t> a{d.g, d.mom, static_cast<bf16_t*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.mu, d.nesterov, d.muon};
+    return stage_launch(a, d.batch, d.rows > d.cols, s);
+  }
+  StageArgs<TG, TM, float> a{d.g, d.mom, static_cast<float*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.mu, d.nesterov, d.muon};
+  return stage_launch(a, d.batch, d.rows > d.cols, s);
+}
+
+template <typename TX, typename TW>
+int unstage_launch(const DaUnstage& d, hipStream_t s) {
+  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.decay, d.step, d.muon};
+  const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
+  dim3 grid(tiles, d.batch);
+  if (d.rows > d.cols) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((unstage_kernel<TX, TW, false>), grid, dim3(256), 0, s, a);
+  return da_launch_status();
+}
+
+}  // namespace
+
+int da_stage_tiles(int rows, int cols) { return ((rows + TS - 1) / TS) * ((cols + TS - 1) / TS); }
+
+int da_stage_wide(const DaStage& d, hipStream_t s) {
+  if (d.batch <= 0 || d.batch > DA_MAX_PTRS) return DA_ERR_LIMIT;
+  if ((d.rows | d.cols | d.ld) & 7) return DA_ERR_ALIGN;
+  const int gd = d.g_dtype, md = d.muon ? d.m_dtype : d.g_dtype;
+  if (gd == DA_BF16 && md == DA_BF16) return stage_dispatch_w<bf16_t, bf16_t>(d, s);
+  if (gd == DA_F32 && md == DA_BF16) return stage_dispatch_w<float, bf16_t>(d, s);
+  if (gd == DA_BF16 && md == DA_F32) return stage_dispatch_w<bf16_t, float>(d, s);
+  if (gd == DA_F32 && md == DA_F32) return stage_dispatch_w<float, float>(d, s);
+  return DA_ERR_DTYPE;
+}
+
+int da_norm_finish(const float* partials, int tiles, int batch, float eps, int bf16_mode, float* divisor,
+                   hipStream_t s) {
+  hipLaunchKernelGGL(norm_finish_kernel, dim3(batch), dim3(256), 0, s, partials, tiles, eps, bf16_mode, divisor);
+  return da_launch_status();
+}
+
+int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor, hipStream_t s) {
+  if (per_matrix & 7) return DA_ERR_ALIGN;
+  long long blocks = (per_matrix / 8 + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  dim3 grid((unsigned)blocks, batch);
+  if (w_dtype == DA_BF16)
+    hipLaunchKernelGGL(normalize_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(wide), per_matrix, divisor);
+  else
+    hipLaunchKernelGGL(normalize_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(wide), per_matrix, divisor);
+  return da_launch_status();
+}
+
+int da_unstage(const DaUnstage& d, hipStream_t s) {
+  if (d.batch <= 0 || d.batch > DA_MAX_PTRS) return DA_ERR_LIMIT;
+  if ((d.rows | d.cols | d.ld) & 7) return DA_ERR_ALIGN;
+  if (d.x_dtype == DA_BF16 && d.w_dtype == DA_BF16) return unstage_launch<bf16_t, bf16_t>(d, s);
+  if (d.x_dtype == DA_F32 && d.w_dtype == DA_BF16) return unstage_launch<float, bf16_t>(d, s);
+  if (d.x_dtype == DA_F32 && d.w_dtype == DA_F32) return unstage_launch<float, float>(d, s);
+  if (d.x_dtype == DA_BF16 && d.w_dtype == DA_F32) return unstage_launch<bf16_t, float>(d, s);
+  return DA_ERR_DTYPE;
+}

@@ -1,0 +1,126 @@
+/*
+ * dion_amd -- C ABI of the MI355X (gfx950) Muon / Dion optimizer-step kernels.
+ *
+ * The reference (microsoft/dion) is pure Python on PyTorch and has no FFI of its own:
+ * the boundary this library slots in behind is its operator level -- the functions the
+ * optimizer classes call on lists of tensors.  Each entry point below names the reference
+ * function it replaces (file:line in the reference tree).
+ *
+ * Conventions
+ *   - Plain C types only.  Every pointer is a device pointer unless said otherwise; the
+ *     caller owns all memory including the workspace (the library allocates nothing).
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and nothing
+ *     synchronises with the host.
+ *   - Matrices are row-major.  dtype codes: DION_AMD_BF16 / _F32 / _F64.
+ *   - Return value: 0 ok; <0 argument error (DION_AMD_ERR_*); >0 a hipError_t.
+ *   - Alignment: bf16 matrices need every dimension, pitch and batch stride to be a
+ *     multiple of 8 elements and 16-byte aligned base pointers (fp32: multiples of 4).
+ *     Violations return DION_AMD_ERR_ALIGN; nothing is launched.
+ */
+#ifndef DION_AMD_H
+#define DION_AMD_H
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DION_AMD_BF16 0
+#define DION_AMD_F32 1
+#define DION_AMD_F64 2
+
+#define DION_AMD_OK 0
+#define DION_AMD_ERR_ARG (-1)
+#define DION_AMD_ERR_ALIGN (-2)
+#define DION_AMD_ERR_WORKSPACE (-3)
+#define DION_AMD_ERR_DTYPE (-4)
+#define DION_AMD_ERR_LIMIT (-5)
+
+#define DION_AMD_EPI_STORE 0
+#define DION_AMD_EPI_AXPBY 1
+
+/* Library version string (static storage). */
+const char* dion_amd_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Newton-Schulz orthogonalisation
+ * ------------------------------------------------------------------------------------- */
+
+/* Bytes of workspace dion_amd_newton_schulz wants for `batch` matrices of m x n.  A smaller
+ * workspace is accepted as long as one matrix fits: the batch is then processed in chunks. */
+size_t dion_amd_ns_workspace_bytes(int batch, int m, int n, int compute_dtype);
+
+/* Replaces zeropower_via_newtonschulz5 (reference dion/muon.py:620-647, twin in
+ * dion/newton_schulz_triton.py:305-333 and the Triton driver newton_schulz_triton
+ * dion/newton_schulz_triton.py:336-374; fixed-coefficient variant
+ * dion/muon_reference.py:10-27).
+ *
+ * For each of `batch` matrices G_b (m x n, dtype g_dtype, row pitch ldg, batch stride
+ * g_stride): cast to compute_dtype, transpose to wide if m > n, divide by
+ * (||.||_F + eps), run `steps` iterations  A = X X^T; B = b A + c A A; X = a X + B X  with
+ * (a, b, c) = coeffs[3*i .. 3*i+2] (host array), transpose back, store to out_b (m x n,
+ * dtype compute_dtype, row pitch ldo, batch stride out_stride).
+ * faithful != 0 reproduces every intermediate bf16 rounding of the reference's separate
+ * tensor ops inside the GEMM epilogues; 0 rounds once per GEMM. */
+int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int ldg,
+                           void* out, long long out_stride, int ldo,
+                           int batch, int m, int n,
+                           const float* coeffs, int steps, float eps,
+                           int compute_dtype, int faithful,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* Replaces ns_line_1 (reference dion/newton_schulz_triton.py:134-170):
+ * C_b (m x m) = A_b A_b^T for A_b (m x k); upper tiles computed, mirrored store. */
+int dion_amd_syrk(const void* A, long long a_stride, int lda,
+                  void* C, long long c_stride, int ldc,
+                  int batch, int m, int k, int dtype, void* stream);
+
+/* Replaces ns_line_2 (reference dion/newton_schulz_triton.py:261-302):
+ * C_b = alpha * A_b A_b^T + beta * A_b for symmetric A_b (m x m). */
+int dion_amd_sym_poly(const void* A, long long a_stride, int lda,
+                      void* C, long long c_stride, int ldc,
+                      int batch, int m, float alpha, float beta,
+                      int dtype, int faithful, void* stream);
+
+/* General batched GEMM with fused epilogue; replaces the torch matmul / baddbmm / addmm
+ * call sites of the hot path (reference dion/newton_schulz_triton.py:363,369;
+ * dion/dion.py:801, 839, 1513-1530).
+ *   C_b (M x N) = s0 * E_b + s1 * sum_k Aop_b(i,k) Bop_b(j,k)      (epilogue AXPBY)
+ *   C_b         = s1 * sum_k ...                                   (epilogue STORE)
+ * a_kstrided = 0: A stored M x K (pitch lda); 1: stored K x M.  Same for B (N x K / K x N).
+ * in_dtype bf16 or f32; c_dtype (for C and E) bf16 or f32 (f32 only when in_dtype is f32).
+ * E may alias C. */
+int dion_amd_gemm(const void* A, long long a_stride, int lda, int a_kstrided,
+                  const void* B, long long b_stride, int ldb, int b_kstrided,
+                  void* C, long long c_stride, int ldc,
+                  const void* E, long long e_stride, int lde,
+                  int batch, int M, int N, int K,
+                  int in_dtype, int c_dtype, int epilogue, float s0, float s1,
+                  int faithful, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Muon step for one bucket of same-shape matrices
+ * ------------------------------------------------------------------------------------- */
+
+size_t dion_amd_muon_workspace_bytes(int batch, int m, int n);
+
+/* Replaces muon_update_batch_async on one GPU (reference dion/muon.py:356-391, 437-448,
+ * 461-486): muon_update_pre_orthogonalize (525-552), muon_update_newton_schulz (576-593)
+ * and muon_update_post_orthogonalize (556-573), batched over a bucket of `batch` matrices
+ * of identical shape m x n (create_param_batches, reference dion/opt_utils.py:48-65).
+ *
+ * X, G, M: HOST arrays of `batch` device pointers (weights, gradients, momentum; contiguous
+ * m x n).  x_dtype is the dtype of X and M, g_dtype that of G.  Per matrix, in place:
+ *   M <- mu M + G;  U = nesterov ? mu M + G : M;  O = NS(bf16(U));
+ *   X <- (1 - lr wd) X - adjusted_lr O.
+ * decay = 1 - lr*wd and adjusted_lr are passed as already-evaluated fp32 values. */
+int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
+                       int batch, int m, int n, int x_dtype, int g_dtype,
+                       float mu, int nesterov, float decay, float adjusted_lr,
+                       const float* coeffs, int steps, float eps, int faithful,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DION_AMD_H */

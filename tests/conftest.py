@@ -1,0 +1,30 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def dev():
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device("cuda:0")
+
+
+def rel_fro(x, ref):
+    """Relative Frobenius error ||x - ref|| / ||ref|| in float64."""
+    import torch
+
+    x = x.detach().to("cpu", torch.float64)
+    ref = ref.detach().to("cpu", torch.float64)
+    return ((x - ref).norm() / ref.norm().clamp_min(1e-300)).item()
