@@ -1,2 +1,3 @@
 """MI355X-native Muon / Dion optimizer step (drop-in for the `dion` package's single-GPU path)."""
+from .muon import Muon  # noqa: F401
 from .newton_schulz import zeropower_via_newtonschulz5  # noqa: F401

@@ -37,6 +37,9 @@ _SIGNATURES = {
     "dion_amd_gemm": (_i, [_vp, _ll, _i, _i, _vp, _ll, _i, _i, _vp, _ll, _i, _vp, _ll, _i,
                            _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _vp]),
     "dion_amd_muon_workspace_bytes": (_sz, [_i, _i, _i]),
+    "dion_amd_profile_enable": (_i, [_i]),
+    "dion_amd_profile_reset": (_i, []),
+    "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),
     "dion_amd_muon_step": (_i, [_vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _f, _i, _f, _f, _fp, _i, _f, _i, _vp, _sz, _vp]),
 }
 
@@ -116,3 +119,19 @@ class Workspace:
             self._buf = None
             self._buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         return self._buf
+
+
+PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
+              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem")
+
+
+def profile_read():
+    """{kind: (launches, total_ms, total_work)} for every kind with at least one recorded launch."""
+    lib = load()
+    out = {}
+    for k, name in enumerate(PROF_KINDS):
+        n, ms, work = _ll(0), _c.c_double(0), _c.c_double(0)
+        check(lib.dion_amd_profile_read(k, _c.byref(n), _c.byref(ms), _c.byref(work)), "dion_amd_profile_read")
+        if n.value:
+            out[name] = (n.value, ms.value, work.value)
+    return out

@@ -3,6 +3,7 @@
 #include "../../include/dion_amd.h"
 #include "common.h"
 #include "elementwise.h"
+#include "prof.h"
 
 namespace {
 
@@ -53,7 +54,14 @@ struct NsBuffers {
   }
 };
 
-int gemm_any(const GemmDesc& d, int dtype, hipStream_t s) {
+// Executed multiply-adds of one launch (symmetric outputs: upper triangle incl. diagonal).
+double gemm_flops(const GemmDesc& d) {
+  const double mn = d.symmetric ? 0.5 * (double)d.M * ((double)d.M + 1.0) : (double)d.M * d.N;
+  return 2.0 * mn * d.K * d.batch;
+}
+
+int gemm_any(const GemmDesc& d, int dtype, hipStream_t s, int kind = DA_PROF_GEMM) {
+  DaProfScope prof(kind, gemm_flops(d), s);
   return dtype == DA_BF16 ? da_gemm_bf16(d, s) : da_gemm_f32(d, s);
 }
 
@@ -75,7 +83,7 @@ int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const f
     g.M = L.mw; g.N = L.mw; g.K = L.nw;
     g.a_kstrided = 0; g.b_kstrided = 0; g.symmetric = 1;
     g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
-    int rc = gemm_any(g, dtype, s);
+    int rc = gemm_any(g, dtype, s, DA_PROF_NS_SYRK);
     if (rc) return rc;
     // B = b A + c A A^T   (A symmetric, so A A = A A^T: both operands k-contiguous)
     g.A = W.a; g.B = W.a; g.C = W.b; g.E = W.a;
@@ -83,7 +91,7 @@ int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const f
     g.lda = L.mw; g.ldb = L.mw; g.ldc = L.mw; g.lde = L.mw;
     g.M = L.mw; g.N = L.mw; g.K = L.mw;
     g.epilogue = DA_EPI_AXPBY; g.s0 = b; g.s1 = c;
-    rc = gemm_any(g, dtype, s);
+    rc = gemm_any(g, dtype, s, DA_PROF_NS_POLY);
     if (rc) return rc;
     // X' = a X + B X   (B symmetric: k-contiguous; X is the k-strided operand)
     g.A = W.b; g.B = x; g.C = y; g.E = x;
@@ -92,7 +100,7 @@ int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const f
     g.M = L.mw; g.N = L.nw; g.K = L.mw;
     g.a_kstrided = 0; g.b_kstrided = 1; g.symmetric = 0;
     g.epilogue = DA_EPI_AXPBY; g.s0 = a; g.s1 = 1.f;
-    rc = gemm_any(g, dtype, s);
+    rc = gemm_any(g, dtype, s, DA_PROF_NS_AXPY);
     if (rc) return rc;
     char* t = x; x = y; y = t;
   }
@@ -101,6 +109,7 @@ int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const f
 }
 
 int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
+  DaProfScope prof(DA_PROF_NORMALIZE, 2.0 * (double)L.mw * L.nw * L.esz * cb, s);
   int rc = da_norm_finish(W.partials, L.tiles, cb, eps, dtype == DA_BF16, W.divisor, s);
   if (rc) return rc;
   // x_bytes is padded per matrix; the pad is never read by the GEMMs, normalising it is harmless.
@@ -143,7 +152,11 @@ int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int l
     st.batch = cb; st.rows = m; st.cols = n; st.ld = ldg;
     st.g_dtype = g_dtype; st.m_dtype = g_dtype; st.w_dtype = compute_dtype;
     st.mu = 0.f; st.nesterov = 0; st.muon = 0;
-    int rc = da_stage_wide(st, s);
+    int rc;
+    {
+      DaProfScope prof(DA_PROF_STAGE, (double)m * n * (gsz + L.esz) * cb, s);
+      rc = da_stage_wide(st, s);
+    }
     if (rc) return rc;
     rc = ns_normalize_chunk(L, W, cb, compute_dtype, eps, s);
     if (rc) return rc;
@@ -155,7 +168,10 @@ int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int l
     us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = ldo;
     us.x_dtype = compute_dtype; us.w_dtype = compute_dtype;
     us.decay = 1.f; us.step = 1.f; us.muon = 0;
-    rc = da_unstage(us, s);
+    {
+      DaProfScope prof(DA_PROF_UNSTAGE, 2.0 * (double)m * n * L.esz * cb, s);
+      rc = da_unstage(us, s);
+    }
     if (rc) return rc;
   }
   return DA_OK;
@@ -234,7 +250,13 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
     st.batch = cb; st.rows = m; st.cols = n; st.ld = n;
     st.g_dtype = g_dtype; st.m_dtype = x_dtype; st.w_dtype = DA_BF16;
     st.mu = mu; st.nesterov = nesterov; st.muon = 1;
-    int rc = da_stage_wide(st, s);
+    const double xsz = x_dtype == DA_BF16 ? 2 : 4, gsz = g_dtype == DA_BF16 ? 2 : 4;
+    int rc;
+    {
+      // algorithmic bytes: read G and M, write M and the bf16 working matrix
+      DaProfScope prof(DA_PROF_STAGE, (double)m * n * (gsz + 2 * xsz + 2) * cb, s);
+      rc = da_stage_wide(st, s);
+    }
     if (rc) return rc;
     rc = ns_normalize_chunk(L, W, cb, DA_BF16, eps, s);
     if (rc) return rc;
@@ -246,7 +268,11 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
     us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = n;
     us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
     us.decay = decay; us.step = adjusted_lr; us.muon = 1;
-    rc = da_unstage(us, s);
+    {
+      // algorithmic bytes: read X and the bf16 result, write X
+      DaProfScope prof(DA_PROF_UNSTAGE, (double)m * n * (2 * xsz + 2) * cb, s);
+      rc = da_unstage(us, s);
+    }
     if (rc) return rc;
   }
   return DA_OK;

@@ -120,6 +120,33 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
                        const float* coeffs, int steps, float eps, int faithful,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Measurement hooks (no counterpart in the reference; used by the benchmark only)
+ * ------------------------------------------------------------------------------------- */
+
+/* When enabled, every kernel launch made by the entry points above is bracketed by a pair
+ * of HIP events on its launch stream and tagged with a kernel kind (DION_AMD_PROF_*) and
+ * its algorithmic work (flops for GEMM kinds, bytes for the HBM-bound passes). */
+#define DION_AMD_PROF_NS_SYRK 0
+#define DION_AMD_PROF_NS_POLY 1
+#define DION_AMD_PROF_NS_AXPY 2
+#define DION_AMD_PROF_STAGE 3
+#define DION_AMD_PROF_NORMALIZE 4
+#define DION_AMD_PROF_UNSTAGE 5
+#define DION_AMD_PROF_GEMM 6
+#define DION_AMD_PROF_DION_BQ 7
+#define DION_AMD_PROF_DION_BTP 8
+#define DION_AMD_PROF_DION_EF 9
+#define DION_AMD_PROF_DION_UPD 10
+#define DION_AMD_PROF_DION_ORTH 11
+#define DION_AMD_PROF_DION_ELEM 12
+#define DION_AMD_PROF_KINDS 13
+int dion_amd_profile_enable(int on);
+int dion_amd_profile_reset(void);
+/* Waits for the recorded events of `kind`; returns launch count, summed milliseconds and
+ * summed work. */
+int dion_amd_profile_read(int kind, long long* launches, double* total_ms, double* total_work);
+
 #ifdef __cplusplus
 }
 #endif

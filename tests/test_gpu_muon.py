@@ -1,0 +1,157 @@
+"""GPU parity of `dion_amd.Muon.step()` against the CPU oracle (reference dion/muon.py:356-486)."""
+import pytest
+import torch
+
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+
+SHAPES_GPT_SMALL_LAYER = [(768, 768)] * 4 + [(3072, 768), (768, 3072)]
+
+
+def _make(shapes, dtype, seed, gscale=1e-3):
+    g = torch.Generator().manual_seed(seed)
+    X = [(torch.randn(s, generator=g) * 0.02).to(dtype) for s in shapes]
+    return X, g
+
+
+def _grads(shapes, gen, dtype, gscale=1e-3):
+    return [(torch.randn(s, generator=gen) * gscale).to(dtype) for s in shapes]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("nesterov", [True, False])
+def test_muon_step_matches_oracle(dev, dtype, nesterov):
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    shapes = SHAPES_GPT_SMALL_LAYER * 2
+    X0, gen = _make(shapes, dtype, seed=1)
+    Xo = [x.clone() for x in X0]
+    Mo = [torch.zeros_like(x) for x in X0]
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    lr, mu, wd = 0.02, 0.95, 0.01
+    opt = Muon(params, lr=lr, mu=mu, weight_decay=wd, nesterov=nesterov, adjust_lr="spectral_norm")
+    for step in range(3):
+        G = _grads(shapes, gen, dtype)
+        for p, g in zip(params, G):
+            p.grad = g.to(dev)
+        prev = [x.clone() for x in Xo]
+        O.muon_step(Xo, G, Mo, lr=lr, mu=mu, weight_decay=wd, epsilon=1e-8, nesterov=nesterov)
+        opt.step()
+        for i, p in enumerate(params):
+            mom = opt.state[p]["momentum"]
+            assert mom.dtype == dtype and mom.shape == p.shape
+            # the momentum pass is element-wise with the reference's rounding points: bit exact
+            assert torch.equal(mom.cpu(), Mo[i]), f"momentum differs, matrix {i} step {step}"
+            # the applied update  X_prev * decay - X_new  is adjusted_lr * NS(U): NS bar 2e-2
+            decay = (1 - torch.tensor(lr) * torch.tensor(wd)).item()
+            upd_ref = prev[i].double() * decay - Xo[i].double()
+            upd_got = prev[i].double() * decay - p.detach().cpu().double()
+            if dtype == torch.float32:
+                assert rel_fro(upd_got, upd_ref) <= 2e-2
+            # weights themselves: the NS bar scaled by how large the update is next to the weights
+            # (+ one bf16 ulp of rounding noise for bf16 weights)
+            bound = 2e-2 * (upd_ref.norm() / Xo[i].double().norm()).item()
+            assert rel_fro(p.detach(), Xo[i]) <= bound + (4e-3 if dtype == torch.bfloat16 else 1e-6)
+        # keep the two trajectories from drifting apart through the (chaotic at 1e-2) bf16 NS noise
+        for i, p in enumerate(params):
+            p.data.copy_(Xo[i])
+    assert all(g["step"] == 3 for g in opt.param_groups)
+
+
+def test_muon_bf16_single_step_bits(dev):
+    """With bf16 weights the update is a few ulps per element; on one step from identical state at
+    least 85% of the weights must be bit-identical to the oracle's (the ~1e-2 NS noise flips some roundings)
+    and none may differ by more than one ulp of the largest weight."""
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    shapes = [(768, 768), (3072, 768), (768, 3072)]
+    X0, gen = _make(shapes, torch.bfloat16, seed=7)
+    G = _grads(shapes, gen, torch.bfloat16)
+    Xo = [x.clone() for x in X0]
+    Mo = [torch.zeros_like(x) for x in X0]
+    O.muon_step(Xo, G, Mo, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True)
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    for p, g in zip(params, G):
+        p.grad = g.to(dev)
+    Muon(params, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True).step()
+    for p, xo in zip(params, Xo):
+        same = (p.detach().cpu() == xo).float().mean().item()
+        assert same > 0.85, same
+        assert (p.detach().cpu().float() - xo.float()).abs().max().item() <= 2 ** -7 * xo.float().abs().max().item()
+
+
+@pytest.mark.parametrize("adjust", ["spectral_norm", "rms_norm", "keller_muon", None])
+def test_muon_adjust_lr_modes_and_groups(dev, adjust):
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    shapes = [(256, 512), (512, 256)]
+    X0, gen = _make(shapes, torch.float32, seed=3)
+    G = _grads(shapes, gen, torch.float32)
+    Xo = [x.clone() for x in X0]
+    Mo = [torch.zeros_like(x) for x in X0]
+    O.muon_step(Xo, G, Mo, lr=0.01, mu=0.9, weight_decay=0.0, nesterov=False, adjust=adjust)
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    bias = torch.nn.Parameter(torch.zeros(64, device=dev))
+    emb = torch.nn.Parameter(torch.randn(100, 32, device=dev))
+    opt = Muon(
+        [dict(params=params), dict(params=[bias], algorithm="adamw", lr=1e-3), dict(params=[emb], algorithm="lion")],
+        lr=0.01, mu=0.9, weight_decay=0.0, adjust_lr=adjust,
+    )
+    for p, g in zip(params, G):
+        p.grad = g.to(dev)
+    bias.grad = torch.ones_like(bias)
+    emb.grad = torch.randn_like(emb)
+    e0 = emb.detach().clone()
+    opt.step()
+    for x0, p, xo in zip(X0, params, Xo):
+        upd_ref = x0.double() - xo.double()
+        upd_got = x0.double() - p.detach().cpu().double()
+        assert rel_fro(upd_got, upd_ref) <= 2e-2
+    # AdamW first step moves by -lr * sign(g) (bias-corrected), Lion by -lr * sign
+    assert torch.allclose(bias.detach(), torch.full_like(bias, -1e-3), rtol=1e-4, atol=1e-7)
+    assert torch.allclose(emb.detach(), e0 - 0.01 * torch.sign(emb.grad), atol=1e-6)
+    assert set(opt.state[bias]) == {"momentum", "variance"} and set(opt.state[emb]) == {"momentum"}
+
+
+def test_muon_3d_batch_flatten_and_missing_grad(dev):
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    torch.manual_seed(5)
+    W = torch.randn(3, 128, 256) * 0.02       # batch of three matrices
+    C = torch.randn(64, 8, 4, 4) * 0.02       # conv weight, flattened to 64 x 128
+    Gw, Gc = torch.randn_like(W) * 1e-3, torch.randn_like(C) * 1e-3
+    pw, pc = torch.nn.Parameter(W.clone().to(dev)), torch.nn.Parameter(C.clone().to(dev))
+    unused = torch.nn.Parameter(torch.randn(128, 128, device=dev))
+    opt = Muon([dict(params=[pw, unused]), dict(params=[pc], flatten=True)], lr=0.01, weight_decay=0.0)
+    pw.grad, pc.grad = Gw.to(dev), Gc.to(dev)
+    u0 = unused.detach().clone()
+    opt.step()
+    Xo, Mo = [W.clone()], [torch.zeros_like(W)]
+    O.muon_step(Xo, [Gw], Mo, lr=0.01, mu=0.95, weight_decay=0.0)
+    assert rel_fro(W.double() - pw.detach().cpu().double(), W.double() - Xo[0].double()) <= 2e-2
+    Xc, Mc = [C.clone()], [torch.zeros_like(C)]
+    O.muon_step(Xc, [Gc], Mc, lr=0.01, mu=0.95, weight_decay=0.0, flatten=True)
+    assert rel_fro(C.double() - pc.detach().cpu().double(), C.double() - Xc[0].double()) <= 2e-2
+    assert torch.equal(unused.detach(), u0) and unused not in opt.state
+
+
+def test_muon_custom_newton_schulz_hook(dev):
+    from dion_amd import Muon
+
+    calls = []
+
+    def hook(X, epsilon):
+        calls.append((X.dtype, tuple(X.shape), float(epsilon)))
+        return X  # identity "orthogonalisation"
+
+    p = torch.nn.Parameter(torch.ones(64, 32, device=dev))
+    p.grad = torch.full_like(p, 0.5)
+    Muon([p], lr=0.1, mu=0.0, weight_decay=0.0, adjust_lr=None, newton_schulz_func=hook).step()
+    assert calls and calls[0][0] == torch.bfloat16 and calls[0][1] == (64, 32)
+    assert abs(calls[0][2] - 1e-8) < 1e-12
+    assert torch.allclose(p.detach(), torch.full_like(p, 1 - 0.1 * 0.5), atol=1e-3)  # U * lr rounds in bf16
