@@ -199,58 +199,108 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
   }
 
   // ---- epilogue -------------------------------------------------------------------
-  Epi ep{d.s0, d.s1, d.epilogue, d.faithful, d.c_dtype == DA_F32};
+  // The accumulators go through LDS (the stage buffers are free now), one 32-row band of
+  // the wavefront's sub-tile at a time, so that C and E move as 16-byte row segments and
+  // the code stays small enough to keep every accumulator index a compile-time constant.
+  constexpr int W = BT / 2;          // columns of a wavefront's sub-tile
+  constexpr int PITCH = W + 4;       // floats; 16-byte aligned rows, conflict-free float4 writes
+  constexpr int CPR = W / 8;         // 8-column chunks per row
+  constexpr int RPP = 64 / CPR;      // rows per pass of the wavefront
+  float* stg = reinterpret_cast<float*>(lds) + wave * (32 * PITCH);
+  const Epi ep{d.s0, d.s1, d.epilogue, d.faithful, d.c_dtype == DA_F32};
   const bool mirror = SYM && (ti != tj);
   const bool has_e = d.epilogue == DA_EPI_AXPBY;
+  const int wm0 = m0 + wm * W, wn0 = n0 + wn * W;
+  const long long cb = (long long)b * d.sC, eb = (long long)b * d.sE;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m0 + wm * (BT / 2) + i * 32 + (lane & 31);
+    {
+      float* row = stg + (lane & 31) * PITCH + (lane >> 5) * 4;
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
+      for (int j = 0; j < TM; ++j)
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        const int n = n0 + wn * (BT / 2) + j * 32 + vq * 8 + (lane >> 5) * 4;
-        if (m >= d.M || n >= d.N) continue;
-        float e[4] = {0.f, 0.f, 0.f, 0.f};
-        float o[4];
+        for (int vq = 0; vq < 4; ++vq)
+          *reinterpret_cast<float4*>(row + j * 32 + vq * 8) =
+              make_float4(acc[i][j][vq * 4], acc[i][j][vq * 4 + 1], acc[i][j][vq * 4 + 2], acc[i][j][vq * 4 + 3]);
+    }
+    __syncthreads();
+    const int band_m = wm0 + i * 32;
+    for (int pass = 0; pass < 32 / RPP; ++pass) {
+      const int r = pass * RPP + lane / CPR;
+      const int c8 = (lane % CPR) * 8;
+      const int m = band_m + r, n = wn0 + c8;
+      if (m < d.M && n < d.N) {
+        float* sp = stg + r * PITCH + c8;
+        const float4 a0 = *reinterpret_cast<const float4*>(sp);
+        const float4 a1 = *reinterpret_cast<const float4*>(sp + 4);
+        float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        float e[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const long long off = (long long)m * d.ldc + n;
         if (ep.c_f32) {
-          float* Cp = static_cast<float*>(d.C) + (long long)b * d.sC + (long long)m * d.ldc + n;
           if (has_e) {
-            const float4 ev = *reinterpret_cast<const float4*>(static_cast<const float*>(d.E) + (long long)b * d.sE +
-                                                               (long long)m * d.lde + n);
-            e[0] = ev.x; e[1] = ev.y; e[2] = ev.z; e[3] = ev.w;
+            const float* Ep = static_cast<const float*>(d.E) + eb + (long long)m * d.lde + n;
+            const float4 e0 = *reinterpret_cast<const float4*>(Ep);
+            const float4 e1 = *reinterpret_cast<const float4*>(Ep + 4);
+            e[0] = e0.x; e[1] = e0.y; e[2] = e0.z; e[3] = e0.w; e[4] = e1.x; e[5] = e1.y; e[6] = e1.z; e[7] = e1.w;
           }
 #pragma unroll
-          for (int q = 0; q < 4; ++q) o[q] = epi_value(ep, acc[i][j][vq * 4 + q], e[q]);
-          *reinterpret_cast<float4*>(Cp) = make_float4(o[0], o[1], o[2], o[3]);
-          if (mirror) {
-            float* Ct = static_cast<float*>(d.C) + (long long)b * d.sC + (long long)n * d.ldc + m;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) Ct[(long long)q * d.ldc] = o[q];
-          }
+          for (int q = 0; q < 8; ++q) v[q] = epi_value(ep, v[q], e[q]);
+          float* Cp = static_cast<float*>(d.C) + cb + off;
+          *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
         } else {
-          bf16_t* Cp = static_cast<bf16_t*>(d.C) + (long long)b * d.sC + (long long)m * d.ldc + n;
           if (has_e) {
-            const uint2 ev = *reinterpret_cast<const uint2*>(static_cast<const bf16_t*>(d.E) + (long long)b * d.sE +
-                                                             (long long)m * d.lde + n);
-            e[0] = bf2f((bf16_t)(ev.x & 0xffffu)); e[1] = bf2f((bf16_t)(ev.x >> 16));
-            e[2] = bf2f((bf16_t)(ev.y & 0xffffu)); e[3] = bf2f((bf16_t)(ev.y >> 16));
+            const uint4 ev = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(d.E) + eb + (long long)m * d.lde + n);
+            const uint32_t w[4] = {ev.x, ev.y, ev.z, ev.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              e[2 * q] = bf2f((bf16_t)(w[q] & 0xffffu));
+              e[2 * q + 1] = bf2f((bf16_t)(w[q] >> 16));
+            }
           }
-          bf16_t h[4];
+          uint32_t pk[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) h[q] = f2bf(epi_value(ep, acc[i][j][vq * 4 + q], e[q]));
-          uint2 pk;
-          pk.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-          pk.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
-          *reinterpret_cast<uint2*>(Cp) = pk;
-          if (mirror) {
-            bf16_t* Ct = static_cast<bf16_t*>(d.C) + (long long)b * d.sC + (long long)n * d.ldc + m;
+          for (int q = 0; q < 4; ++q) {
+            const bf16_t lo = f2bf(epi_value(ep, v[2 * q], e[2 * q]));
+            const bf16_t hi = f2bf(epi_value(ep, v[2 * q + 1], e[2 * q + 1]));
+            pk[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+            v[2 * q] = bf2f(lo);
+            v[2 * q + 1] = bf2f(hi);
+          }
+          *reinterpret_cast<uint4*>(static_cast<bf16_t*>(d.C) + cb + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        }
+        if (mirror) {  // keep the final values for the transposed store
+          *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(sp + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+      }
+    }
+    if (mirror) {
+      __syncthreads();
+      // C^T: row n of the mirrored tile holds 32 consecutive m of this band
+      for (int pass = 0; pass < (W / 64) * 4; ++pass) {
+        const int nl = (pass >> 2) * 64 + lane;
+        const int mg = (pass & 3) * 8;
+        const int n = wn0 + nl, m = band_m + mg;
+        if (n < d.N && m < d.M) {  // M is a multiple of 8 for symmetric outputs
+          float v[8];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) Ct[(long long)q * d.ldc] = h[q];
+          for (int q = 0; q < 8; ++q) v[q] = stg[(mg + q) * PITCH + nl];
+          const long long off = (long long)n * d.ldc + m;
+          if (ep.c_f32) {
+            float* Cp = static_cast<float*>(d.C) + cb + off;
+            *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
+          } else {
+            uint32_t pk[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) pk[q] = (uint32_t)f2bf(v[2 * q]) | ((uint32_t)f2bf(v[2 * q + 1]) << 16);
+            *reinterpret_cast<uint4*>(static_cast<bf16_t*>(d.C) + cb + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
           }
         }
       }
     }
+    __syncthreads();
   }
 }
 
