@@ -4,6 +4,7 @@
 #include "common.h"
 #include "elementwise.h"
 #include "prof.h"
+#include "dion.h"
 
 namespace {
 
@@ -274,6 +275,208 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
       rc = da_unstage(us, s);
     }
     if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+
+// ---------------------------------------------------------------------------------------
+// Dion
+// ---------------------------------------------------------------------------------------
+}  // extern "C"
+
+namespace {
+
+struct DionLayout {
+  int mp, np, r;        // working orientation: B is mp x np with mp >= np; Q is np x r
+  size_t msz;           // bytes per element of the momentum dtype
+  size_t qc, p, rb, qn, orth, small;  // per-matrix byte sizes
+  size_t per_matrix;
+  DionLayout(int m, int n, int rank, int m_dtype) {
+    mp = m < n ? n : m;
+    np = m < n ? m : n;
+    r = rank;
+    msz = m_dtype == DA_BF16 ? 2 : 4;
+    qc = (size_t)np * r * msz;   // exact: the orthonormaliser and the GEMMs take these as
+    p = (size_t)mp * r * msz;    // contiguous batches (multiples of 128 bytes by the alignment rule)
+    rb = qc;
+    qn = qc;
+    orth = align_up(da_orth_workspace_bytes(1, mp, r), 256);
+    small = 256;  // flags, info, pointer-table slots
+    per_matrix = qc + p + rb + qn + orth + small + 256;
+  }
+  size_t fixed() const { return 4 * DA_MAX_PTRS * sizeof(void*) + 2 * DA_MAX_PTRS * sizeof(int) + 1024; }
+  int chunk(int batch, size_t ws_bytes) const {
+    if (ws_bytes < fixed()) return 0;
+    size_t c = (ws_bytes - fixed()) / per_matrix;
+    if (c > (size_t)batch) c = batch;
+    if (c > DA_MAX_PTRS) c = DA_MAX_PTRS;
+    return (int)c;
+  }
+  size_t recommended(int batch) const {
+    size_t c = ((size_t)6 << 30) / per_matrix;
+    if (c < 1) c = 1;
+    if (c > (size_t)batch) c = batch;
+    if (c > DA_MAX_PTRS) c = DA_MAX_PTRS;
+    return c * per_matrix + fixed();
+  }
+};
+
+}  // namespace
+
+extern "C" {
+
+size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype) {
+  if (batch <= 0 || m <= 0 || n <= 0 || r <= 0 || !dtype_ok(m_dtype)) return 0;
+  return DionLayout(m, n, r, m_dtype).recommended(batch);
+}
+
+size_t dion_amd_orthonormalize_workspace_bytes(int batch, int rows, int r) {
+  if (batch <= 0 || rows <= 0 || r <= 0) return 0;
+  return da_orth_workspace_bytes(batch, rows, r) + 256 + (size_t)batch * sizeof(int);
+}
+
+int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
+                            int* info, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!P || !out || !workspace || batch <= 0 || rows <= 0 || r <= 0 || passes < 1 || passes > 3) return DA_ERR_ARG;
+  if (!dtype_ok(dtype)) return DA_ERR_DTYPE;
+  if (r > rows) return DA_ERR_ARG;
+  if (workspace_bytes < dion_amd_orthonormalize_workspace_bytes(batch, rows, r)) return DA_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int* inf = info;
+  if (!inf) inf = reinterpret_cast<int*>(static_cast<char*>(workspace) + align_up(da_orth_workspace_bytes(batch, rows, r), 256));
+  int rc = da_fill_int(inf, batch, 0, s);
+  if (rc) return rc;
+  DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
+  return da_orthonormalize(P, out, dtype, batch, rows, r, passes, workspace, inf, s);
+}
+
+int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
+                       int r, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
+                       float scaled_lr, float eps, int faithful, int* info, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+  if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || r <= 0) return DA_ERR_ARG;
+  if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype) || !dtype_ok(m_dtype) || !dtype_ok(q_dtype)) return DA_ERR_DTYPE;
+  if (m_dtype == DA_F32 && x_dtype != DA_F32) return DA_ERR_DTYPE;  // fp32 products update fp32 weights only
+  if ((m | n | r) & 7) return DA_ERR_ALIGN;
+  if (r > m || r > n) return DA_ERR_ARG;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
+  for (int i = 0; i < batch; ++i) {
+    if (!X[i] || !G[i] || !M[i] || !Q[i]) return DA_ERR_ARG;
+    if (((uintptr_t)X[i] | (uintptr_t)G[i] | (uintptr_t)M[i] | (uintptr_t)Q[i]) & 15) return DA_ERR_ALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const DionLayout L(m, n, r, m_dtype);
+  const int chunk = L.chunk(batch, workspace_bytes);
+  if (chunk < 1) return DA_ERR_WORKSPACE;
+  const bool transposed = m < n;
+  const int mp = L.mp, np = L.np;
+  const long long mn = (long long)m * n;
+  const double msz = (double)L.msz, xsz = x_dtype == DA_BF16 ? 2 : 4, gsz = g_dtype == DA_BF16 ? 2 : 4;
+
+  for (int b0 = 0; b0 < batch; b0 += chunk) {
+    const int cb = batch - b0 < chunk ? batch - b0 : chunk;
+    // ---- carve the workspace
+    char* w = static_cast<char*>(workspace);
+    void** tabM = reinterpret_cast<void**>(w); w += DA_MAX_PTRS * sizeof(void*);
+    void** tabX = reinterpret_cast<void**>(w); w += DA_MAX_PTRS * sizeof(void*);
+    w += 2 * DA_MAX_PTRS * sizeof(void*);
+    int* nonzero = reinterpret_cast<int*>(w); w += DA_MAX_PTRS * sizeof(int);
+    int* linfo = reinterpret_cast<int*>(w); w += DA_MAX_PTRS * sizeof(int);
+    w = static_cast<char*>(workspace) + L.fixed();
+    char* Qc = w; w += L.qc * cb;
+    char* P = w; w += L.p * cb;
+    char* R = w; w += L.rb * cb;
+    char* Qn = w; w += L.qn * cb;
+    char* orth_ws = reinterpret_cast<char*>(align_up(reinterpret_cast<uintptr_t>(w), 256));
+    const long long sQ = (long long)(L.qc / L.msz), sP = (long long)(L.p / L.msz);
+
+    DaPtrTable tx{}, tg{}, tm{}, tq{};
+    for (int i = 0; i < cb; ++i) {
+      tx.p[i] = X[b0 + i]; tg.p[i] = const_cast<void*>(G[b0 + i]); tm.p[i] = M[b0 + i]; tq.p[i] = Q[b0 + i];
+    }
+    int rc;
+    {
+      DaProfScope prof(DA_PROF_DION_ELEM, (double)mn * (2 * msz + gsz) * cb, s);
+      rc = da_fill_int(nonzero, 2 * DA_MAX_PTRS, 0, s);  // nonzero[] and linfo[] are adjacent
+      if (rc) return rc;
+      rc = da_write_table(tm, tabM, cb, s);
+      if (rc) return rc;
+      rc = da_write_table(tx, tabX, cb, s);
+      if (rc) return rc;
+      // B = M + G, kept in M   (reference dion/dion.py:794)
+      rc = da_add_grad(tm, tg, m_dtype, g_dtype, mn, cb, nonzero, s);
+      if (rc) return rc;
+      // Q in the momentum dtype   (reference dion/dion.py:1216)
+      rc = da_cast_table(tq, q_dtype, Qc, m_dtype, (long long)np * r, cb, s);
+      if (rc) return rc;
+    }
+    GemmDesc g{};
+    g.batch = cb; g.faithful = faithful;
+    // ---- P = B Q   (reference dion/dion.py:801); B is M (mp x np) or M^T when m < n
+    g.Atab = const_cast<const void* const*>(tabM); g.A = nullptr; g.lda = n; g.a_kstrided = transposed ? 1 : 0;
+    g.B = Qc; g.sB = sQ; g.ldb = r; g.b_kstrided = 1;
+    g.C = P; g.sC = sP; g.ldc = r; g.c_dtype = m_dtype;
+    g.M = mp; g.N = r; g.K = np;
+    g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
+    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
+    if (rc) return rc;
+    // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
+    {
+      DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
+      rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, 2, orth_ws, linfo, s);
+      if (rc) return rc;
+      // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
+      rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);
+      if (rc) return rc;
+    }
+    // ---- R = B^T P   (reference dion/dion.py:839)
+    g = GemmDesc{};
+    g.batch = cb; g.faithful = faithful;
+    g.Atab = const_cast<const void* const*>(tabM); g.lda = n; g.a_kstrided = transposed ? 0 : 1;
+    g.B = P; g.sB = sP; g.ldb = r; g.b_kstrided = 1;
+    g.C = R; g.sC = sQ; g.ldc = r; g.c_dtype = m_dtype;
+    g.M = np; g.N = r; g.K = mp;
+    g.epilogue = DA_EPI_STORE; g.s1 = 1.f;
+    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BTP);
+    if (rc) return rc;
+    {
+      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+      rc = da_fix(R, Qc, m_dtype, sQ, cb, nonzero, s);
+      if (rc) return rc;
+    }
+    // ---- error feedback  M <- M - (1 - mu) P R^T  (or R P^T)   (reference dion/dion.py:851-853)
+    g = GemmDesc{};
+    g.batch = cb; g.faithful = faithful;
+    if (!transposed) { g.A = P; g.sA = sP; g.B = R; g.sB = sQ; g.M = mp; g.N = np; }
+    else             { g.A = R; g.sA = sQ; g.B = P; g.sB = sP; g.M = np; g.N = mp; }
+    g.lda = r; g.ldb = r; g.K = r;
+    g.Ctab = tabM; g.Etab = const_cast<const void* const*>(tabM); g.ldc = n; g.lde = n; g.c_dtype = m_dtype;
+    g.epilogue = DA_EPI_AXPBY; g.s0 = 1.f; g.s1 = ef_alpha;
+    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_EF);
+    if (rc) return rc;
+    // ---- Q_new = column-normalised R   (reference dion/dion.py:856, 875, 1460-1491, 1533-1561)
+    {
+      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+      rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, eps, cb, s);
+      if (rc) return rc;
+    }
+    // ---- X <- (1 - lr wd) X - scaled_lr P Q_new^T  (or Q_new P^T)   (reference dion/dion.py:865-872)
+    g = GemmDesc{};
+    g.batch = cb; g.faithful = faithful;
+    if (!transposed) { g.A = P; g.sA = sP; g.B = Qn; g.sB = sQ; g.M = mp; g.N = np; }
+    else             { g.A = Qn; g.sA = sQ; g.B = P; g.sB = sP; g.M = np; g.N = mp; }
+    g.lda = r; g.ldb = r; g.K = r;
+    g.Ctab = tabX; g.Etab = const_cast<const void* const*>(tabX); g.ldc = n; g.lde = n; g.c_dtype = x_dtype;
+    g.epilogue = DA_EPI_AXPBY; g.s0 = decay; g.s1 = -scaled_lr;
+    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_UPD);
+    if (rc) return rc;
+    (void)xsz;
+    if (info) {
+      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+      DA_HIP_CHECK(hipMemcpyAsync(info + b0, linfo, cb * sizeof(int), hipMemcpyDeviceToDevice, s));
+    }
   }
   return DA_OK;
 }

@@ -67,6 +67,12 @@ struct GemmDesc {
   const void* B;
   void* C;
   const void* E;      // epilogue operand (same shape / layout as C), may be null
+  // Optional device arrays of per-matrix base pointers; when set they replace base + b * stride
+  // (matrices that live in separate allocations, e.g. the optimizer's momentum buffers).
+  const void* const* Atab;
+  const void* const* Btab;
+  void* const* Ctab;
+  const void* const* Etab;
   long long sA, sB, sC, sE;  // batch strides
   int lda, ldb, ldc, lde;
   int M, N, K;

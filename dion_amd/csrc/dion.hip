@@ -1,0 +1,317 @@
+// Dion step building blocks that are not GEMMs: the momentum accumulation with its all-zero
+// guard, dtype casts, the NaN / all-zero fix-up of P and R, the column normalisation that
+// turns R into the next Q, and the host-side driver of the fp64 CholeskyQR2
+// orthonormalisation (Gram -> blocked Cholesky -> blocked triangular solve, twice).
+#include "dion.h"
+#include "gemm_f64.h"
+#include "prof.h"
+
+namespace {
+
+template <typename T> struct V8;
+template <> struct V8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = bf2f((bf16_t)(w[i] & 0xffffu));
+      v[2 * i + 1] = bf2f((bf16_t)(w[i] >> 16));
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(v[2 * i]) | ((uint32_t)f2bf(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+  static __device__ __forceinline__ float round(float x) { return rbf(x); }
+  static __device__ __forceinline__ float maxval() { return 3.3895313892515355e38f; }
+};
+template <> struct V8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+  static __device__ __forceinline__ float round(float x) { return x; }
+  static __device__ __forceinline__ float maxval() { return 3.4028234663852886e38f; }
+};
+
+__global__ void fill_int_kernel(int* p, int n, int v) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ void write_table_kernel(DaPtrTable t, void** dst, int n) {
+  if ((int)threadIdx.x < n) dst[threadIdx.x] = t.p[threadIdx.x];
+}
+
+// M <- M + G (rounded to M's dtype); nonzero[b] |= any(M != 0).
+template <typename TM, typename TG>
+__global__ __launch_bounds__(256) void add_grad_kernel(DaPtrTable mt, DaPtrTable gt, long long n, int* nonzero) {
+  const int b = blockIdx.y;
+  TM* M = static_cast<TM*>(mt.p[b]);
+  const TG* G = static_cast<const TG*>(gt.p[b]);
+  bool any = false;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
+    float m[8], g[8];
+    V8<TM>::load(M + i, m);
+    V8<TG>::load(G + i, g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      m[e] = V8<TM>::round(m[e] + g[e]);
+      any |= (m[e] != 0.f);
+    }
+    V8<TM>::store(M + i, m);
+  }
+  if (__any(any) && (threadIdx.x & 63) == 0) atomicOr(nonzero + b, 1);
+}
+
+// dst[b] (contiguous, TD) <- src table[b] (TS)
+template <typename TS, typename TD>
+__global__ __launch_bounds__(256) void cast_table_kernel(DaPtrTable st, TD* dst, long long n) {
+  const int b = blockIdx.y;
+  const TS* S = static_cast<const TS*>(st.p[b]);
+  TD* D = dst + (long long)b * n;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
+    float v[8];
+    V8<TS>::load(S + i, v);
+    V8<TD>::store(D + i, v);
+  }
+}
+
+// v <- nan_to_num(v) * nonzero + alt * (1 - nonzero)      (alt may be null: treated as 0)
+template <typename T>
+__global__ __launch_bounds__(256) void fix_kernel(T* V, const T* alt, long long n, const int* nonzero) {
+  const int b = blockIdx.y;
+  const bool nz = nonzero[b] != 0;
+  T* p = V + (long long)b * n;
+  const T* a = alt ? alt + (long long)b * n : nullptr;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
+    float v[8], q[8];
+    V8<T>::load(p + i, v);
+    if (a && !nz) V8<T>::load(a + i, q);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = v[e];
+      if (x != x) x = 0.f;
+      else if (x > V8<T>::maxval()) x = V8<T>::maxval();
+      else if (x < -V8<T>::maxval()) x = -V8<T>::maxval();
+      v[e] = nz ? x : (a ? q[e] : 0.f);
+    }
+    V8<T>::store(p + i, v);
+  }
+}
+
+// Column normalisation of R[b] (rows x r, TM): Qn = R / (sqrt(sum_rows R^2) + eps), computed in
+// fp32 (column sums accumulated in fp64), stored as TM into qn[b] and, cast to TQ, into the
+// optimizer's Q state.  One workgroup per 64 columns: 4 row groups x 64 columns.
+template <typename TM, typename TQ>
+__global__ __launch_bounds__(256) void colnorm_kernel(const TM* __restrict__ R, TM* __restrict__ qn, DaPtrTable qt,
+                                                      int rows, int r, float eps) {
+  __shared__ double part[4][64];
+  __shared__ float denom[64];
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int g = threadIdx.x >> 6;
+  const TM* Rb = R + (long long)b * rows * r;
+  double s = 0.0;
+  if (c < r)
+    for (int i = g; i < rows; i += 4) {
+      const float v = ld_as_float<TM>(Rb + (long long)i * r + c);
+      s += (double)v * (double)v;
+    }
+  part[g][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (g == 0) {
+    const double t = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+    denom[threadIdx.x] = sqrtf((float)t) + eps;
+  }
+  __syncthreads();
+  if (c < r) {
+    const float d = denom[threadIdx.x & 63];
+    TM* Qn = qn + (long long)b * rows * r;
+    TQ* Q = static_cast<TQ*>(qt.p[b]);
+    for (int i = g; i < rows; i += 4) {
+      const long long o = (long long)i * r + c;
+      const float v = ld_as_float<TM>(Rb + o) / d;
+      st_from_float<TM>(Qn + o, v);
+      st_from_float<TQ>(Q + o, ld_as_float<TM>(Qn + o));
+    }
+  }
+}
+
+inline unsigned ew_blocks(long long n) {
+  long long b = (n / 8 + 255) / 256;
+  return (unsigned)(b > 1024 ? 1024 : (b < 1 ? 1 : b));
+}
+
+}  // namespace
+
+int da_fill_int(int* p, int n, int v, hipStream_t s) {
+  hipLaunchKernelGGL(fill_int_kernel, dim3((n + 255) / 256), dim3(256), 0, s, p, n, v);
+  return da_launch_status();
+}
+
+int da_write_table(const DaPtrTable& t, void** dst, int n, hipStream_t s) {
+  if (n > DA_MAX_PTRS) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL(write_table_kernel, dim3(1), dim3(64), 0, s, t, dst, n);
+  return da_launch_status();
+}
+
+int da_add_grad(const DaPtrTable& m, const DaPtrTable& g, int m_dtype, int g_dtype, long long n, int batch,
+                int* nonzero, hipStream_t s) {
+  if (n & 7) return DA_ERR_ALIGN;
+  dim3 grid(ew_blocks(n), batch);
+  if (m_dtype == DA_BF16 && g_dtype == DA_BF16)
+    hipLaunchKernelGGL((add_grad_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, m, g, n, nonzero);
+  else if (m_dtype == DA_BF16 && g_dtype == DA_F32)
+    hipLaunchKernelGGL((add_grad_kernel<bf16_t, float>), grid, dim3(256), 0, s, m, g, n, nonzero);
+  else if (m_dtype == DA_F32 && g_dtype == DA_BF16)
+    hipLaunchKernelGGL((add_grad_kernel<float, bf16_t>), grid, dim3(256), 0, s, m, g, n, nonzero);
+  else if (m_dtype == DA_F32 && g_dtype == DA_F32)
+    hipLaunchKernelGGL((add_grad_kernel<float, float>), grid, dim3(256), 0, s, m, g, n, nonzero);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, long long n, int batch, hipStream_t s) {
+  if (n & 7) return DA_ERR_ALIGN;
+  dim3 grid(ew_blocks(n), batch);
+  if (s_dtype == DA_BF16 && d_dtype == DA_BF16)
+    hipLaunchKernelGGL((cast_table_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
+  else if (s_dtype == DA_F32 && d_dtype == DA_BF16)
+    hipLaunchKernelGGL((cast_table_kernel<float, bf16_t>), grid, dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
+  else if (s_dtype == DA_BF16 && d_dtype == DA_F32)
+    hipLaunchKernelGGL((cast_table_kernel<bf16_t, float>), grid, dim3(256), 0, s, src, static_cast<float*>(dst), n);
+  else if (s_dtype == DA_F32 && d_dtype == DA_F32)
+    hipLaunchKernelGGL((cast_table_kernel<float, float>), grid, dim3(256), 0, s, src, static_cast<float*>(dst), n);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const int* nonzero, hipStream_t s) {
+  if (n & 7) return DA_ERR_ALIGN;
+  dim3 grid(ew_blocks(n), batch);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL(fix_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(v), static_cast<const bf16_t*>(alt), n, nonzero);
+  else if (dtype == DA_F32)
+    hipLaunchKernelGGL(fix_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(v), static_cast<const float*>(alt), n, nonzero);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, float eps,
+               int batch, hipStream_t s) {
+  dim3 grid((r + 63) / 64, batch);
+  if (m_dtype == DA_BF16 && q_dtype == DA_BF16)
+    hipLaunchKernelGGL((colnorm_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, rows, r, eps);
+  else if (m_dtype == DA_BF16 && q_dtype == DA_F32)
+    hipLaunchKernelGGL((colnorm_kernel<bf16_t, float>), grid, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, rows, r, eps);
+  else if (m_dtype == DA_F32 && q_dtype == DA_BF16)
+    hipLaunchKernelGGL((colnorm_kernel<float, bf16_t>), grid, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, rows, r, eps);
+  else if (m_dtype == DA_F32 && q_dtype == DA_F32)
+    hipLaunchKernelGGL((colnorm_kernel<float, float>), grid, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, rows, r, eps);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// CholeskyQR2 in fp64
+// ---------------------------------------------------------------------------------------
+size_t da_orth_workspace_bytes(int batch, int rows, int r) {
+  const size_t nblk = (r + DA_CHOL_NB - 1) / DA_CHOL_NB;
+  size_t per = 2 * (size_t)rows * r * 8        // P0, P1
+               + (size_t)rows * DA_CHOL_NB * 8  // S
+               + 2 * (size_t)r * r * 8          // G, L
+               + nblk * DA_CHOL_NB * DA_CHOL_NB * 8;
+  return per * batch + 256;
+}
+
+int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
+                      int* info, hipStream_t s) {
+  const int NB = DA_CHOL_NB;
+  const int nblk = (r + NB - 1) / NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r, sS = (long long)rows * NB,
+                  sD = (long long)nblk * NB * NB;
+  double* P0 = static_cast<double*>(ws);
+  double* P1 = P0 + pr * batch;
+  double* S = P1 + pr * batch;
+  double* G = S + sS * batch;
+  double* L = G + rr * batch;
+  double* D = L + rr * batch;
+  int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
+  if (rc) return rc;
+  for (int pass = 0; pass < passes; ++pass) {
+    Gemm64Desc g{};
+    g.batch = batch;
+    // G = P0^T P0
+    g.A = P0; g.B = P0; g.C = G; g.E = nullptr;
+    g.sA = pr; g.sB = pr; g.sC = rr;
+    g.lda = r; g.ldb = r; g.ldc = r;
+    g.M = r; g.N = r; g.K = rows;
+    g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
+    rc = da_gemm_f64(g, s);
+    if (rc) return rc;
+    // blocked lower Cholesky G = L L^T
+    for (int j = 0; j < nblk; ++j) {
+      const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
+      rc = da_chol_diag(G, L, rr, r, o, nb, D + (long long)j * NB * NB, sD, info, batch, s);
+      if (rc) return rc;
+      if (rest <= 0) break;
+      Gemm64Desc t{};
+      t.batch = batch;
+      // L21 = A21 L11^-T
+      t.A = G + (long long)(o + nb) * r + o; t.sA = rr; t.lda = r; t.a_kstrided = 0;
+      t.B = D + (long long)j * NB * NB; t.sB = sD; t.ldb = NB; t.b_kstrided = 0;
+      t.C = L + (long long)(o + nb) * r + o; t.sC = rr; t.ldc = r;
+      t.M = rest; t.N = nb; t.K = nb; t.alpha = 1.0; t.beta = 0.0; t.E = nullptr;
+      rc = da_gemm_f64(t, s);
+      if (rc) return rc;
+      // A22 -= L21 L21^T
+      Gemm64Desc u{};
+      u.batch = batch;
+      u.A = t.C; u.sA = rr; u.lda = r; u.a_kstrided = 0;
+      u.B = t.C; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+      u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
+      u.E = u.C; u.sE = rr; u.lde = r;
+      u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0;
+      rc = da_gemm_f64(u, s);
+      if (rc) return rc;
+    }
+    // P1 = P0 R^-1 with R = L^T, block column by block column
+    for (int j = 0; j < nblk; ++j) {
+      const int o = j * NB, nb = r - o < NB ? r - o : NB;
+      Gemm64Desc a{};
+      a.batch = batch;
+      // S = P0[:, blk] - P1[:, :o] L[blk, :o]^T
+      a.A = P1; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+      a.B = L + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
+      a.C = S; a.sC = sS; a.ldc = NB;
+      a.E = P0 + o; a.sE = pr; a.lde = r;
+      a.M = rows; a.N = nb; a.K = o; a.alpha = -1.0; a.beta = 1.0;
+      rc = da_gemm_f64(a, s);
+      if (rc) return rc;
+      // P1[:, blk] = S L_jj^-T
+      Gemm64Desc c{};
+      c.batch = batch;
+      c.A = S; c.sA = sS; c.lda = NB; c.a_kstrided = 0;
+      c.B = D + (long long)j * NB * NB; c.sB = sD; c.ldb = NB; c.b_kstrided = 0;
+      c.C = P1 + o; c.sC = pr; c.ldc = r;
+      c.M = rows; c.N = nb; c.K = nb; c.alpha = 1.0; c.beta = 0.0; c.E = nullptr;
+      rc = da_gemm_f64(c, s);
+      if (rc) return rc;
+    }
+    double* tmp = P0; P0 = P1; P1 = tmp;
+  }
+  return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+}

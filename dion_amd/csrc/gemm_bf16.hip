@@ -149,8 +149,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
   }
   const int m0 = ti * BT, n0 = tj * BT;
 
-  const bf16_t* A = static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
-  const bf16_t* B = static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
+  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
+  const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
 
   f32x16_t acc[TM][TM];
 #pragma unroll
@@ -211,7 +211,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
   const bool mirror = SYM && (ti != tj);
   const bool has_e = d.epilogue == DA_EPI_AXPBY;
   const int wm0 = m0 + wm * W, wn0 = n0 + wn * W;
-  const long long cb = (long long)b * d.sC, eb = (long long)b * d.sE;
+  // C and E base pointers of this matrix, as byte addresses (element size depends on c_dtype)
+  const int csz = ep.c_f32 ? 4 : 2;
+  char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * csz;
+  const char* const Ebase = !has_e ? nullptr
+                            : d.Etab ? static_cast<const char*>(d.Etab[b])
+                                     : static_cast<const char*>(d.E) + (long long)b * d.sE * csz;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     {
@@ -238,19 +243,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
         const long long off = (long long)m * d.ldc + n;
         if (ep.c_f32) {
           if (has_e) {
-            const float* Ep = static_cast<const float*>(d.E) + eb + (long long)m * d.lde + n;
+            const float* Ep = reinterpret_cast<const float*>(Ebase) + (long long)m * d.lde + n;
             const float4 e0 = *reinterpret_cast<const float4*>(Ep);
             const float4 e1 = *reinterpret_cast<const float4*>(Ep + 4);
             e[0] = e0.x; e[1] = e0.y; e[2] = e0.z; e[3] = e0.w; e[4] = e1.x; e[5] = e1.y; e[6] = e1.z; e[7] = e1.w;
           }
 #pragma unroll
           for (int q = 0; q < 8; ++q) v[q] = epi_value(ep, v[q], e[q]);
-          float* Cp = static_cast<float*>(d.C) + cb + off;
+          float* Cp = reinterpret_cast<float*>(Cbase) + off;
           *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
           *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
         } else {
           if (has_e) {
-            const uint4 ev = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(d.E) + eb + (long long)m * d.lde + n);
+            const uint4 ev = *reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(Ebase) + (long long)m * d.lde + n);
             const uint32_t w[4] = {ev.x, ev.y, ev.z, ev.w};
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -267,7 +272,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
             v[2 * q] = bf2f(lo);
             v[2 * q + 1] = bf2f(hi);
           }
-          *reinterpret_cast<uint4*>(static_cast<bf16_t*>(d.C) + cb + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+          *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(Cbase) + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
         }
         if (mirror) {  // keep the final values for the transposed store
           *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
@@ -288,14 +293,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
           for (int q = 0; q < 8; ++q) v[q] = stg[(mg + q) * PITCH + nl];
           const long long off = (long long)n * d.ldc + m;
           if (ep.c_f32) {
-            float* Cp = static_cast<float*>(d.C) + cb + off;
+            float* Cp = reinterpret_cast<float*>(Cbase) + off;
             *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
             *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
           } else {
             uint32_t pk[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) pk[q] = (uint32_t)f2bf(v[2 * q]) | ((uint32_t)f2bf(v[2 * q + 1]) << 16);
-            *reinterpret_cast<uint4*>(static_cast<bf16_t*>(d.C) + cb + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(Cbase) + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
           }
         }
       }
@@ -336,12 +341,12 @@ int dispatch_layout(const GemmDesc& d, hipStream_t stream) {
 // Alignment contract: K, N, every leading dimension and every batch stride are multiples
 // of 8 elements (16-byte chunks); M too when A is k-strided; pointers 16-byte aligned.
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
-  if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
-  if (d.epilogue == DA_EPI_AXPBY && !d.E) return DA_ERR_ARG;
+  if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
+  if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
   if (d.c_dtype != DA_BF16 && d.c_dtype != DA_F32) return DA_ERR_DTYPE;
   if ((d.K | d.N | d.lda | d.ldb | d.ldc) & 7) return DA_ERR_ALIGN;
   if ((d.sA | d.sB | d.sC) & 7) return DA_ERR_ALIGN;
-  if (d.E && ((d.lde & 7) || (d.sE & 7))) return DA_ERR_ALIGN;
+  if ((d.E || d.Etab) && ((d.lde & 7) || (d.sE & 7))) return DA_ERR_ALIGN;
   if (d.a_kstrided && (d.M & 7)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;
   if (d.symmetric && (d.M != d.N || d.a_kstrided || d.b_kstrided)) return DA_ERR_ARG;

@@ -81,8 +81,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
     tj = t - ti * tiles_n;
   }
   const int m0 = ti * BT, n0 = tj * BT;
-  const float* A = static_cast<const float*>(d.A) + (long long)b * d.sA;
-  const float* B = static_cast<const float*>(d.B) + (long long)b * d.sB;
+  const float* A = d.Atab ? static_cast<const float*>(d.Atab[b]) : static_cast<const float*>(d.A) + (long long)b * d.sA;
+  const float* B = d.Btab ? static_cast<const float*>(d.Btab[b]) : static_cast<const float*>(d.B) + (long long)b * d.sB;
 
   f32x16_t acc[2][2];
 #pragma unroll
@@ -130,6 +130,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
 
   const bool mirror = SYM && (ti != tj);
   const bool has_e = d.epilogue == DA_EPI_AXPBY;
+  float* const Cbase = d.Ctab ? static_cast<float*>(d.Ctab[b]) : static_cast<float*>(d.C) + (long long)b * d.sC;
+  const float* const Ebase = !has_e ? nullptr
+                             : d.Etab ? static_cast<const float*>(d.Etab[b])
+                                      : static_cast<const float*>(d.E) + (long long)b * d.sE;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int m = m0 + wm * 64 + i * 32 + (lane & 31);
@@ -139,19 +143,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
       for (int vq = 0; vq < 4; ++vq) {
         const int n = n0 + wn * 64 + j * 32 + vq * 8 + (lane >> 5) * 4;
         if (m >= d.M || n >= d.N) continue;
-        float* Cp = static_cast<float*>(d.C) + (long long)b * d.sC + (long long)m * d.ldc + n;
+        float* Cp = Cbase + (long long)m * d.ldc + n;
         float o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) o[q] = d.s1 * acc[i][j][vq * 4 + q];
         if (has_e) {
-          const float4 ev = *reinterpret_cast<const float4*>(static_cast<const float*>(d.E) + (long long)b * d.sE +
-                                                             (long long)m * d.lde + n);
+          const float4 ev = *reinterpret_cast<const float4*>(Ebase + (long long)m * d.lde + n);
           o[0] = d.s0 * ev.x + o[0]; o[1] = d.s0 * ev.y + o[1];
           o[2] = d.s0 * ev.z + o[2]; o[3] = d.s0 * ev.w + o[3];
         }
         *reinterpret_cast<float4*>(Cp) = make_float4(o[0], o[1], o[2], o[3]);
         if (mirror) {
-          float* Ct = static_cast<float*>(d.C) + (long long)b * d.sC + (long long)n * d.ldc + m;
+          float* Ct = Cbase + (long long)n * d.ldc + m;
 #pragma unroll
           for (int q = 0; q < 4; ++q) Ct[(long long)q * d.ldc] = o[q];
         }
@@ -175,12 +178,12 @@ int launch(const GemmDesc& d, hipStream_t stream) {
 // Alignment contract: K, N, leading dimensions and batch strides multiples of 4 elements,
 // M too when A is k-strided; pointers 16-byte aligned.  C and E are fp32.
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream) {
-  if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
-  if (d.epilogue == DA_EPI_AXPBY && !d.E) return DA_ERR_ARG;
+  if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
+  if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
   if (d.c_dtype != DA_F32) return DA_ERR_DTYPE;
   if ((d.K | d.N | d.lda | d.ldb | d.ldc) & 3) return DA_ERR_ALIGN;
   if ((d.sA | d.sB | d.sC) & 3) return DA_ERR_ALIGN;
-  if (d.E && ((d.lde & 3) || (d.sE & 3))) return DA_ERR_ALIGN;
+  if ((d.E || d.Etab) && ((d.lde & 3) || (d.sE & 3))) return DA_ERR_ALIGN;
   if (d.a_kstrided && (d.M & 3)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;
   if (d.symmetric) {

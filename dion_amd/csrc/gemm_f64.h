@@ -1,0 +1,33 @@
+// fp64 building blocks of the CholeskyQR orthonormalisation (see gemm_f64.hip, cholesky.hip).
+#pragma once
+#include "common.h"
+
+// C[b] (M x N) = alpha * sum_k Aop[b](i,k) Bop[b](j,k) + beta * E[b]   (all fp64, row-major)
+// Operand layouts as in GemmDesc.  E may alias C.  K == 0 is allowed (C = beta * E).
+struct Gemm64Desc {
+  const double* A;
+  const double* B;
+  double* C;
+  const double* E;
+  long long sA, sB, sC, sE;
+  int lda, ldb, ldc, lde;
+  int M, N, K, batch;
+  int a_kstrided, b_kstrided, symmetric;
+  double alpha, beta;
+};
+
+int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
+
+// dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s);
+int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s);
+
+// Factor the nb x nb diagonal block at offset `o` of each r x r matrix G[b] (lower Cholesky,
+// G = L L^T), write L11 into Lmat[b] at the same position, and its inverse (lower
+// triangular, pitch nb) into Dinv[b].  A non-positive or non-finite pivot zeroes that
+// column (of L11 and of the inverse) and records (o + column + 1) in info[b] if it is the
+// first failure of that matrix.
+int da_chol_diag(const double* G, double* Lmat, long long sG, int r, int o, int nb, double* Dinv, long long sD,
+                 int* info, int batch, hipStream_t s);
+
+#define DA_CHOL_NB 64

@@ -1,0 +1,176 @@
+// Batched fp64 GEMM on the matrix cores (v_mfma_f64_16x16x4_f64) for the CholeskyQR
+// orthonormalisation of Dion's P factor: the r x r Gram matrix P^T P (its condition number
+// is the square of P's, hence fp64), the blocked Cholesky's panel / trailing updates and
+// the blocked triangular solve P R^-1.
+//
+//   C[b] (M x N) = alpha * sum_k Aop[b](i,k) * Bop[b](j,k) + beta * E[b]
+//
+// 256 threads (2 x 2 wavefronts) per 64 x 64 tile, 16 k per stage; each wavefront owns
+// 32 x 32 as 2 x 2 accumulators of 16 x 16.  LDS tiles are k-major [16][64] doubles for
+// either operand layout, so the one-double-per-lane MFMA operands are conflict-free reads.
+// The fp64 MFMA takes 64 cycles, which hides the staging of the next tile.
+#include "gemm_f64.h"
+
+namespace {
+
+constexpr int BT = 64;
+constexpr int BK = 16;
+
+// Stage one 64 x 16 operand tile into lds[k][row].  4 elements per thread.
+template <bool KS>
+__device__ __forceinline__ void stage(double* lds, const double* __restrict__ base, int ld, int row0, int k0,
+                                      int rows, int K, int tid) {
+  if (!KS) {
+    const int r = tid >> 2, k4 = (tid & 3) * 4;
+    const int gr = row0 + r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int gk = k0 + k4 + e;
+      lds[(k4 + e) * BT + r] = (gr < rows && gk < K) ? base[(long long)gr * ld + gk] : 0.0;
+    }
+  } else {
+    const int k = tid >> 4, r4 = (tid & 15) * 4;
+    const int gk = k0 + k;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int gr = row0 + r4 + e;
+      lds[k * BT + r4 + e] = (gr < rows && gk < K) ? base[(long long)gk * ld + gr] : 0.0;
+    }
+  }
+}
+
+template <bool A_KS, bool B_KS, bool SYM>
+__global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
+  __shared__ double lds_a[BK * BT];
+  __shared__ double lds_b[BK * BT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
+  const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  const int b = blockIdx.x / per_batch;
+  int t = blockIdx.x - b * per_batch;
+  int ti, tj;
+  if (SYM) {
+    ti = 0;
+    int len = tiles_m;
+    while (t >= len) { t -= len; ++ti; --len; }
+    tj = ti + t;
+  } else {
+    ti = t / tiles_n;
+    tj = t - ti * tiles_n;
+  }
+  const int m0 = ti * BT, n0 = tj * BT;
+  const double* A = d.A + (long long)b * d.sA;
+  const double* B = d.B + (long long)b * d.sB;
+
+  f64x4_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+
+  for (int k0 = 0; k0 < d.K; k0 += BK) {
+    stage<A_KS>(lds_a, A, d.lda, m0, k0, d.M, d.K, tid);
+    stage<B_KS>(lds_b, B, d.ldb, n0, k0, d.N, d.K, tid);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < BK / 4; ++ks) {
+      const int k = ks * 4 + (lane >> 4);
+      double af[2], bfv[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = lds_a[k * BT + wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bfv[j] = lds_b[k * BT + wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // D layout: lane l, register v -> row 4 v + (l >> 4), column (l & 15)
+  double* C = d.C + (long long)b * d.sC;
+  const double* E = d.E ? d.E + (long long)b * d.sE : nullptr;
+  const bool mirror = SYM && (ti != tj);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = m0 + wm * 32 + i * 16 + v * 4 + (lane >> 4);
+        const int n = n0 + wn * 32 + j * 16 + (lane & 15);
+        if (m < d.M && n < d.N) {
+          double o = d.alpha * acc[i][j][v];
+          if (E) o += d.beta * E[(long long)m * d.lde + n];
+          C[(long long)m * d.ldc + n] = o;
+          if (mirror) C[(long long)n * d.ldc + m] = o;
+        }
+      }
+}
+
+template <bool A_KS, bool B_KS, bool SYM>
+int launch(const Gemm64Desc& d, hipStream_t s) {
+  const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
+  const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
+  const long long blocks = per_batch * d.batch;
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL((gemm_f64_kernel<A_KS, B_KS, SYM>), dim3((unsigned)blocks), dim3(256), 0, s, d);
+  return da_launch_status();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void cvt_to_f64_kernel(const T* __restrict__ src, double* __restrict__ dst,
+                                                         long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    dst[i] = (double)ld_as_float<T>(src + i);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void cvt_from_f64_kernel(const double* __restrict__ src, T* __restrict__ dst,
+                                                           long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    st_from_float<T>(dst + i, (float)src[i]);
+}
+
+inline unsigned cvt_blocks(long long n) {
+  long long b = (n + 255) / 256;
+  return (unsigned)(b > 8192 ? 8192 : (b < 1 ? 1 : b));
+}
+
+}  // namespace
+
+int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) {
+  if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K < 0 || d.batch <= 0) return DA_ERR_ARG;
+  if (d.symmetric) {
+    if (d.M != d.N || !d.a_kstrided || !d.b_kstrided) return DA_ERR_ARG;  // only the Gram form A^T A
+    return launch<true, true, true>(d, s);
+  }
+  if (!d.a_kstrided && !d.b_kstrided) return launch<false, false, false>(d, s);
+  if (!d.a_kstrided && d.b_kstrided) return launch<false, true, false>(d, s);
+  if (d.a_kstrided && !d.b_kstrided) return launch<true, false, false>(d, s);
+  return launch<true, true, false>(d, s);
+}
+
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  if (src_dtype == DA_BF16)
+    hipLaunchKernelGGL(cvt_to_f64_kernel<bf16_t>, dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n);
+  else if (src_dtype == DA_F32)
+    hipLaunchKernelGGL(cvt_to_f64_kernel<float>, dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  if (dst_dtype == DA_BF16)
+    hipLaunchKernelGGL(cvt_from_f64_kernel<bf16_t>, dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
+  else if (dst_dtype == DA_F32)
+    hipLaunchKernelGGL(cvt_from_f64_kernel<float>, dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<float*>(dst), n);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}

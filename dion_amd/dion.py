@@ -1,0 +1,264 @@
+"""`Dion` optimizer whose matrix path runs on the MI355X kernels.
+
+Signature-compatible with the reference class (dion/dion.py:75-231): same constructor
+arguments, defaults, validation errors, param-group keys and `self.state` layout
+(`state[p]["momentum"]`, `state[p]["Q"]`, plus `"variance"` for AdamW groups).  One GPU only:
+`replicate_mesh`, `outer_shard_mesh` and `inner_shard_mesh` must be None.
+
+Per `step()` the matrices of every "dion" group are bucketed by (shape, dtype) and each bucket
+goes, as arrays of device pointers, to `dion_amd_dion_step`: B = M + G, the tall-skinny MFMA
+GEMMs P = B Q and R = B^T P, an fp64 CholeskyQR2 orthonormalisation of P on the device, the
+error-feedback and weight updates fused into GEMM epilogues, and the column normalisation
+that yields the next Q.
+"""
+import math
+from collections import defaultdict
+from dataclasses import dataclass
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+from torch import Tensor
+from torch.optim.optimizer import Optimizer, ParamsT
+
+from . import _lib
+from .elementwise_opts import adamw_update_foreach, lion_update_foreach
+
+
+@dataclass
+class DionMixedPrecisionConfig:
+    """dtypes of the optimizer states (reference dion/dion.py:59-72); None = the parameter's dtype."""
+
+    momentum_dtype: Optional[torch.dtype] = None
+    Q_dtype: Optional[torch.dtype] = None
+    variance_dtype: Optional[torch.dtype] = None
+
+
+class Dion(Optimizer):
+    """
+    Dion (https://arxiv.org/abs/2504.05295) for a single MI355X.
+
+    Args (identical to the reference, dion/dion.py:105-124):
+        params: parameters or param-group dicts; `algorithm` in {"dion", "lion", "adamw"}.
+        replicate_mesh, outer_shard_mesh, inner_shard_mesh: must be None (one GPU).
+        replicate_mesh_grad_sync: accepted; irrelevant on one GPU.
+        rank_fraction, rank_multiple_of: r = multiple_of * ceil(fraction * min(m, n) / multiple_of).
+        lr, mu, betas, weight_decay, epsilon: as in the reference.
+        power_iters: must be 1.  qr_method: must be "rcqr" (the reference's only accepted value;
+            the device orthonormaliser is a CholeskyQR2 that yields the same factor up to column signs).
+        cqr_warmup_steps, rcqr_oversample: accepted for compatibility (no sketch is drawn).
+        mixed_precision_config: dtypes of momentum / Q / variance.
+    """
+
+    def __init__(
+        self,
+        params: ParamsT,
+        replicate_mesh=None,
+        outer_shard_mesh=None,
+        inner_shard_mesh=None,
+        replicate_mesh_grad_sync: bool = True,
+        rank_fraction: float = 1.0,
+        rank_multiple_of: int = 1,
+        lr: float = 0.01,
+        mu: float = 0.95,
+        betas: Tuple[float, float] = (0.9, 0.95),
+        weight_decay: float = 0.01,
+        epsilon: float = 1e-8,
+        power_iters: int = 1,
+        qr_method: str = "rcqr",
+        cqr_warmup_steps: int = 150,
+        rcqr_oversample: float = 1.25,
+        mixed_precision_config: Optional[DionMixedPrecisionConfig] = None,
+    ):
+        if lr < 0.0:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if mu < 0.0:
+            raise ValueError(f"Invalid momentum factor (mu): {mu}")
+        if len(betas) != 2 or betas[0] < 0.0 or betas[1] < 0.0:
+            raise ValueError(f"Invalid betas: {betas}")
+        if weight_decay < 0.0:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        if rank_fraction <= 0 or rank_fraction > 1:
+            raise ValueError(f"Invalid rank fraction: {rank_fraction}")
+        if rank_multiple_of <= 0:
+            raise ValueError(f"Invalid rank multiple of: {rank_multiple_of}")
+        if power_iters != 1:
+            raise ValueError("Async Dion only supports power_iters=1")
+        if qr_method != "rcqr":
+            raise ValueError("Async Dion only supports qr_method='rcqr'")
+        for name, mesh in (("replicate_mesh", replicate_mesh), ("outer_shard_mesh", outer_shard_mesh),
+                           ("inner_shard_mesh", inner_shard_mesh)):
+            if mesh is not None:
+                raise NotImplementedError(
+                    f"dion_amd.Dion runs on one GPU: {name} must be None (got {type(mesh).__name__})."
+                )
+
+        defaults = dict(
+            rank_fraction=rank_fraction, rank_multiple_of=rank_multiple_of, lr=lr, mu=mu,
+            beta1=betas[0], beta2=betas[1], weight_decay=weight_decay, epsilon=epsilon,
+            oversample=rcqr_oversample, algorithm="dion", step=0,
+        )
+        super().__init__(params, defaults)
+
+        self._replicate_mesh = None
+        self._outer_shard_mesh = None
+        self._inner_shard_mesh = None
+        self._replicate_mesh_grad_sync = replicate_mesh_grad_sync
+        self._replicate_world_size = 1
+        if mixed_precision_config is None:
+            mixed_precision_config = DionMixedPrecisionConfig()
+        self._mixed_precision_config = mixed_precision_config
+        self._workspace = _lib.Workspace()
+        self._info = {}
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+
+        dion_groups, lion_groups, adamw_groups = [], [], []
+        for group in self.param_groups:
+            group["step"] += 1
+            algo = group["algorithm"]
+            if algo == "dion":
+                dion_groups.append(group)
+            elif algo == "lion":
+                lion_groups.append(group)
+            elif algo == "adamw":
+                adamw_groups.append(group)
+            else:
+                raise ValueError(f"Unknown algorithm: {algo}")
+
+        for group in dion_groups:
+            self._dion_group_step(group)
+        for group in lion_groups:
+            self._lion_group_step(group)
+        for group in adamw_groups:
+            self._adamw_group_step(group)
+        return loss
+
+    @torch.no_grad()
+    def synchronize_for_checkpoint(self):
+        """No-op on one GPU (reference dion/dion.py:273-287)."""
+        return
+
+    def cholesky_info(self) -> Dict[Tuple, Tensor]:
+        """Device tensors with the orthonormaliser's per-matrix status of the last step, keyed by bucket:
+        0 = success, k > 0 = pivot k-1 was not positive (the analogue of `torch.linalg.cholesky_ex`'s info)."""
+        return dict(self._info)
+
+    # ------------------------------------------------------------------ state
+    def _get_or_initialize_state(self, param: Tensor, group: dict) -> dict:
+        state = self.state[param]
+        algo = group["algorithm"]
+        if not state:
+            if algo == "dion":
+                self._init_opt_state_dion(param, state, group["rank_fraction"], group["rank_multiple_of"])
+            elif algo == "adamw":
+                self._init_opt_state_adam(param, state)
+            elif algo == "lion" or algo == "clion":
+                self._init_opt_state_momentum(param, state)
+            else:
+                raise ValueError(f"Unknown algorithm: {algo}")
+        return state
+
+    def _init_opt_state_momentum(self, param: Tensor, state: Dict[str, Any]):
+        state["momentum"] = torch.zeros_like(param, dtype=self._mixed_precision_config.momentum_dtype)
+
+    def _init_opt_state_adam(self, param: Tensor, state: Dict[str, Any]):
+        self._init_opt_state_momentum(param, state)
+        state["variance"] = torch.zeros_like(param, dtype=self._mixed_precision_config.variance_dtype)
+
+    def _init_opt_state_dion(self, param: Tensor, state: Dict[str, Any], rank_fraction: float, rank_multiple_of: int):
+        """momentum = 0 and Q ~ N(0, 1) of shape (n, r), or (m, r) when m < n (reference dion/dion.py:649-721)."""
+        if param.ndim != 2:
+            raise ValueError(
+                f"Expected Dion parameters to be 2D matrix, but got {param.ndim}D. "
+                f"For scalar parameters, set 'algorithm' to 'lion' or 'adamw' when creating param group."
+            )
+        self._init_opt_state_momentum(param, state)
+        m, n = param.shape
+        r = rank_fraction * min(m, n)
+        r = rank_multiple_of * math.ceil(r / rank_multiple_of)
+        r = min(r, m, n)
+        q_shape = (m, r) if m < n else (n, r)
+        q_dtype = self._mixed_precision_config.Q_dtype
+        if q_dtype is None:
+            q_dtype = param.dtype
+        state["Q"] = torch.randn(q_shape, device=param.device, dtype=q_dtype)
+
+    # ------------------------------------------------------------------ dion
+    def _dion_group_step(self, group: dict):
+        params = [p for p in group["params"] if p.grad is not None]
+        if not params:
+            return
+        for p in params:
+            if p.ndim > 2:
+                raise NotImplementedError(
+                    f"Tensors with more than 2 dimensions are not supported. Got {p.ndim}D tensor."
+                )
+        # hyper-parameters as 0-dim fp32 tensors, evaluated like reference dion/dion.py:327-331, 852, 859-870
+        lr = torch.tensor(group["lr"])
+        mu = torch.tensor(group["mu"])
+        weight_decay = torch.tensor(group["weight_decay"])
+        epsilon = torch.tensor(group["epsilon"])
+        ef_alpha = -(1 - mu)
+        decay = 1 - lr * weight_decay
+
+        buckets = defaultdict(list)
+        for p in params:
+            buckets[(p.shape, p.dtype, p.grad.dtype, p.device)].append(p)
+        lib = _lib.load()
+        for (shape, dtype, gdtype, device), plist in buckets.items():
+            _lib.require_gpu(plist[0], "Dion.step")
+            states = [self._get_or_initialize_state(p, group) for p in plist]
+            m, n = shape
+            Ms = [s["momentum"] for s in states]
+            Qs = [s["Q"] for s in states]
+            r = Qs[0].size(1)
+            Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
+            for t in (*plist, *Ms, *Qs):
+                if not t.is_contiguous():
+                    raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
+            scaled_lr = ((m / n) ** 0.5) * lr
+            mcode = _lib.dtype_code(Ms[0].dtype)
+            ws = self._workspace.get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
+            info = self._info.get((shape, dtype, device))
+            if info is None or info.numel() != len(plist):
+                info = torch.zeros(len(plist), dtype=torch.int32, device=device)
+                self._info[(shape, dtype, device)] = info
+            with torch.cuda.device(device):
+                rc = lib.dion_amd_dion_step(
+                    _lib.ptr_array(plist), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
+                    len(plist), m, n, r,
+                    _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
+                    ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1,
+                    info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
+                )
+            _lib.check(rc, "dion_amd_dion_step")
+            del Gs
+
+    # ------------------------------------------------------------------ element-wise groups
+    def _lion_group_step(self, group: dict):
+        params = [p for p in group["params"] if p.grad is not None]
+        if not params:
+            return
+        states = [self._get_or_initialize_state(p, group) for p in params]
+        lion_update_foreach(
+            params, [p.grad for p in params], [s["momentum"] for s in states],
+            lr=torch.tensor(group["lr"]), beta1=torch.tensor(group["beta1"]), beta2=torch.tensor(group["beta2"]),
+            weight_decay=torch.tensor(group["weight_decay"]),
+        )
+
+    def _adamw_group_step(self, group: dict):
+        params = [p for p in group["params"] if p.grad is not None]
+        if not params:
+            return
+        states = [self._get_or_initialize_state(p, group) for p in params]
+        adamw_update_foreach(
+            params, [p.grad for p in params], [s["momentum"] for s in states], [s["variance"] for s in states],
+            lr=torch.tensor(group["lr"]), beta1=torch.tensor(group["beta1"]), beta2=torch.tensor(group["beta2"]),
+            weight_decay=torch.tensor(group["weight_decay"]), step=torch.tensor(group["step"]),
+            epsilon=torch.tensor(group["epsilon"]),
+        )

@@ -141,3 +141,22 @@ def gemm(A: Tensor, B: Tensor, *, a_kstrided=False, b_kstrided=False, E: Tensor 
             _lib.stream_ptr(A.device))
     _lib.check(rc, "dion_amd_gemm")
     return out if A.ndim == 3 else out[0]
+
+
+def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False):
+    """Thin-QR Q factor of P (rows x r) or a batch of them on the device (CholeskyQR `passes` times in fp64);
+    counterpart of `orthogonalize` (reference dion/dion.py:1267-1308), equal up to column signs."""
+    lib = _lib.load()
+    _lib.require_gpu(P, "orthonormalize")
+    P3 = (P if P.ndim == 3 else P.unsqueeze(0)).contiguous()
+    batch, rows, r = P3.shape
+    out = torch.empty_like(P3)
+    info = torch.zeros(batch, dtype=torch.int32, device=P.device)
+    nbytes = lib.dion_amd_orthonormalize_workspace_bytes(batch, rows, r)
+    ws = _workspace.get(nbytes, P.device)
+    with torch.cuda.device(P.device):
+        rc = lib.dion_amd_orthonormalize(P3.data_ptr(), out.data_ptr(), _lib.dtype_code(P.dtype), batch, rows, r,
+                                         passes, info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(P.device))
+    _lib.check(rc, "dion_amd_orthonormalize")
+    out = out if P.ndim == 3 else out[0]
+    return (out, info) if return_info else out

@@ -121,6 +121,46 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
                        void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Dion step for one bucket of same-shape matrices
+ * ------------------------------------------------------------------------------------- */
+
+size_t dion_amd_orthonormalize_workspace_bytes(int batch, int rows, int r);
+
+/* Replaces orthogonalize (reference dion/dion.py:1267-1308; per-matrix variants
+ * dion/dion_reference.py:733-789): thin-QR Q factor of each of `batch` contiguous matrices
+ * P_b (rows x r, rows >= r, dtype bf16 or f32), written to out_b (same layout; may alias P).
+ * Method: CholeskyQR repeated `passes` times (2 = CholeskyQR2) with the Gram matrix, the
+ * blocked Cholesky factorisation and the triangular solve all in fp64 on the device; no
+ * host synchronisation.  The factor equals the reference's Householder / randomised
+ * Cholesky QR result up to column signs (Cholesky's diagonal is positive).
+ * info (device, `batch` ints, may be NULL): 0, or 1 + the first column whose pivot was not
+ * positive -- the analogue of torch.linalg.cholesky_ex's info; such columns come out as 0. */
+int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
+                            int* info, void* workspace, size_t workspace_bytes, void* stream);
+
+size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype);
+
+/* Replaces dion_update_ddp with replicate_mesh=None (reference dion/dion.py:742-875) and its
+ * helpers tensor_list_to_batch (1200-1218), orthogonalize (1267-1308), fix_all_zero_or_nan
+ * (1416-1444), column_normalize (1460-1491), foreach_baddbmm_ (1494-1530) and
+ * update_Q_matrix_ (1533-1561), for a bucket of `batch` matrices of identical shape m x n.
+ *
+ * X, G, M, Q: HOST arrays of `batch` device pointers: weights (m x n, x_dtype), gradients
+ * (g_dtype), momentum (m_dtype) and the power-iteration factor Q ((min(m,n)) x r... i.e.
+ * n x r when m >= n, m x r when m < n; q_dtype), all contiguous, all updated in place
+ * except G.  Per matrix, with B' = B if m >= n else B^T:
+ *   B = M + G;  P = orth(B' Q);  R = B'^T P;  (all-zero / NaN guard on P, R)
+ *   M <- B - (1-mu) P R^T  (transposed back when m < n);   Q <- R / (||R||_col + eps);
+ *   X <- decay X - scaled_lr P Q^T.
+ * ef_alpha = -(1 - mu), decay = 1 - lr*wd and scaled_lr = sqrt(m/n)*lr are passed as
+ * already-evaluated fp32 values.  m_dtype f32 requires x_dtype f32.  info as above. */
+int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q,
+                       int batch, int m, int n, int r,
+                       int x_dtype, int g_dtype, int m_dtype, int q_dtype,
+                       float ef_alpha, float decay, float scaled_lr, float eps, int faithful,
+                       int* info, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Measurement hooks (no counterpart in the reference; used by the benchmark only)
  * ------------------------------------------------------------------------------------- */
 
