@@ -1,15 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X Muon / Dion optimizer-step hot path (one GPU).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu-baseline]
 
-A "step" is one full optimizer step over every matrix of the workload with synthetic
-Gaussian gradients already resident in HBM.  Prints ONE JSON line.
+A "step" is one full optimizer step over every matrix of the workload, with synthetic
+Gaussian gradients already resident in HBM.  Prints ONE JSON line whose `value` is the
+milliseconds per step of the selected workload; the other BASELINE configurations that fit
+in a short run are reported under `extra`.
 
 Workloads (BASELINE.json `configs`):
-  muon_gpt_small   (default) full Muon step, GPT-small: 72 bf16 matrices (48 x 768^2,
-                   12 x 3072x768, 12 x 768x3072), G ~ N(0,1e-3) seed 1, mu 0.95 Nesterov.
-  muon_llama8b_layer   Muon NS5 on one Llama-3-8B layer's matrices (bf16), seed 4.
+  muon_gpt_small        (default, configs[1]) full Muon step, GPT-small: 72 bf16 matrices
+                        (48 x 768^2, 12 x 3072x768, 12 x 768x3072), G ~ N(0,1e-3) seed 1, Nesterov.
+  dion_gpt_small_r025   (configs[2]) full Dion step on the same matrices, rank fraction 0.25,
+  dion_gpt_small_r1     rank fraction 1.0; bf16 weights / momentum, fp32 Q, G seed 3.
+  muon_llama8b_layer    (configs[3], one of the 32 layers) Muon on 7 bf16 matrices incl. 4096x14336.
+  dion_llama70b_layer   (configs[4], one of the 8 layers) Dion r=512 on 2 x 28672x8192 + 8192x28672.
 """
 import argparse
 import json
@@ -25,25 +30,31 @@ PEAK_HBM_BPS = 8.0e12      # MI355X HBM3E
 
 GPT_SMALL_LAYER = [(768, 768)] * 4 + [(3072, 768), (768, 3072)]
 LLAMA8B_LAYER = [(4096, 4096)] * 2 + [(1024, 4096)] * 2 + [(14336, 4096)] * 2 + [(4096, 14336)]
+LLAMA70B_MLP_LAYER = [(28672, 8192)] * 2 + [(8192, 28672)]
 
 WORKLOADS = {
-    "muon_gpt_small": dict(shapes=GPT_SMALL_LAYER * 12, seed=1,
+    "muon_gpt_small": dict(kind="muon", shapes=GPT_SMALL_LAYER * 12, seed=1,
                            desc="Full Muon step, GPT-small (12 layers, d=768): 72 bf16 matrices"),
-    "muon_llama8b_layer": dict(shapes=LLAMA8B_LAYER, seed=4,
+    "dion_gpt_small_r025": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=0.25,
+                                desc="Full Dion step, GPT-small matrices, rank fraction 0.25 (r=192), bf16 M, fp32 Q"),
+    "dion_gpt_small_r1": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=1.0,
+                              desc="Full Dion step, GPT-small matrices, rank fraction 1.0 (r=768), bf16 M, fp32 Q"),
+    "muon_llama8b_layer": dict(kind="muon", shapes=LLAMA8B_LAYER, seed=4,
                                desc="Muon step, one Llama-3-8B layer: 7 bf16 matrices incl. 4096x14336"),
+    "dion_llama70b_layer": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER, seed=5, rank_fraction=1.0 / 16,
+                                desc="Dion step, one Llama-3-70B MLP layer (28672x8192 x2, 8192x28672), r=512"),
 }
+GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd")
 
 
-def make_problem(shapes, seed, device, dtype):
+def make_problem(shapes, seed, dtype):
     import torch
 
     gen = torch.Generator(device="cpu").manual_seed(seed)
     params, grads = [], []
     for s in shapes:
-        w = (torch.randn(s, generator=gen) * 0.02).to(dtype)
-        g = (torch.randn(s, generator=gen) * 1e-3).to(dtype)
-        params.append(w)
-        grads.append(g)
+        params.append((torch.randn(s, generator=gen) * 0.02).to(dtype))
+        grads.append((torch.randn(s, generator=gen) * 1e-3).to(dtype))
     return params, grads
 
 
@@ -55,73 +66,49 @@ def ns_flops(shapes, symmetric):
     return tot
 
 
-def cpu_baseline(shapes, seed, budget_s=20.0):
-    """The oracle (eager-PyTorch CPU restatement of the reference step) timed on the host cores."""
+def build_optimizer(wl, dev):
     import torch
-    from oracle import muon_step as O
+    from dion_amd import Dion, DionMixedPrecisionConfig, Muon
 
-    X, G = make_problem(shapes, seed, "cpu", torch.bfloat16)
-    M = [torch.zeros_like(x) for x in X]
-    t0 = time.perf_counter()
-    O.muon_step(X, G, M, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True)  # warm-up
-    first = time.perf_counter() - t0
-    reps = max(1, min(10, int(budget_s / max(first, 1e-3)) - 1))
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        O.muon_step(X, G, M, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True)
-    ms = (time.perf_counter() - t0) / reps * 1e3
-    return dict(value=round(ms, 3), unit="ms", cores=torch.get_num_threads(), kind="port",
-                sample=f"{reps} full steps of the same {len(shapes)}-matrix workload after 1 warm-up "
-                       f"(eager PyTorch CPU, bf16, Nesterov)")
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="muon_gpt_small", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
-              file=sys.stderr)
-        sys.exit(2)
-
-    import torch
-    from dion_amd import Muon, _lib
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    dev = torch.device("cuda:0")
-    wl = WORKLOADS[args.workload]
-    shapes = wl["shapes"]
-    X, G = make_problem(shapes, wl["seed"], dev, torch.bfloat16)
+    X, G = make_problem(wl["shapes"], wl["seed"], torch.bfloat16)
     params = [torch.nn.Parameter(x.to(dev)) for x in X]
     for p, g in zip(params, G):
         p.grad = g.to(dev)
-    opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True, adjust_lr="spectral_norm")
+    if wl["kind"] == "muon":
+        opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True, adjust_lr="spectral_norm")
+        desc = "Muon(lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr=spectral_norm)"
+    else:
+        torch.manual_seed(2)
+        opt = Dion(params, rank_fraction=wl["rank_fraction"], lr=0.01, mu=0.95, weight_decay=0.01,
+                   mixed_precision_config=DionMixedPrecisionConfig(momentum_dtype=torch.bfloat16, Q_dtype=torch.float32))
+        desc = (f"Dion(rank_fraction={wl['rank_fraction']:.4g}, lr=0.01, mu=0.95, weight_decay=0.01, "
+                "momentum bf16, Q fp32)")
+    return opt, params, desc
 
-    for _ in range(args.warmup):
+
+def measure(wl, dev, steps, warmup):
+    """Timed region + a second pass of the same steps with per-launch HIP events."""
+    import torch
+    from dion_amd import _lib
+
+    opt, params, desc = build_optimizer(wl, dev)
+    for _ in range(warmup):
         opt.step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(args.steps):
+    for _ in range(steps):
         opt.step()
     e1.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ev_ms = e0.elapsed_time(e1) / args.steps
-    ms_per_step = max(wall_ms, ev_ms)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
 
-    # per-kernel HIP-event timing of the same steps (events bracket every launch on its stream)
     lib = _lib.load()
     lib.dion_amd_profile_reset()
     lib.dion_amd_profile_enable(1)
-    for _ in range(args.steps):
+    for _ in range(steps):
         opt.step()
     torch.cuda.synchronize()
     lib.dion_amd_profile_enable(0)
@@ -130,50 +117,144 @@ def main():
 
     kernels = {}
     for name, (n, ms, work) in prof.items():
-        is_gemm = name.startswith("ns_") or name in ("gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd")
         rate = work / (ms * 1e-3) if ms > 0 else 0.0
-        kernels[name] = dict(launches_per_step=n / args.steps, avg_ms=ms / n, ms_per_step=ms / args.steps,
-                             **({"tflops": rate / 1e12, "frac_mfma": rate / PEAK_BF16_FLOPS} if is_gemm
-                                else {"gbps": rate / 1e9, "frac_hbm": rate / PEAK_HBM_BPS}))
-    gemm_kinds = [k for k in ("ns_syrk", "ns_poly", "ns_axpy") if k in prof]
-    dom = max(gemm_kinds, key=lambda k: prof[k][1])
+        k = dict(launches_per_step=round(n / steps, 2), avg_ms=round(ms / n, 5), ms_per_step=round(ms / steps, 4))
+        if name in GEMM_KINDS:
+            k.update(tflops=round(rate / 1e12, 1), frac_mfma=round(rate / PEAK_BF16_FLOPS, 4))
+        elif work > 0:
+            k.update(gbps=round(rate / 1e9, 1), frac_hbm=round(rate / PEAK_HBM_BPS, 4))
+        kernels[name] = k
+    res = dict(ms_per_step=max(wall_ms, ev_ms), wall_ms=wall_ms, event_ms=ev_ms, kernels=kernels, prof=prof,
+               optimizer=desc, steps=steps)
+    del opt, params
+    torch.cuda.empty_cache()
+    return res
+
+
+def summarize(name, wl, res):
+    shapes = wl["shapes"]
+    out = dict(workload=name, ms_per_step=round(res["ms_per_step"], 4), steps=res["steps"],
+               orthogonalisations_per_s=round(len(shapes) / (res["ms_per_step"] * 1e-3), 1))
+    prof = res["prof"]
+    if wl["kind"] == "muon":
+        ns_ms = sum(prof[k][1] for k in ("ns_syrk", "ns_poly", "ns_axpy") if k in prof) / res["steps"]
+        f_sym = ns_flops(shapes, True)
+        out.update(ns_gemm_ms_per_step=round(ns_ms, 4),
+                   ns_executed_tflops=round(f_sym / (ns_ms * 1e-3) / 1e12, 1),
+                   ns_frac_mfma_peak=round(f_sym / (ns_ms * 1e-3) / PEAK_BF16_FLOPS, 4),
+                   ns_dense_convention_tflops=round(ns_flops(shapes, False) / (ns_ms * 1e-3) / 1e12, 1))
+    out["kernels"] = res["kernels"]
+    return out
+
+
+def roofline_of(res, kind):
+    """Dominant GEMM kernel of the run: algorithmic flops per launch / average launch duration."""
+    prof = res["prof"]
+    cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
+                         else ("dion_bq", "dion_btp", "dion_ef", "dion_upd")) if k in prof]
+    dom = max(cands, key=lambda k: prof[k][1])
     n, ms, work = prof[dom]
     achieved = work / (ms * 1e-3) / 1e12
-    roofline = dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=PEAK_BF16_FLOPS / 1e12,
-                    unit="TFLOP/s", frac=round(achieved * 1e12 / PEAK_BF16_FLOPS, 4), traffic=None,
-                    avg_launch_ms=round(ms / n, 5),
-                    flops_per_launch=work / n)
-    ns_ms = sum(prof[k][1] for k in gemm_kinds) / args.steps
-    f_sym = ns_flops(shapes, True)
+    return dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=PEAK_BF16_FLOPS / 1e12, unit="TFLOP/s",
+                frac=round(achieved * 1e12 / PEAK_BF16_FLOPS, 4), traffic=None,
+                avg_launch_ms=round(ms / n, 5), flops_per_launch=work / n)
+
+
+def cpu_baseline(wl, budget_s=20.0):
+    """The oracle (eager-PyTorch CPU restatement of the reference step) timed on the host cores."""
+    import torch
+
+    shapes = wl["shapes"]
+    X, G = make_problem(shapes, wl["seed"], torch.bfloat16)
+    if wl["kind"] == "muon":
+        from oracle import muon_step as O
+
+        M = [torch.zeros_like(x) for x in X]
+
+        def step():
+            O.muon_step(X, G, M, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True)
+        what = "eager PyTorch CPU, bf16, Nesterov"
+    else:
+        from oracle import dion_step as O
+
+        torch.manual_seed(2)
+        M = [torch.zeros_like(x) for x in X]
+        Q = [torch.randn((min(s), O.rank_of(s[0], s[1], wl["rank_fraction"]))) for s in shapes]
+        gen = torch.Generator().manual_seed(0)
+
+        def step():
+            O.dion_step(X, G, M, Q, lr=0.01, mu=0.95, weight_decay=0.01, generator=gen)
+        what = "eager PyTorch CPU, bf16 momentum, fp32 Q, reference orthogonalize rule"
+    t0 = time.perf_counter()
+    step()  # warm-up
+    first = time.perf_counter() - t0
+    reps = max(1, min(10, int(budget_s / max(first, 1e-3)) - 1))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step()
+    ms = (time.perf_counter() - t0) / reps * 1e3
+    return dict(value=round(ms, 3), unit="ms", cores=torch.get_num_threads(), kind="port",
+                sample=f"{reps} full steps of the same {len(shapes)}-matrix workload after 1 warm-up ({what})")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="muon_gpt_small", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    wl = WORKLOADS[args.workload]
+    res = measure(wl, dev, args.steps, args.warmup)
+    main_sum = summarize(args.workload, wl, res)
 
     out = {
         "metric": "Muon/Dion optimizer-step ms (GPT-160M, 8B-layer) + % bf16 MFMA peak",
-        "value": round(ms_per_step, 4),
+        "value": round(res["ms_per_step"], 4),
         "unit": "ms",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": round(res["ms_per_step"], 4),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": args.workload, "description": wl["desc"], "matrices": len(shapes),
-                   "optimizer": "Muon(lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr=spectral_norm)",
-                   "grad": f"N(0,1e-3) seed {wl['seed']}", "parallelism": "single GPU"},
-        "orthogonalisations_per_s": round(len(shapes) / (ms_per_step * 1e-3), 1),
-        "ns_gemm_ms_per_step": round(ns_ms, 4),
-        "ns_executed_tflops": round(f_sym / (ns_ms * 1e-3) / 1e12, 2) if ns_ms > 0 else None,
-        "ns_frac_mfma_peak": round(f_sym / (ns_ms * 1e-3) / PEAK_BF16_FLOPS, 4) if ns_ms > 0 else None,
-        "ns_dense_convention_tflops": round(ns_flops(shapes, False) / (ns_ms * 1e-3) / 1e12, 2) if ns_ms > 0 else None,
-        "event_ms_per_step": round(ev_ms, 4),
-        "wall_ms_per_step": round(wall_ms, 4),
-        "roofline": roofline,
-        "kernels": kernels,
+        "config": {"workload": args.workload, "description": wl["desc"], "matrices": len(wl["shapes"]),
+                   "optimizer": res["optimizer"], "grad": f"N(0,1e-3) seed {wl['seed']}", "parallelism": "single GPU"},
+        "event_ms_per_step": round(res["event_ms"], 4),
+        "wall_ms_per_step": round(res["wall_ms"], 4),
+        "roofline": roofline_of(res, wl["kind"]),
     }
+    out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
+    if not args.no_extra:
+        extra = {}
+        for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "dion_llama70b_layer"):
+            if name == args.workload:
+                continue
+            w = WORKLOADS[name]
+            big = "llama" in name
+            r = measure(w, dev, 3 if big else 10, 1 if big else 2)
+            s = summarize(name, w, r)
+            s["roofline"] = roofline_of(r, w["kind"])
+            extra[name] = s
+        out["extra"] = extra
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(shapes, wl["seed"])
+        out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
 
 

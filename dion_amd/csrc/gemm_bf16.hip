@@ -2,100 +2,137 @@
 //
 //   C[b] (M x N) = epilogue( sum_k Aop[b](i,k) * Bop[b](j,k) )
 //
-// Work decomposition: one 256-thread workgroup (4 wavefronts of 64 lanes, 2 x 2) per
-// BT x BT output tile, BT in {128, 256}; each wavefront owns a (BT/2) x (BT/2) sub-tile
-// as (BT/64)^2 accumulators of 32 x 32.  The K loop advances 64 elements per stage and
-// is double buffered through LDS: while the matrix cores work on stage s, the 16-byte
-// global loads of stage s+1 are in flight in registers.
+// Work decomposition: one workgroup per BT x BT output tile.  Two shapes are built:
+//   * BT = 256, 8 wavefronts (2 x 4): each wavefront owns 128 x 64 as 4 x 2 accumulators of
+//     32 x 32.  Two wavefronts share a SIMD, so while one waits for LDS or a barrier the
+//     other keeps the matrix core busy; LDS traffic is 6 fragment reads per 8 MFMAs.
+//   * BT = 128, 4 wavefronts (2 x 2), 64 x 64 each: for problems too small to fill the
+//     256 CUs with large tiles.
+// The K loop advances 64 elements per stage and is double buffered through LDS.
 //
 // Operand staging in LDS:
 //   * k-contiguous operand (rows x K in memory): tile [BT][64] of 16-byte chunks, chunk
-//     index XOR-swizzled with (row & 7) so that the 32 rows one ds_read_b128 fragment
-//     read touches spread over all banks.
-//   * k-strided operand (K x rows in memory, e.g. X in  X' = aX + B X): the tile is kept
-//     exactly as it lies in memory, [64][BT + 16], and the fragment is fetched with two
-//     ds_read_b64_tr_b16 (the LDS transpose read of CDNA4), which hands each lane the four
-//     k-consecutive values of its own column.  No register shuffles, no second copy of X.
+//     index XOR-swizzled with ((row >> 1) & 7): the 16 lanes served per clock by a
+//     ds_read_b128 fragment read (16 consecutive rows, same logical chunk) then fall into
+//     16 different 16-byte slots of the 64-bank, 256-byte LDS line.
+//   * k-strided operand (K x rows in memory, e.g. X in  X' = aX + B X): the tile keeps the
+//     memory orientation, [64][BT] with 32-byte slots XOR-swizzled by (k-row & 3), and the
+//     fragment is fetched with two ds_read_b64_tr_b16 (the LDS transpose read of CDNA4),
+//     which hands each lane the four k-consecutive values of its own column.  No register
+//     shuffles, no second copy of X.
+// Interior tiles are staged with direct-to-LDS loads (global_load_lds_dwordx4): no staging
+// registers and no ds_write instructions; the swizzles are applied to the global address.
 //
 // The MFMA is issued with the operands swapped (D' = Bfrag x Afrag^T), so that a lane ends
-// up with four *column-consecutive* results of one output row: 8-byte epilogue loads and
-// stores for row-major C and E.  For a symmetric result only tiles on or above the
-// diagonal are computed and every off-diagonal tile is also written transposed.
+// up with four *column-consecutive* results of one output row; the epilogue then passes the
+// accumulators through LDS so that C and E move as 16-byte row segments.  For a symmetric
+// result only tiles on or above the diagonal are computed and every off-diagonal tile is
+// also written transposed.
 #include "common.h"
+#include <cstdlib>
 
 namespace {
 
-constexpr int BK = 64;       // k elements per stage
-constexpr int KS_PAD = 16;   // padding (elements) per k-row of a k-strided LDS tile
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 
-template <int BT, bool KS>
-struct Tile {
-  static constexpr int ks_ld = BT + KS_PAD;
-  static constexpr int bytes = KS ? BK * ks_ld * 2 : BT * BK * 2;
-  static constexpr int chunks = BT / 32;  // 16-byte chunks per thread per stage
+constexpr int BK = 64;       // k elements per stage
+
+template <int BT_, int WGM_, int WGN_>
+struct Cfg {
+  static constexpr int BT = BT_, WGM = WGM_, WGN = WGN_;
+  static constexpr int NT = 64 * WGM * WGN;        // threads
+  static constexpr int TMI = BT / (32 * WGM);      // accumulators per wavefront, row direction
+  static constexpr int TNJ = BT / (32 * WGN);      // ... column direction
+  static constexpr int NCH = BT * 8 / NT;          // 16-byte chunks per thread per operand stage
+  static constexpr int WROWS = BT / WGM, WCOLS = BT / WGN;
 };
 
 template <int BT, bool KS>
-__device__ __forceinline__ void load_tile_global(uint4 (&r)[BT / 32], const bf16_t* __restrict__ base, int ld,
-                                                 int row0, int k0, int rows, int K, int tid) {
-#pragma unroll
-  for (int i = 0; i < BT / 32; ++i) {
-    const int c = tid + 256 * i;
-    uint4 v = make_uint4(0u, 0u, 0u, 0u);
-    if (!KS) {
-      const int gr = row0 + (c >> 3);
-      const int gk = k0 + (c & 7) * 8;
-      if (gr < rows && gk < K) v = *reinterpret_cast<const uint4*>(base + (long long)gr * ld + gk);
-    } else {
-      constexpr int CPR = BT / 8;  // chunks per k-row
-      const int gk = k0 + c / CPR;
-      const int gr = row0 + (c % CPR) * 8;
-      if (gk < K && gr < rows) v = *reinterpret_cast<const uint4*>(base + (long long)gk * ld + gr);
-    }
-    r[i] = v;
-  }
-}
+struct Tile {
+  static constexpr int bytes = BT * BK * 2;   // either layout: 64 x BT bf16
+};
 
-template <int BT, bool KS>
-__device__ __forceinline__ void store_tile_lds(const uint4 (&r)[BT / 32], char* lds, int tid) {
-#pragma unroll
-  for (int i = 0; i < BT / 32; ++i) {
-    const int c = tid + 256 * i;
+// Physical 16-byte chunk of a k-contiguous tile row ([BT][8 chunks]) and of a k-strided tile
+// row ([64][BT/8 chunks], 32-byte slots swizzled with the k-row).
+__device__ __forceinline__ int kc_swizzle(int chunk, int row) { return chunk ^ ((row >> 1) & 7); }
+__device__ __forceinline__ int ks_swizzle(int chunk, int krow) { return (((chunk >> 1) ^ (krow & 3)) << 1) | (chunk & 1); }
+
+// Per-thread addressing of the NCH 16-byte chunks a thread moves per operand stage.
+//   Register-staged path (bounds-checked): chunk i lies at global `g + i * gstep` (elements)
+//   and goes to LDS byte offset `l + i * lstep`.
+//   Direct-to-LDS path: wave-instruction i of wavefront w fills the 1024-byte LDS block
+//   (i * NW + w); lane p of it fetches the chunk whose *physical* position is p, i.e. the
+//   swizzle is applied to the global address (`gd + i * gdstep`).
+template <typename C, bool KS>
+struct StageAddr {
+  const bf16_t* g;
+  const bf16_t* gd;
+  long long gstep, gdstep, tstep;   // per chunk (register / direct) and per stage, in elements
+  int l, lstep;
+  int row, col;             // first chunk's (row within tile, k offset) resp. (k row, row offset)
+  __device__ __forceinline__ StageAddr(const bf16_t* base, int ld, int row0, int tid) {
+    constexpr int NW = C::NT / 64;
+    const int lane = tid & 63, wave = tid >> 6;
     if (!KS) {
-      const int row = c >> 3;
-      const int phys = (c & 7) ^ (row & 7);
-      *reinterpret_cast<uint4*>(lds + row * 128 + phys * 16) = r[i];
+      row = tid >> 3;
+      col = (tid & 7) * 8;
+      g = base + (long long)(row0 + row) * ld + col;
+      gstep = (long long)(C::NT / 8) * ld;
+      tstep = BK;
+      l = row * 128 + kc_swizzle(tid & 7, row) * 16;
+      lstep = (C::NT / 8) * 128;   // NT/8 is a multiple of 16: the swizzle term is the same for all chunks
+      const int drow = wave * 8 + (lane >> 3);             // block (0 * NW + wave), 8 rows per block
+      gd = base + (long long)(row0 + drow) * ld + kc_swizzle(lane & 7, drow) * 8;
+      gdstep = (long long)(NW * 8) * ld;                   // NW * 8 is a multiple of 16
     } else {
-      constexpr int CPR = BT / 8;
-      const int kr = c / CPR;
-      const int mc = c % CPR;
-      *reinterpret_cast<uint4*>(lds + (kr * Tile<BT, true>::ks_ld + mc * 8) * 2) = r[i];
+      constexpr int CPR = C::BT / 8;                       // chunks per k-row
+      constexpr int RPB = 64 / CPR;                        // k-rows per 1024-byte block
+      row = tid / CPR;
+      col = (tid % CPR) * 8;
+      g = base + (long long)row * ld + row0 + col;
+      gstep = (long long)(C::NT / CPR) * ld;
+      tstep = (long long)BK * ld;
+      l = row * (C::BT * 2) + ks_swizzle(tid % CPR, row) * 16;
+      lstep = (C::NT / CPR) * (C::BT * 2);                 // NT / CPR = 16: swizzle term unchanged
+      const int drow = wave * RPB + lane / CPR;
+      gd = base + (long long)drow * ld + row0 + ks_swizzle(lane % CPR, drow) * 8;
+      gdstep = (long long)(NW * RPB) * ld;                 // NW * RPB = 16
     }
   }
-}
+};
 
 // Fragment of 32 rows x 16 k for one MFMA: lane l gets row (l & 31), k = 8 * (l >> 5) .. +8.
 template <int BT, bool KS>
 __device__ __forceinline__ bf16x8_t read_frag(const char* lds, int r0, int ks, int lane) {
   if (!KS) {
     const int row = r0 + (lane & 31);
-    const int phys = (ks * 2 + (lane >> 5)) ^ (row & 7);
-    const uint4 v = *reinterpret_cast<const uint4*>(lds + row * 128 + phys * 16);
+    const int phys = kc_swizzle(ks * 2 + (lane >> 5), row);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * 128 + phys * 16);
     return __builtin_bit_cast(bf16x8_t, v);
   } else {
     // Per 16-lane group g: rows r0 + 16 * (g & 1) .. +16, k-group g >> 1.  The four lanes
     // 4q .. 4q+3 of a group together supply 16 consecutive rows of k-row q; the transpose
-    // read returns to lane i of the group the four k values of row i.
-    constexpr int LD = Tile<BT, true>::ks_ld;
+    // read returns to lane i of the group the four k values of row i.  The 32-byte slot a
+    // group reads is swizzled with (k-row & 3) = q, so its four k-rows hit different banks.
     const int g = lane >> 4;
-    const int col = r0 + (g & 1) * 16 + (lane & 3) * 4;
-    const int kr = ks * 16 + (g >> 1) * 8 + ((lane & 15) >> 2);
-    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, lds + (kr * LD + col) * 2));
-    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, lds + ((kr + 4) * LD + col) * 2));
+    const int q = (lane & 15) >> 2;
+    const int slot = ((r0 >> 4) + (g & 1)) ^ q;
+    const int kr = ks * 16 + (g >> 1) * 8 + q;
+    const char* p = lds + kr * (BT * 2) + slot * 32 + (lane & 3) * 8;
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, p));
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, p + 4 * (BT * 2)));
     typedef short s16x8_t __attribute__((ext_vector_type(8)));
     const s16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(bf16x8_t, v);
   }
+}
+
+__device__ __forceinline__ int wave_uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// 16 bytes per lane from global memory straight into LDS: lane p's data lands at l + 16 p
+// (l must be wave-uniform).
+__device__ __forceinline__ void dma16(const void* g, char* l) {
+  __builtin_amdgcn_global_load_lds(g, DA_LDS_PTR(void, l), 16, 0, 0);
 }
 
 struct Epi {
@@ -118,91 +155,49 @@ __device__ __forceinline__ float epi_value(const Epi& ep, float acc, float e) {
   return ep.mode == DA_EPI_AXPBY ? ep.s0 * e + ep.s1 * acc : ep.s1 * acc;
 }
 
-template <int BT, bool A_KS, bool B_KS, bool SYM>
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
-  constexpr int TM = BT / 64;  // 32x32 accumulators per wavefront in each direction
-  constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
-  constexpr int B_BYTES = Tile<BT, B_KS>::bytes;
-  constexpr int STAGE = A_BYTES + B_BYTES;
-  extern __shared__ __attribute__((aligned(16))) char lds[];
+// Which output tile a workgroup owns.  Workgroups are dealt round-robin to the 8 XCDs (each
+// with its own L2), so consecutive *logical* tiles -- which share an operand panel -- are
+// mapped to the same XCD when the grid divides evenly.
+struct TileId { int b, ti, tj; };
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-
-  // ---- which tile ---------------------------------------------------------------
+template <int BT, bool SYM>
+__device__ __forceinline__ TileId decode_tile(const GemmDesc& d) {
   const int tiles_m = (d.M + BT - 1) / BT;
   const int tiles_n = (d.N + BT - 1) / BT;
   const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
-  const int b = blockIdx.x / per_batch;
-  int t = blockIdx.x - b * per_batch;
-  int ti, tj;
+  int bid = blockIdx.x;
+  const int nblk = gridDim.x;
+  if ((nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  TileId r;
+  r.b = bid / per_batch;
+  int t = bid - r.b * per_batch;
   if (SYM) {
-    ti = 0;
+    r.ti = 0;
     int len = tiles_m;
-    while (t >= len) { t -= len; ++ti; --len; }
-    tj = ti + t;
+    while (t >= len) { t -= len; ++r.ti; --len; }
+    r.tj = r.ti + t;
+  } else if ((tiles_m % 4) == 0 && (tiles_n % 8) == 0) {
+    // 4 x 8 super-tiles: the 32 workgroups that an XCD runs at a time then share 4 A panels
+    // and 8 B panels (12 panel loads per k-step instead of 33 for a row of 32 tiles)
+    const int sup = t >> 5, within = t & 31;
+    const int sup_per_row = tiles_n >> 3;
+    const int sr = sup / sup_per_row, sc = sup - sr * sup_per_row;
+    r.ti = sr * 4 + (within >> 3);
+    r.tj = sc * 8 + (within & 7);
   } else {
-    ti = t / tiles_n;
-    tj = t - ti * tiles_n;
+    r.ti = t / tiles_n;
+    r.tj = t - r.ti * tiles_n;
   }
-  const int m0 = ti * BT, n0 = tj * BT;
+  return r;
+}
 
-  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
-  const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
-
-  f32x16_t acc[TM][TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  uint4 ra[BT / 32], rb[BT / 32];
-  const int KT = (d.K + BK - 1) / BK;
-
-  load_tile_global<BT, A_KS>(ra, A, d.lda, m0, 0, d.M, d.K, tid);
-  load_tile_global<BT, B_KS>(rb, B, d.ldb, n0, 0, d.N, d.K, tid);
-  store_tile_lds<BT, A_KS>(ra, lds, tid);
-  store_tile_lds<BT, B_KS>(rb, lds + A_BYTES, tid);
-  __syncthreads();
-
-  for (int kt = 0; kt < KT; ++kt) {
-    const char* sa = lds + (kt & 1) * STAGE;
-    const char* sb = sa + A_BYTES;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      load_tile_global<BT, A_KS>(ra, A, d.lda, m0, (kt + 1) * BK, d.M, d.K, tid);
-      load_tile_global<BT, B_KS>(rb, B, d.ldb, n0, (kt + 1) * BK, d.N, d.K, tid);
-    }
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8_t af[TM], bfr[TM];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) af[i] = read_frag<BT, A_KS>(sa, wm * (BT / 2) + i * 32, ks, lane);
-#pragma unroll
-      for (int j = 0; j < TM; ++j) bfr[j] = read_frag<BT, B_KS>(sb, wn * (BT / 2) + j * 32, ks, lane);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
-    }
-    if (more) {
-      char* na = lds + ((kt + 1) & 1) * STAGE;
-      store_tile_lds<BT, A_KS>(ra, na, tid);
-      store_tile_lds<BT, B_KS>(rb, na + A_BYTES, tid);
-    }
-    __syncthreads();
-  }
-
-  // ---- epilogue -------------------------------------------------------------------
-  // The accumulators go through LDS (the stage buffers are free now), one 32-row band of
-  // the wavefront's sub-tile at a time, so that C and E move as 16-byte row segments and
-  // the code stays small enough to keep every accumulator index a compile-time constant.
-  constexpr int W = BT / 2;          // columns of a wavefront's sub-tile
+// The accumulators go through LDS (the stage buffers are free by now), one 32-row band of the
+// wavefront's sub-tile at a time, so that C and E move as 16-byte row segments and the code
+// stays small enough to keep every accumulator index a compile-time constant.
+template <typename C, bool SYM>
+__device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
+                                         int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
+  constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
   constexpr int PITCH = W + 4;       // floats; 16-byte aligned rows, conflict-free float4 writes
   constexpr int CPR = W / 8;         // 8-column chunks per row
   constexpr int RPP = 64 / CPR;      // rows per pass of the wavefront
@@ -210,7 +205,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
   const Epi ep{d.s0, d.s1, d.epilogue, d.faithful, d.c_dtype == DA_F32};
   const bool mirror = SYM && (ti != tj);
   const bool has_e = d.epilogue == DA_EPI_AXPBY;
-  const int wm0 = m0 + wm * W, wn0 = n0 + wn * W;
+  const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
   // C and E base pointers of this matrix, as byte addresses (element size depends on c_dtype)
   const int csz = ep.c_f32 ? 4 : 2;
   char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * csz;
@@ -218,11 +213,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
                             : d.Etab ? static_cast<const char*>(d.Etab[b])
                                      : static_cast<const char*>(d.E) + (long long)b * d.sE * csz;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < C::TMI; ++i) {
     {
       float* row = stg + (lane & 31) * PITCH + (lane >> 5) * 4;
 #pragma unroll
-      for (int j = 0; j < TM; ++j)
+      for (int j = 0; j < C::TNJ; ++j)
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq)
           *reinterpret_cast<float4*>(row + j * 32 + vq * 8) =
@@ -309,31 +304,169 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmDesc d) {
   }
 }
 
-template <int BT, bool A_KS, bool B_KS, bool SYM>
+// ---------------------------------------------------------------------------------------
+// One kernel, two K loops.
+//   FULL: every tile is interior (M, N multiples of BT, K a multiple of 64).  Stages are
+//     fetched with direct-to-LDS loads issued one stage ahead; the only wait is the
+//     vmcnt(0) in front of the per-stage barrier.
+//   !FULL: bounds-checked 16-byte loads into registers (out-of-range chunks zero filled),
+//     written to LDS after the stage's MFMAs.
+// ---------------------------------------------------------------------------------------
+template <typename C, bool A_KS, bool B_KS, bool SYM, bool FULL>
+__global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
+  constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ, NCH = C::NCH, NW = C::NT / 64;
+  constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
+  constexpr int B_BYTES = Tile<BT, B_KS>::bytes;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = wave_uniform(tid >> 6);
+  const int wm = wave / C::WGN, wn = wave % C::WGN;
+  const TileId tile = decode_tile<BT, SYM>(d);
+  const int b = tile.b, ti = tile.ti, tj = tile.tj;
+  const int m0 = ti * BT, n0 = tj * BT;
+  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
+  const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
+
+  f32x16_t acc[TMI][TNJ];
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNJ; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  StageAddr<C, A_KS> sa(A, d.lda, m0, tid);
+  StageAddr<C, B_KS> sb(B, d.ldb, n0, tid);
+  const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
+  const int KT = (d.K + BK - 1) / BK;
+  bf16x8_t fa[TMI], fb[TNJ];
+
+#define DA_FREAD(st, ks)                                                                           \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        fa[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
+    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
+        fb[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+  } while (0)
+#define DA_MMA()                                                                                   \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0); \
+  } while (0)
+
+  if (FULL) {
+// one stage of both operands, straight into LDS: NCH wave-instructions of 1024 bytes each
+#define DA_DMA(st)                                                                                 \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        dma16(sa.gd + i * sa.gdstep, (st) + (i * NW + wave) * 1024);                               \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        dma16(sb.gd + i * sb.gdstep, (st) + A_BYTES + (i * NW + wave) * 1024);                     \
+    sa.gd += sa.tstep;                                                                             \
+    sb.gd += sb.tstep;                                                                             \
+  } while (0)
+    DA_DMA(lds);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      char* cur = lds + (kt & 1) * STAGE;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE;
+      if (kt + 1 < KT) DA_DMA(nxt);
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        DA_FREAD(cur, ks);
+        DA_MMA();
+      }
+      __syncthreads();
+    }
+#undef DA_DMA
+  } else {
+    u32x4_t ra[NCH], rb[NCH];
+    constexpr int A_RSTEP = A_KS ? C::NT / (BT / 8) : C::NT / 8;  // tile rows (k rows if k-strided) per chunk
+    constexpr int B_RSTEP = B_KS ? C::NT / (BT / 8) : C::NT / 8;
+#define DA_GLOAD(kt)                                                                               \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
+      const int r_ = sa.row + i * A_RSTEP;                                                         \
+      const bool ok = A_KS ? ((kt) * BK + r_ < d.K && m0 + sa.col < d.M)                           \
+                           : (m0 + r_ < d.M && (kt) * BK + sa.col < d.K);                          \
+      const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
+      ra[i] = ok ? *reinterpret_cast<const u32x4_t*>(sa.g + i * sa.gstep) : z_;                    \
+    }                                                                                              \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
+      const int r_ = sb.row + i * B_RSTEP;                                                         \
+      const bool ok = B_KS ? ((kt) * BK + r_ < d.K && n0 + sb.col < d.N)                           \
+                           : (n0 + r_ < d.N && (kt) * BK + sb.col < d.K);                          \
+      const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
+      rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;                    \
+    }                                                                                              \
+    sa.g += sa.tstep;                                                                              \
+    sb.g += sb.tstep;                                                                              \
+  } while (0)
+#define DA_LSTORE(st)                                                                              \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        *reinterpret_cast<u32x4_t*>((st) + sa.l + i * sa.lstep) = ra[i];                           \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        *reinterpret_cast<u32x4_t*>((st) + A_BYTES + sb.l + i * sb.lstep) = rb[i];                 \
+  } while (0)
+    DA_GLOAD(0);
+    DA_LSTORE(lds);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      char* cur = lds + (kt & 1) * STAGE;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE;
+      const bool more = kt + 1 < KT;
+      if (more) DA_GLOAD(kt + 1);
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        DA_FREAD(cur, ks);
+        DA_MMA();
+      }
+      if (more) DA_LSTORE(nxt);
+      __syncthreads();
+    }
+#undef DA_GLOAD
+#undef DA_LSTORE
+  }
+#undef DA_FREAD
+#undef DA_MMA
+  epilogue<C, SYM>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
+}
+
+template <typename C, bool A_KS, bool B_KS, bool SYM>
 int launch(const GemmDesc& d, hipStream_t stream) {
-  constexpr int smem = 2 * (Tile<BT, A_KS>::bytes + Tile<BT, B_KS>::bytes);
-  auto kern = gemm_bf16_kernel<BT, A_KS, B_KS, SYM>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
+  constexpr int BT = C::BT;
+  constexpr int stage2 = 2 * (Tile<BT, A_KS>::bytes + Tile<BT, B_KS>::bytes);
+  constexpr int epi = (C::NT / 64) * 32 * (C::WCOLS + 4) * 4;
+  constexpr int smem = stage2 > epi ? stage2 : epi;
+  const bool full = (d.M % BT == 0) && (d.N % BT == 0) && (d.K % BK == 0);
+  auto kfull = gemm_bf16_kernel<C, A_KS, B_KS, SYM, true>;
+  auto kgen = gemm_bf16_kernel<C, A_KS, B_KS, SYM, false>;
+  static bool configured = false;  // benign race: the attribute calls are idempotent
   if (!configured) {
-    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kfull), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kgen), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
   const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
   const long long blocks = per_batch * d.batch;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), smem, stream, d);
+  hipLaunchKernelGGL(full ? kfull : kgen, dim3((unsigned)blocks), dim3(C::NT), smem, stream, d);
   return da_launch_status();
 }
 
-template <int BT>
+template <typename C>
 int dispatch_layout(const GemmDesc& d, hipStream_t stream) {
-  if (d.symmetric) return launch<BT, false, false, true>(d, stream);
-  if (!d.a_kstrided && !d.b_kstrided) return launch<BT, false, false, false>(d, stream);
-  if (!d.a_kstrided && d.b_kstrided) return launch<BT, false, true, false>(d, stream);
-  if (d.a_kstrided && !d.b_kstrided) return launch<BT, true, false, false>(d, stream);
-  return launch<BT, true, true, false>(d, stream);
+  if (d.symmetric) return launch<C, false, false, true>(d, stream);
+  if (!d.a_kstrided && !d.b_kstrided) return launch<C, false, false, false>(d, stream);
+  if (!d.a_kstrided && d.b_kstrided) return launch<C, false, true, false>(d, stream);
+  if (d.a_kstrided && !d.b_kstrided) return launch<C, true, false, false>(d, stream);
+  return launch<C, true, true, false>(d, stream);
 }
 
 }  // namespace
@@ -341,7 +474,8 @@ int dispatch_layout(const GemmDesc& d, hipStream_t stream) {
 // Alignment contract: K, N, every leading dimension and every batch stride are multiples
 // of 8 elements (16-byte chunks); M too when A is k-strided; pointers 16-byte aligned.
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
-  if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
+  if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0)
+    return DA_ERR_ARG;
   if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
   if (d.c_dtype != DA_BF16 && d.c_dtype != DA_F32) return DA_ERR_DTYPE;
   if ((d.K | d.N | d.lda | d.ldb | d.ldc) & 7) return DA_ERR_ALIGN;
@@ -350,8 +484,13 @@ int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
   if (d.a_kstrided && (d.M & 7)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;
   if (d.symmetric && (d.M != d.N || d.a_kstrided || d.b_kstrided)) return DA_ERR_ARG;
+  typedef Cfg<256, 2, 4> Big;
+  typedef Cfg<128, 2, 2> Small;
+  static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
+  if (forced == 128) return dispatch_layout<Small>(d, stream);
+  if (forced == 256) return dispatch_layout<Big>(d, stream);
   // Large tiles once there are enough of them to cover the 256 CUs; small tiles otherwise.
   const long long t256 = (long long)((d.M + 255) / 256) * ((d.N + 255) / 256) * d.batch / (d.symmetric ? 2 : 1);
-  if (d.M >= 1024 && d.N >= 1024 && t256 >= 200) return dispatch_layout<256>(d, stream);
-  return dispatch_layout<128>(d, stream);
+  if (d.M >= 1024 && d.N >= 1024 && t256 >= 200) return dispatch_layout<Big>(d, stream);
+  return dispatch_layout<Small>(d, stream);
 }
