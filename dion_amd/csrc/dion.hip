@@ -69,7 +69,8 @@ __global__ __launch_bounds__(256) void add_grad_kernel(DaPtrTable mt, DaPtrTable
     }
     V8<TM>::store(M + i, m);
   }
-  if (__any(any) && (threadIdx.x & 63) == 0) atomicOr(nonzero + b, 1);
+  // every writer stores the same value: no atomic needed
+  if (__any(any) && (threadIdx.x & 63) == 0) nonzero[b] = 1;
 }
 
 // dst[b] (contiguous, TD) <- src table[b] (TS)

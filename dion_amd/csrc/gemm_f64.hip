@@ -8,7 +8,7 @@
 // 256 threads (2 x 2 wavefronts) per 64 x 64 tile, 16 k per stage; each wavefront owns
 // 32 x 32 as 2 x 2 accumulators of 16 x 16.  LDS tiles are k-major [16][64] doubles for
 // either operand layout, so the one-double-per-lane MFMA operands are conflict-free reads.
-// The fp64 MFMA takes 64 cycles, which hides the staging of the next tile.
+// Double buffered: the global loads of the next stage are in flight during the MFMAs.
 #include "gemm_f64.h"
 
 namespace {
@@ -16,33 +16,43 @@ namespace {
 constexpr int BT = 64;
 constexpr int BK = 16;
 
-// Stage one 64 x 16 operand tile into lds[k][row].  4 elements per thread.
+// One 64 x 16 operand tile: 4 elements per thread, fetched into registers (zero filled out of
+// range) and later written to lds[k][row].
 template <bool KS>
-__device__ __forceinline__ void stage(double* lds, const double* __restrict__ base, int ld, int row0, int k0,
+__device__ __forceinline__ void fetch(double (&v)[4], const double* __restrict__ base, int ld, int row0, int k0,
                                       int rows, int K, int tid) {
+  // the thread's 4 elements are contiguous in memory in either layout
+  const int outer = KS ? k0 + (tid >> 4) : row0 + (tid >> 2);
+  const int inner = KS ? row0 + (tid & 15) * 4 : k0 + (tid & 3) * 4;
+  const int outer_n = KS ? K : rows, inner_n = KS ? rows : K;
+  const double* p = base + (long long)outer * ld + inner;
+  if (outer < outer_n && inner + 3 < inner_n && ((reinterpret_cast<uintptr_t>(p) & 15) == 0)) {
+    const double2 lo = *reinterpret_cast<const double2*>(p);
+    const double2 hi = *reinterpret_cast<const double2*>(p + 2);
+    v[0] = lo.x; v[1] = lo.y; v[2] = hi.x; v[3] = hi.y;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (outer < outer_n && inner + e < inner_n) ? p[e] : 0.0;
+  }
+}
+
+template <bool KS>
+__device__ __forceinline__ void put(double* lds, const double (&v)[4], int tid) {
   if (!KS) {
     const int r = tid >> 2, k4 = (tid & 3) * 4;
-    const int gr = row0 + r;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int gk = k0 + k4 + e;
-      lds[(k4 + e) * BT + r] = (gr < rows && gk < K) ? base[(long long)gr * ld + gk] : 0.0;
-    }
+    for (int e = 0; e < 4; ++e) lds[(k4 + e) * BT + r] = v[e];
   } else {
     const int k = tid >> 4, r4 = (tid & 15) * 4;
-    const int gk = k0 + k;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int gr = row0 + r4 + e;
-      lds[k * BT + r4 + e] = (gr < rows && gk < K) ? base[(long long)gk * ld + gr] : 0.0;
-    }
+    for (int e = 0; e < 4; ++e) lds[k * BT + r4 + e] = v[e];
   }
 }
 
 template <bool A_KS, bool B_KS, bool SYM>
 __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
-  __shared__ double lds_a[BK * BT];
-  __shared__ double lds_b[BK * BT];
+  __shared__ double lds_a[2][BK * BT];
+  __shared__ double lds_b[2][BK * BT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
@@ -69,22 +79,40 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
 
-  for (int k0 = 0; k0 < d.K; k0 += BK) {
-    stage<A_KS>(lds_a, A, d.lda, m0, k0, d.M, d.K, tid);
-    stage<B_KS>(lds_b, B, d.ldb, n0, k0, d.N, d.K, tid);
-    __syncthreads();
+  // double buffered: the global loads of stage s+1 are in flight while stage s is multiplied
+  const int KT = (d.K + BK - 1) / BK;
+  double pa[4], pb[4];
+  if (KT > 0) {
+    fetch<A_KS>(pa, A, d.lda, m0, 0, d.M, d.K, tid);
+    fetch<B_KS>(pb, B, d.ldb, n0, 0, d.N, d.K, tid);
+    put<A_KS>(lds_a[0], pa, tid);
+    put<B_KS>(lds_b[0], pb, tid);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const double* sa = lds_a[kt & 1];
+    const double* sb = lds_b[kt & 1];
+    const bool more = kt + 1 < KT;
+    if (more) {
+      fetch<A_KS>(pa, A, d.lda, m0, (kt + 1) * BK, d.M, d.K, tid);
+      fetch<B_KS>(pb, B, d.ldb, n0, (kt + 1) * BK, d.N, d.K, tid);
+    }
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       const int k = ks * 4 + (lane >> 4);
       double af[2], bfv[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) af[i] = lds_a[k * BT + wm * 32 + i * 16 + (lane & 15)];
+      for (int i = 0; i < 2; ++i) af[i] = sa[k * BT + wm * 32 + i * 16 + (lane & 15)];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) bfv[j] = lds_b[k * BT + wn * 32 + j * 16 + (lane & 15)];
+      for (int j = 0; j < 2; ++j) bfv[j] = sb[k * BT + wn * 32 + j * 16 + (lane & 15)];
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      put<A_KS>(lds_a[(kt + 1) & 1], pa, tid);
+      put<B_KS>(lds_b[(kt + 1) & 1], pb, tid);
     }
     __syncthreads();
   }
