@@ -1,0 +1,161 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares, and the
+host-side mirror of the reference's optimizer interface validates and dispatches like the reference
+(reference dion/muon.py:55-131, dion/dion.py:105-231).  No GPU compute is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "dion_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dion_amd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dion_amd import _lib
+
+    names = _declared_functions()
+    assert len(names) >= 14
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/dion_amd.h but not exported"
+    # and the ctypes binding covers them all
+    assert set(names) == set(_lib.exported_symbols())
+    lib2 = _lib.load()
+    assert lib2.dion_amd_version().startswith(b"dion_amd")
+
+
+def test_workspace_queries_and_argument_errors_without_gpu():
+    from dion_amd import _lib
+
+    lib = _lib.load()
+    per = lib.dion_amd_ns_workspace_bytes(1, 768, 3072, _lib.BF16)
+    assert per >= 2 * 768 * 3072 * 2 + 2 * 768 * 768 * 2
+    assert lib.dion_amd_ns_workspace_bytes(48, 768, 768, _lib.BF16) >= 48 * 4 * 768 * 768 * 2
+    assert lib.dion_amd_ns_workspace_bytes(0, 768, 768, _lib.BF16) == 0
+    assert lib.dion_amd_muon_workspace_bytes(96, 4096, 14336) <= (4 << 30) + (1 << 20)  # chunked to ~4 GiB
+    assert lib.dion_amd_dion_workspace_bytes(24, 3072, 768, 192, _lib.BF16) > 0
+    # argument validation happens before anything is launched
+    coeffs = _lib.float_array([1.0, 1.0, 1.0])
+    assert lib.dion_amd_newton_schulz(None, 0, 0, 8, None, 0, 8, 1, 8, 8, coeffs, 1, 1e-7, 0, 1, None, 0, None) == -1
+    assert lib.dion_amd_profile_read(99, None, None, None) == -1
+    with pytest.raises(_lib.DionAmdError):
+        _lib.check(-2, "x")
+    with pytest.raises(_lib.DionAmdError):
+        _lib.dtype_code(torch.float16)
+
+
+def test_no_cpu_fallback():
+    from dion_amd import Dion, Muon, _lib, zeropower_via_newtonschulz5
+
+    with pytest.raises(_lib.DionAmdError):
+        zeropower_via_newtonschulz5(torch.randn(16, 32))
+    p = torch.nn.Parameter(torch.randn(16, 8))
+    p.grad = torch.randn(16, 8)
+    with pytest.raises(_lib.DionAmdError):
+        Muon([p]).step()
+    with pytest.raises(_lib.DionAmdError):
+        Dion([p]).step()
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "dion_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_muon_constructor_contract():
+    from dion_amd import Muon
+
+    p = [torch.nn.Parameter(torch.randn(8, 8))]
+    opt = Muon(p)
+    assert opt.defaults == dict(lr=0.01, mu=0.95, beta1=0.9, beta2=0.95, weight_decay=0.01, algorithm="muon", step=0,
+                                epsilon=1e-8, nesterov=False, flatten=False, adjust_lr="spectral_norm")
+    for kw in (dict(lr=-1.0), dict(mu=-0.1), dict(betas=(0.9,)), dict(betas=(-0.1, 0.9)), dict(adjust_lr="bogus")):
+        with pytest.raises(ValueError):
+            Muon(p, **kw)
+    with pytest.raises(TypeError):
+        Muon(p, newton_schulz_func=3)
+    with pytest.raises(NotImplementedError):
+        Muon(p, distributed_mesh=object())
+    Muon(p, use_triton=True, adjust_lr=None)  # accepted
+    bad = Muon([dict(params=p, algorithm="sgd")])
+    with pytest.raises(ValueError, match="Unknown algorithm"):
+        bad.step()
+    assert bad.param_groups[0]["step"] == 1
+    vec = Muon([torch.nn.Parameter(torch.randn(8))])
+    vec.param_groups[0]["params"][0].grad = torch.zeros(8)
+    with pytest.raises(AssertionError):
+        vec.step()
+    # parameters without gradients are skipped, element-wise groups work on any device
+    w = torch.nn.Parameter(torch.randn(4, 4))
+    e = torch.nn.Parameter(torch.ones(5))
+    e.grad = torch.ones(5)
+    opt = Muon([dict(params=[w]), dict(params=[e], algorithm="adamw", lr=0.1, weight_decay=0.0)])
+    opt.step()
+    assert torch.allclose(e.detach(), torch.full((5,), 0.9), atol=1e-6)
+    assert w not in opt.state and set(opt.state[e]) == {"momentum", "variance"}
+
+
+def test_dion_constructor_contract():
+    from dion_amd import Dion, DionMixedPrecisionConfig
+
+    p = [torch.nn.Parameter(torch.randn(8, 8))]
+    opt = Dion(p)
+    assert opt.defaults == dict(rank_fraction=1.0, rank_multiple_of=1, lr=0.01, mu=0.95, beta1=0.9, beta2=0.95,
+                                weight_decay=0.01, epsilon=1e-8, oversample=1.25, algorithm="dion", step=0)
+    for kw in (dict(lr=-1.0), dict(mu=-1.0), dict(betas=(1.0,)), dict(weight_decay=-1.0), dict(rank_fraction=0.0),
+               dict(rank_fraction=1.5), dict(rank_multiple_of=0), dict(power_iters=2), dict(qr_method="qr")):
+        with pytest.raises(ValueError):
+            Dion(p, **kw)
+    for kw in ("replicate_mesh", "outer_shard_mesh", "inner_shard_mesh"):
+        with pytest.raises(NotImplementedError):
+            Dion(p, **{kw: object()})
+    cfg = DionMixedPrecisionConfig(momentum_dtype=torch.bfloat16, Q_dtype=torch.float32, variance_dtype=torch.bfloat16)
+    opt = Dion([dict(params=p, rank_fraction=0.5, rank_multiple_of=3)], mixed_precision_config=cfg)
+    st = opt._get_or_initialize_state(p[0], opt.param_groups[0])
+    assert st["momentum"].dtype == torch.bfloat16 and st["Q"].dtype == torch.float32
+    assert st["Q"].shape == (8, 6)                       # 3 * ceil(0.5 * 8 / 3) = 6
+    wide = torch.nn.Parameter(torch.randn(4, 16))
+    st = opt._get_or_initialize_state(wide, dict(algorithm="dion", rank_fraction=1.0, rank_multiple_of=1))
+    assert st["Q"].shape == (4, 4)                       # m < n: Q is (m, r)
+    with pytest.raises(ValueError):
+        opt._get_or_initialize_state(torch.nn.Parameter(torch.randn(4)), dict(algorithm="dion", rank_fraction=1.0,
+                                                                               rank_multiple_of=1))
+    a = torch.nn.Parameter(torch.ones(3))
+    st = opt._get_or_initialize_state(a, dict(algorithm="adamw"))
+    assert st["variance"].dtype == torch.bfloat16
+    opt.synchronize_for_checkpoint()                     # no-op on one GPU
+    bad = Dion([dict(params=p, algorithm="nope")])
+    with pytest.raises(ValueError, match="Unknown algorithm"):
+        bad.step()
+
+
+def test_elementwise_groups_match_closed_forms():
+    """Lion / AdamW element-wise rules (reference dion/scalar_opts.py:89-187) against their textbook forms."""
+    from dion_amd.elementwise_opts import adamw_update_foreach, lion_update_foreach
+
+    torch.manual_seed(0)
+    x, g = torch.randn(50, dtype=torch.float64), torch.randn(50, dtype=torch.float64)
+    m, v = torch.randn(50, dtype=torch.float64) * 0.1, torch.rand(50, dtype=torch.float64) * 0.1
+    lr, b1, b2, wd, eps, step = 0.01, 0.9, 0.95, 0.1, 1e-8, 3
+    m1 = b1 * m + (1 - b1) * g
+    v1 = b2 * v + (1 - b2) * g * g
+    want = x * (1 - lr * wd) - lr * (m1 / (1 - b1**step)) / ((v1 / (1 - b2**step)).sqrt() + eps)
+    X, M, V = [x.clone()], [m.clone()], [v.clone()]
+    t = lambda z: torch.tensor(z, dtype=torch.float64)  # noqa: E731
+    adamw_update_foreach(X, [g], M, V, t(lr), t(b1), t(b2), t(wd), t(step), t(eps))
+    assert torch.allclose(X[0], want, rtol=1e-9) and torch.allclose(M[0], m1) and torch.allclose(V[0], v1)
+    want = x * (1 - lr * wd) - lr * torch.sign(b1 * m + (1 - b1) * g)
+    X, M = [x.clone()], [m.clone()]
+    lion_update_foreach(X, [g], M, t(lr), t(b1), t(b2), t(wd))
+    assert torch.allclose(X[0], want, rtol=1e-12) and torch.allclose(M[0], b2 * m + (1 - b2) * g)
