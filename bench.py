@@ -205,6 +205,8 @@ def main():
     ap.add_argument("--workload", default="muon_gpt_small", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run three plain 512 MiB device copies (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); run with --gpus 1",
@@ -217,6 +219,13 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        src = torch.ones(512 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     wl = WORKLOADS[args.workload]
     res = measure(wl, dev, args.steps, args.warmup)
     main_sum = summarize(args.workload, wl, res)
