@@ -459,7 +459,8 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     // ---- Q_new = column-normalised R   (reference dion/dion.py:856, 875, 1460-1491, 1533-1561)
     {
       DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
-      rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, eps, cb, s);
+      // the orthonormaliser is done with its fp64 scratch: reuse its head for the column sums
+      rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, eps, cb, reinterpret_cast<double*>(orth_ws), s);
       if (rc) return rc;
     }
     // ---- X <- (1 - lr wd) X - scaled_lr P Q_new^T  (or Q_new P^T)   (reference dion/dion.py:865-872)

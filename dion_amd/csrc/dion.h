@@ -9,8 +9,9 @@ int da_add_grad(const DaPtrTable& m, const DaPtrTable& g, int m_dtype, int g_dty
                 int* nonzero, hipStream_t s);
 int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, long long n, int batch, hipStream_t s);
 int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const int* nonzero, hipStream_t s);
+// `sums` is scratch for batch * r doubles.
 int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, float eps,
-               int batch, hipStream_t s);
+               int batch, double* sums, hipStream_t s);
 
 // CholeskyQR (passes = 1) / CholeskyQR2 (passes = 2) of `batch` contiguous matrices P[b]
 // (rows x r, dtype bf16 or f32) with fp64 Gram, Cholesky and triangular solve; result in

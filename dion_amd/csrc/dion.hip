@@ -111,40 +111,58 @@ __global__ __launch_bounds__(256) void fix_kernel(T* V, const T* alt, long long 
 
 // Column normalisation of R[b] (rows x r, TM): Qn = R / (sqrt(sum_rows R^2) + eps), computed in
 // fp32 (column sums accumulated in fp64), stored as TM into qn[b] and, cast to TQ, into the
-// optimizer's Q state.  One workgroup per 64 columns: 4 row groups x 64 columns.
-template <typename TM, typename TQ>
-__global__ __launch_bounds__(256) void colnorm_kernel(const TM* __restrict__ R, TM* __restrict__ qn, DaPtrTable qt,
-                                                      int rows, int r, float eps) {
+// optimizer's Q state.  Two launches: partial column sums over row slices (fp64 atomics into a
+// zeroed buffer), then a fully parallel normalise pass.
+template <typename TM>
+__global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, double* __restrict__ sums, int rows, int r,
+                                                     int rows_per_slice) {
   __shared__ double part[4][64];
-  __shared__ float denom[64];
-  const int b = blockIdx.y;
+  const int b = blockIdx.z;
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int g = threadIdx.x >> 6;
   const TM* Rb = R + (long long)b * rows * r;
+  const int i0 = blockIdx.y * rows_per_slice;
+  const int i1 = i0 + rows_per_slice < rows ? i0 + rows_per_slice : rows;
   double s = 0.0;
   if (c < r)
-    for (int i = g; i < rows; i += 4) {
+    for (int i = i0 + g; i < i1; i += 4) {
       const float v = ld_as_float<TM>(Rb + (long long)i * r + c);
       s += (double)v * (double)v;
     }
   part[g][threadIdx.x & 63] = s;
   __syncthreads();
-  if (g == 0) {
+  if (g == 0 && c < r) {
     const double t = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-    denom[threadIdx.x] = sqrtf((float)t) + eps;
+    atomicAdd(sums + (long long)b * r + c, t);
   }
-  __syncthreads();
-  if (c < r) {
-    const float d = denom[threadIdx.x & 63];
-    TM* Qn = qn + (long long)b * rows * r;
-    TQ* Q = static_cast<TQ*>(qt.p[b]);
-    for (int i = g; i < rows; i += 4) {
-      const long long o = (long long)i * r + c;
-      const float v = ld_as_float<TM>(Rb + o) / d;
-      st_from_float<TM>(Qn + o, v);
-      st_from_float<TQ>(Q + o, ld_as_float<TM>(Qn + o));
+}
+
+template <typename TM, typename TQ>
+__global__ __launch_bounds__(256) void colscale_kernel(const TM* __restrict__ R, TM* __restrict__ qn, DaPtrTable qt,
+                                                       const double* __restrict__ sums, long long n, int r, float eps) {
+  const int b = blockIdx.y;
+  const TM* Rb = R + (long long)b * n;
+  TM* Qn = qn + (long long)b * n;
+  TQ* Q = static_cast<TQ*>(qt.p[b]);
+  const double* sb = sums + (long long)b * r;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
+    const int c0 = (int)(i % r);  // r is a multiple of 8: the 8 elements stay in one row
+    float v[8], q[8];
+    V8<TM>::load(Rb + i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float d = sqrtf((float)sb[c0 + e]) + eps;
+      v[e] = V8<TM>::round(v[e] / d);     // cast back to R's dtype (reference dion/dion.py:1490)
+      q[e] = v[e];
     }
+    V8<TM>::store(Qn + i, v);
+    V8<TQ>::store(Q + i, q);              // Q <- Q_new.to(Q.dtype) (reference dion/dion.py:1559-1561)
   }
+}
+
+__global__ void fill_f64_kernel(double* p, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.0;
 }
 
 inline unsigned ew_blocks(long long n) {
@@ -211,16 +229,30 @@ int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const in
 }
 
 int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, float eps,
-               int batch, hipStream_t s) {
-  dim3 grid((r + 63) / 64, batch);
+               int batch, double* sums, hipStream_t s) {
+  if (r & 7) return DA_ERR_ALIGN;
+  const long long ns = (long long)batch * r;
+  hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, sums, ns);
+  int slices = (rows + 255) / 256;
+  if (slices > 64) slices = 64;
+  const int rps = (rows + slices - 1) / slices;
+  dim3 g1((r + 63) / 64, slices, batch);
+  if (m_dtype == DA_BF16)
+    hipLaunchKernelGGL(colsum_kernel<bf16_t>, g1, dim3(256), 0, s, static_cast<const bf16_t*>(R), sums, rows, r, rps);
+  else if (m_dtype == DA_F32)
+    hipLaunchKernelGGL(colsum_kernel<float>, g1, dim3(256), 0, s, static_cast<const float*>(R), sums, rows, r, rps);
+  else
+    return DA_ERR_DTYPE;
+  const long long n = (long long)rows * r;
+  dim3 g2(ew_blocks(n), batch);
   if (m_dtype == DA_BF16 && q_dtype == DA_BF16)
-    hipLaunchKernelGGL((colnorm_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, rows, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<bf16_t, bf16_t>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, eps);
   else if (m_dtype == DA_BF16 && q_dtype == DA_F32)
-    hipLaunchKernelGGL((colnorm_kernel<bf16_t, float>), grid, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, rows, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<bf16_t, float>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, eps);
   else if (m_dtype == DA_F32 && q_dtype == DA_BF16)
-    hipLaunchKernelGGL((colnorm_kernel<float, bf16_t>), grid, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, rows, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<float, bf16_t>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, eps);
   else if (m_dtype == DA_F32 && q_dtype == DA_F32)
-    hipLaunchKernelGGL((colnorm_kernel<float, float>), grid, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, rows, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<float, float>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, eps);
   else
     return DA_ERR_DTYPE;
   return da_launch_status();
@@ -261,6 +293,19 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     g.lda = r; g.ldb = r; g.ldc = r;
     g.M = r; g.N = r; g.K = rows;
     g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
+    {
+      // few output tiles, long K: slice K until ~512 workgroups exist
+      const int t = (r + 63) / 64;
+      const long long blocks = (long long)t * (t + 1) / 2 * batch;
+      int split = (int)((512 + blocks - 1) / blocks);
+      const int max_split = rows / 256 > 0 ? rows / 256 : 1;
+      if (split > max_split) split = max_split;
+      g.split_k = split;
+      if (split > 1) {
+        rc = da_fill_f64(G, rr * batch, 0.0, s);
+        if (rc) return rc;
+      }
+    }
     rc = da_gemm_f64(g, s);
     if (rc) return rc;
     // blocked lower Cholesky G = L L^T

@@ -14,9 +14,12 @@ struct Gemm64Desc {
   int M, N, K, batch;
   int a_kstrided, b_kstrided, symmetric;
   double alpha, beta;
+  int split_k;   // > 1: K is cut into that many slices whose partial products are added atomically into a
+                 // zeroed C (no E term); the summation order, and so the last bits, vary run to run
 };
 
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
+int da_fill_f64(double* p, long long n, double v, hipStream_t s);
 
 // dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.
 int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s);

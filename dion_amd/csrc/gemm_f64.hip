@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
   const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  const int split = blockIdx.y;  // split-K slice
   const int b = blockIdx.x / per_batch;
   int t = blockIdx.x - b * per_batch;
   int ti, tj;
@@ -80,11 +81,14 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
     for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
 
   // double buffered: the global loads of stage s+1 are in flight while stage s is multiplied
-  const int KT = (d.K + BK - 1) / BK;
+  const int KT_all = (d.K + BK - 1) / BK;
+  const int per_split = (KT_all + (int)gridDim.y - 1) / (int)gridDim.y;
+  const int kt0 = split * per_split;
+  const int KT = KT_all - kt0 < per_split ? KT_all - kt0 : per_split;   // may be <= 0 for the last slices
   double pa[4], pb[4];
   if (KT > 0) {
-    fetch<A_KS>(pa, A, d.lda, m0, 0, d.M, d.K, tid);
-    fetch<B_KS>(pb, B, d.ldb, n0, 0, d.N, d.K, tid);
+    fetch<A_KS>(pa, A, d.lda, m0, kt0 * BK, d.M, d.K, tid);
+    fetch<B_KS>(pb, B, d.ldb, n0, kt0 * BK, d.N, d.K, tid);
     put<A_KS>(lds_a[0], pa, tid);
     put<B_KS>(lds_b[0], pb, tid);
   }
@@ -94,8 +98,8 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
     const double* sb = lds_b[kt & 1];
     const bool more = kt + 1 < KT;
     if (more) {
-      fetch<A_KS>(pa, A, d.lda, m0, (kt + 1) * BK, d.M, d.K, tid);
-      fetch<B_KS>(pb, B, d.ldb, n0, (kt + 1) * BK, d.N, d.K, tid);
+      fetch<A_KS>(pa, A, d.lda, m0, (kt0 + kt + 1) * BK, d.M, d.K, tid);
+      fetch<B_KS>(pb, B, d.ldb, n0, (kt0 + kt + 1) * BK, d.N, d.K, tid);
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
@@ -131,9 +135,14 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
         const int n = n0 + wn * 32 + j * 16 + (lane & 15);
         if (m < d.M && n < d.N) {
           double o = d.alpha * acc[i][j][v];
-          if (E) o += d.beta * E[(long long)m * d.lde + n];
-          C[(long long)m * d.ldc + n] = o;
-          if (mirror) C[(long long)n * d.ldc + m] = o;
+          if (gridDim.y > 1) {  // split-K: partial sums meet in a zeroed C
+            atomicAdd(C + (long long)m * d.ldc + n, o);
+            if (mirror) atomicAdd(C + (long long)n * d.ldc + m, o);
+          } else {
+            if (E) o += d.beta * E[(long long)m * d.lde + n];
+            C[(long long)m * d.ldc + n] = o;
+            if (mirror) C[(long long)n * d.ldc + m] = o;
+          }
         }
       }
 }
@@ -144,7 +153,9 @@ int launch(const Gemm64Desc& d, hipStream_t s) {
   const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
   const long long blocks = per_batch * d.batch;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
-  hipLaunchKernelGGL((gemm_f64_kernel<A_KS, B_KS, SYM>), dim3((unsigned)blocks), dim3(256), 0, s, d);
+  int split = d.split_k > 1 ? d.split_k : 1;
+  if (d.E) split = 1;
+  hipLaunchKernelGGL((gemm_f64_kernel<A_KS, B_KS, SYM>), dim3((unsigned)blocks, split), dim3(256), 0, s, d);
   return da_launch_status();
 }
 
@@ -160,6 +171,11 @@ __global__ __launch_bounds__(256) void cvt_from_f64_kernel(const double* __restr
                                                            long long n) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
     st_from_float<T>(dst + i, (float)src[i]);
+}
+
+__global__ void fill_f64_kernel(double* p, long long n, double v) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
 }
 
 inline unsigned cvt_blocks(long long n) {
@@ -179,6 +195,12 @@ int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) {
   if (!d.a_kstrided && d.b_kstrided) return launch<false, true, false>(d, s);
   if (d.a_kstrided && !d.b_kstrided) return launch<true, false, false>(d, s);
   return launch<true, true, false>(d, s);
+}
+
+int da_fill_f64(double* p, long long n, double v, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
+  return da_launch_status();
 }
 
 int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) {
