@@ -351,6 +351,19 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
     _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
         fb[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
   } while (0)
+#define DA_FREAD2(st, ks, FA, FB)                                                                  \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        FA[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
+    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
+        FB[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+  } while (0)
+#define DA_MMA2(FA, FB)                                                                            \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[j], FA[i], acc[i][j], 0, 0, 0); \
+  } while (0)
 #define DA_MMA()                                                                                   \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
@@ -371,17 +384,36 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
   } while (0)
     DA_DMA(lds);
     __syncthreads();
+    // Fragments are double buffered in registers: the ds_reads of k-step s+1 are issued before
+    // the MFMAs of k-step s (scheduling fences keep the compiler from sinking them back down to
+    // their first use), and the stage barrier sits before the last k-step so that the first
+    // fragments of the next stage are fetched under the last MFMAs of this one.
+    bf16x8_t ga[TMI], gb[TNJ];
+    DA_FREAD(lds, 0);
     for (int kt = 0; kt < KT; ++kt) {
       char* cur = lds + (kt & 1) * STAGE;
       char* nxt = lds + ((kt + 1) & 1) * STAGE;
-      if (kt + 1 < KT) DA_DMA(nxt);
-#pragma unroll
-      for (int ks = 0; ks < BK / 16; ++ks) {
-        DA_FREAD(cur, ks);
-        DA_MMA();
-      }
+      const bool more = kt + 1 < KT;
+      if (more) DA_DMA(nxt);
+      DA_FREAD2(cur, 1, ga, gb);
+      __builtin_amdgcn_sched_barrier(0);
+      DA_MMA();
+      __builtin_amdgcn_sched_barrier(0);
+      DA_FREAD(cur, 2);
+      __builtin_amdgcn_sched_barrier(0);
+      DA_MMA2(ga, gb);
+      __builtin_amdgcn_sched_barrier(0);
+      DA_FREAD2(cur, 3, ga, gb);
+      __builtin_amdgcn_sched_barrier(0);
+      DA_MMA();
+      __builtin_amdgcn_sched_barrier(0);
       __syncthreads();
+      if (more) DA_FREAD(nxt, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      DA_MMA2(ga, gb);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    __syncthreads();
 #undef DA_DMA
   } else {
     u32x4_t ra[NCH], rb[NCH];
@@ -434,6 +466,8 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
   }
 #undef DA_FREAD
 #undef DA_MMA
+#undef DA_FREAD2
+#undef DA_MMA2
   epilogue<C, SYM>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
 }
 
