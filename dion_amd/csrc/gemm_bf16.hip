@@ -62,12 +62,15 @@ __device__ __forceinline__ int ks_swizzle(int chunk, int krow) { return (((chunk
 //   and goes to LDS byte offset `l + i * lstep`.
 //   Direct-to-LDS path: wave-instruction i of wavefront w fills the 1024-byte LDS block
 //   (i * NW + w); lane p of it fetches the chunk whose *physical* position is p, i.e. the
-//   swizzle is applied to the global address (`gd + i * gdstep`).
+//   swizzle is applied to the global address, which is kept as a wave-uniform base pointer
+//   (`dbase`) plus a 32-bit byte offset (`doff + i * dstep`, per lane and loop invariant, plus
+//   the stage's offset, a scalar) so that the loads use SGPR-base addressing.
 template <typename C, bool KS>
 struct StageAddr {
   const bf16_t* g;
-  const bf16_t* gd;
-  long long gstep, gdstep, tstep;   // per chunk (register / direct) and per stage, in elements
+  const char* dbase;
+  unsigned doff, dstep;
+  long long gstep, tstep;   // per chunk and per stage, in elements
   int l, lstep;
   int row, col;             // first chunk's (row within tile, k offset) resp. (k row, row offset)
   __device__ __forceinline__ StageAddr(const bf16_t* base, int ld, int row0, int tid) {
@@ -82,8 +85,9 @@ struct StageAddr {
       l = row * 128 + kc_swizzle(tid & 7, row) * 16;
       lstep = (C::NT / 8) * 128;   // NT/8 is a multiple of 16: the swizzle term is the same for all chunks
       const int drow = wave * 8 + (lane >> 3);             // block (0 * NW + wave), 8 rows per block
-      gd = base + (long long)(row0 + drow) * ld + kc_swizzle(lane & 7, drow) * 8;
-      gdstep = (long long)(NW * 8) * ld;                   // NW * 8 is a multiple of 16
+      dbase = reinterpret_cast<const char*>(base + (long long)row0 * ld);
+      doff = (unsigned)(drow * ld + kc_swizzle(lane & 7, drow) * 8) * 2u;
+      dstep = (unsigned)(NW * 8 * ld) * 2u;                // NW * 8 is a multiple of 16
     } else {
       constexpr int CPR = C::BT / 8;                       // chunks per k-row
       constexpr int RPB = 64 / CPR;                        // k-rows per 1024-byte block
@@ -95,8 +99,9 @@ struct StageAddr {
       l = row * (C::BT * 2) + ks_swizzle(tid % CPR, row) * 16;
       lstep = (C::NT / CPR) * (C::BT * 2);                 // NT / CPR = 16: swizzle term unchanged
       const int drow = wave * RPB + lane / CPR;
-      gd = base + (long long)drow * ld + row0 + ks_swizzle(lane % CPR, drow) * 8;
-      gdstep = (long long)(NW * RPB) * ld;                 // NW * RPB = 16
+      dbase = reinterpret_cast<const char*>(base + row0);
+      doff = (unsigned)(drow * ld + ks_swizzle(lane % CPR, drow) * 8) * 2u;
+      dstep = (unsigned)(NW * RPB * ld) * 2u;              // NW * RPB = 16
     }
   }
 };
@@ -212,6 +217,29 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
   const char* const Ebase = !has_e ? nullptr
                             : d.Etab ? static_cast<const char*>(d.Etab[b])
                                      : static_cast<const char*>(d.E) + (long long)b * d.sE * csz;
+  constexpr int NPASS = 32 / RPP;
+  // E for one band is fetched up front (its latency overlaps the LDS staging of the accumulators)
+  // and the next band's E is requested before the current band is finished.
+  uint4 ev[NPASS][2];
+  auto load_e = [&](int band) {
+    const int band_m = wm0 + band * 32;
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+      const int m = band_m + pass * RPP + lane / CPR, n = wn0 + (lane % CPR) * 8;
+      ev[pass][0] = make_uint4(0u, 0u, 0u, 0u);
+      ev[pass][1] = make_uint4(0u, 0u, 0u, 0u);
+      if (has_e && m < d.M && n < d.N) {
+        if (ep.c_f32) {
+          const float* Ep = reinterpret_cast<const float*>(Ebase) + (long long)m * d.lde + n;
+          ev[pass][0] = *reinterpret_cast<const uint4*>(Ep);
+          ev[pass][1] = *reinterpret_cast<const uint4*>(Ep + 4);
+        } else {
+          ev[pass][0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(Ebase) + (long long)m * d.lde + n);
+        }
+      }
+    }
+  };
+  if (has_e) load_e(0);
 #pragma unroll
   for (int i = 0; i < C::TMI; ++i) {
     {
@@ -225,7 +253,12 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
     }
     __syncthreads();
     const int band_m = wm0 + i * 32;
-    for (int pass = 0; pass < 32 / RPP; ++pass) {
+    uint4 ec[NPASS][2];
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) { ec[pass][0] = ev[pass][0]; ec[pass][1] = ev[pass][1]; }
+    if (has_e && i + 1 < C::TMI) load_e(i + 1);
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
       const int r = pass * RPP + lane / CPR;
       const int c8 = (lane % CPR) * 8;
       const int m = band_m + r, n = wn0 + c8;
@@ -234,29 +267,24 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
         const float4 a0 = *reinterpret_cast<const float4*>(sp);
         const float4 a1 = *reinterpret_cast<const float4*>(sp + 4);
         float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        float e[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float e[8];
         const long long off = (long long)m * d.ldc + n;
         if (ep.c_f32) {
-          if (has_e) {
-            const float* Ep = reinterpret_cast<const float*>(Ebase) + (long long)m * d.lde + n;
-            const float4 e0 = *reinterpret_cast<const float4*>(Ep);
-            const float4 e1 = *reinterpret_cast<const float4*>(Ep + 4);
-            e[0] = e0.x; e[1] = e0.y; e[2] = e0.z; e[3] = e0.w; e[4] = e1.x; e[5] = e1.y; e[6] = e1.z; e[7] = e1.w;
-          }
+          const uint32_t w[8] = {ec[pass][0].x, ec[pass][0].y, ec[pass][0].z, ec[pass][0].w,
+                                 ec[pass][1].x, ec[pass][1].y, ec[pass][1].z, ec[pass][1].w};
+#pragma unroll
+          for (int q = 0; q < 8; ++q) e[q] = __builtin_bit_cast(float, w[q]);
 #pragma unroll
           for (int q = 0; q < 8; ++q) v[q] = epi_value(ep, v[q], e[q]);
           float* Cp = reinterpret_cast<float*>(Cbase) + off;
           *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
           *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
         } else {
-          if (has_e) {
-            const uint4 ev = *reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(Ebase) + (long long)m * d.lde + n);
-            const uint32_t w[4] = {ev.x, ev.y, ev.z, ev.w};
+          const uint32_t w[4] = {ec[pass][0].x, ec[pass][0].y, ec[pass][0].z, ec[pass][0].w};
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              e[2 * q] = bf2f((bf16_t)(w[q] & 0xffffu));
-              e[2 * q + 1] = bf2f((bf16_t)(w[q] >> 16));
-            }
+          for (int q = 0; q < 4; ++q) {
+            e[2 * q] = bf2f((bf16_t)(w[q] & 0xffffu));
+            e[2 * q + 1] = bf2f((bf16_t)(w[q] >> 16));
           }
           uint32_t pk[4];
 #pragma unroll
@@ -376,12 +404,13 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
 #define DA_DMA(st)                                                                                 \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sa.gd + i * sa.gdstep, (st) + (i * NW + wave) * 1024);                               \
+        dma16(sa.dbase + (unsigned)(sa.doff + i * sa.dstep + koff_a), (st) + (i * NW + wave) * 1024); \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sb.gd + i * sb.gdstep, (st) + A_BYTES + (i * NW + wave) * 1024);                     \
-    sa.gd += sa.tstep;                                                                             \
-    sb.gd += sb.tstep;                                                                             \
+        dma16(sb.dbase + (unsigned)(sb.doff + i * sb.dstep + koff_b), (st) + A_BYTES + (i * NW + wave) * 1024); \
+    koff_a += (unsigned)(sa.tstep * 2);                                                            \
+    koff_b += (unsigned)(sb.tstep * 2);                                                            \
   } while (0)
+    unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB)
     DA_DMA(lds);
     __syncthreads();
     // Fragments are double buffered in registers: the ds_reads of k-step s+1 are issued before
