@@ -134,10 +134,28 @@ __device__ __forceinline__ bf16x8_t read_frag(const char* lds, int r0, int ks, i
 
 __device__ __forceinline__ int wave_uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// 16 bytes per lane from global memory straight into LDS: lane p's data lands at l + 16 p
-// (l must be wave-uniform).
-__device__ __forceinline__ void dma16(const void* g, char* l) {
-  __builtin_amdgcn_global_load_lds(g, DA_LDS_PTR(void, l), 16, 0, 0);
+// 16 bytes per lane from global memory straight into LDS: lane p's data lands at LDS byte
+// address `l + 16 p`.  `base` and `l` are wave-uniform, `off` is the lane's byte offset.
+// Written as assembly on purpose: with the compiler's own LDS-DMA intrinsic in the loop, its
+// wait-count insertion degrades every LDS-read wait to lgkmcnt(0), which serialises the
+// fragment reads of k-step s+1 with the MFMAs of k-step s.  The price is that the compiler
+// does not know about these loads: dma_wait() must precede the barrier that publishes a stage.
+// The s_nop covers the M0-write -> LDS-DMA and the VALU-SGPR-write -> VMEM-address hazards,
+// which the hazard recogniser cannot see inside an asm block.
+// (M0 is not in the clobber list -- the compiler rejects reserved registers there; nothing else
+// in this kernel keeps a value in M0.)
+__device__ __forceinline__ void dma16(const char* base, unsigned off, unsigned l) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+  const unsigned long long u = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(a >> 32)) << 32) |
+                               (unsigned)__builtin_amdgcn_readfirstlane((int)a);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(off), "s"(u), "s"(__builtin_amdgcn_readfirstlane((int)l))
+               : "memory");
+}
+__device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ unsigned lds_addr(const char* p) {
+  return (unsigned)(uintptr_t)DA_LDS_PTR(const char, p);
 }
 
 struct Epi {
@@ -404,14 +422,15 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
 #define DA_DMA(st)                                                                                 \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sa.dbase + (unsigned)(sa.doff + i * sa.dstep + koff_a), (st) + (i * NW + wave) * 1024); \
+        dma16(sa.dbase, sa.doff + i * sa.dstep + koff_a, lds_addr(st) + (i * NW + wave) * 1024);   \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sb.dbase + (unsigned)(sb.doff + i * sb.dstep + koff_b), (st) + A_BYTES + (i * NW + wave) * 1024); \
+        dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
     koff_a += (unsigned)(sa.tstep * 2);                                                            \
     koff_b += (unsigned)(sb.tstep * 2);                                                            \
   } while (0)
     unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB)
     DA_DMA(lds);
+    dma_wait();
     __syncthreads();
     // Fragments are double buffered in registers: the ds_reads of k-step s+1 are issued before
     // the MFMAs of k-step s (scheduling fences keep the compiler from sinking them back down to
@@ -436,6 +455,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
       __builtin_amdgcn_sched_barrier(0);
       DA_MMA();
       __builtin_amdgcn_sched_barrier(0);
+      dma_wait();
       __syncthreads();
       if (more) DA_FREAD(nxt, 0);
       __builtin_amdgcn_sched_barrier(0);
