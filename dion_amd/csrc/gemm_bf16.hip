@@ -158,25 +158,26 @@ __device__ __forceinline__ unsigned lds_addr(const char* p) {
   return (unsigned)(uintptr_t)DA_LDS_PTR(const char, p);
 }
 
-struct Epi {
-  float s0, s1;
-  int mode, faithful, c_f32;
-};
-
-// value of C from the accumulator and (optionally) the epilogue operand
-__device__ __forceinline__ float epi_value(const Epi& ep, float acc, float e) {
-  if (ep.faithful) {
+// value of C from the accumulator and (optionally) the epilogue operand; the final rounding to
+// C's dtype happens at the store
+template <bool HAS_E, bool FAITHFUL, bool CF32>
+__device__ __forceinline__ float epi_value(float s0, float s1, float acc, float e) {
+  if (FAITHFUL) {
     float t = rbf(acc);
-    t = rbf(ep.s1 * t);
-    if (ep.mode == DA_EPI_AXPBY) {
-      float u = ep.s0 * e;
-      if (!ep.c_f32) u = rbf(u);
+    t = rbf(s1 * t);
+    if (HAS_E) {
+      float u = s0 * e;
+      if (!CF32) u = rbf(u);
       t = u + t;
     }
-    return t;  // final rounding to C's dtype happens at the store
+    return t;
   }
-  return ep.mode == DA_EPI_AXPBY ? ep.s0 * e + ep.s1 * acc : ep.s1 * acc;
+  return HAS_E ? s0 * e + s1 * acc : s1 * acc;
 }
+
+typedef __attribute__((address_space(1))) u32x4_t global_u32x4_t;
+__device__ __forceinline__ u32x4_t ldg16(const char* p) { return *(const global_u32x4_t*)p; }
+__device__ __forceinline__ void stg16(char* p, u32x4_t v) { *(global_u32x4_t*)p = v; }
 
 // Which output tile a workgroup owns.  Workgroups are dealt round-robin to the 8 XCDs (each
 // with its own L2), so consecutive *logical* tiles -- which share an operand panel -- are
@@ -215,49 +216,52 @@ __device__ __forceinline__ TileId decode_tile(const GemmDesc& d) {
 }
 
 // The accumulators go through LDS (the stage buffers are free by now), one 32-row band of the
-// wavefront's sub-tile at a time, so that C and E move as 16-byte row segments and the code
-// stays small enough to keep every accumulator index a compile-time constant.
-template <typename C, bool SYM>
-__device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
-                                         int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
+// wavefront's sub-tile at a time, so that C and E move as 16-byte row segments.  Each wavefront
+// stages through its own LDS region, so only wavefront-level ordering is needed inside.
+// Output dtype, epilogue form and rounding mode are compile-time here: evaluated per element at
+// run time they cost more than the MFMAs of a short-K product.
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL>
+__device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
+                                              bool mirror, int m0, int n0, int wave, int lane, int wm, int wn) {
   constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
   constexpr int PITCH = W + 4;       // floats; 16-byte aligned rows, conflict-free float4 writes
   constexpr int CPR = W / 8;         // 8-column chunks per row
   constexpr int RPP = 64 / CPR;      // rows per pass of the wavefront
-  float* stg = reinterpret_cast<float*>(lds) + wave * (32 * PITCH);
-  const Epi ep{d.s0, d.s1, d.epilogue, d.faithful, d.c_dtype == DA_F32};
-  const bool mirror = SYM && (ti != tj);
-  const bool has_e = d.epilogue == DA_EPI_AXPBY;
-  const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
-  // C and E base pointers of this matrix, as byte addresses (element size depends on c_dtype)
-  const int csz = ep.c_f32 ? 4 : 2;
-  char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * csz;
-  const char* const Ebase = !has_e ? nullptr
-                            : d.Etab ? static_cast<const char*>(d.Etab[b])
-                                     : static_cast<const char*>(d.E) + (long long)b * d.sE * csz;
   constexpr int NPASS = 32 / RPP;
+  constexpr int CSZ = CF32 ? 4 : 2;
+  constexpr int NV = CF32 ? 2 : 1;   // 16-byte vectors per 8 elements
+  float* stg = reinterpret_cast<float*>(lds) + wave * (32 * PITCH);
+  const float s0 = d.s0, s1 = d.s1;
+  const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
+  char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * CSZ;
+  const char* const Ebase = !HAS_E ? nullptr
+                            : d.Etab ? static_cast<const char*>(d.Etab[b])
+                                     : static_cast<const char*>(d.E) + (long long)b * d.sE * CSZ;
+  const int lr = lane / CPR, c8 = (lane % CPR) * 8;
+  const bool col_ok = FULL || wn0 + c8 < d.N;
   // E for one band is fetched up front (its latency overlaps the LDS staging of the accumulators)
   // and the next band's E is requested before the current band is finished.
-  uint4 ev[NPASS][2];
+  u32x4_t ev[NPASS][NV];
   auto load_e = [&](int band) {
-    const int band_m = wm0 + band * 32;
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
-      const int m = band_m + pass * RPP + lane / CPR, n = wn0 + (lane % CPR) * 8;
-      ev[pass][0] = make_uint4(0u, 0u, 0u, 0u);
-      ev[pass][1] = make_uint4(0u, 0u, 0u, 0u);
-      if (has_e && m < d.M && n < d.N) {
-        if (ep.c_f32) {
-          const float* Ep = reinterpret_cast<const float*>(Ebase) + (long long)m * d.lde + n;
-          ev[pass][0] = *reinterpret_cast<const uint4*>(Ep);
-          ev[pass][1] = *reinterpret_cast<const uint4*>(Ep + 4);
-        } else {
-          ev[pass][0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const bf16_t*>(Ebase) + (long long)m * d.lde + n);
-        }
+      const int m = wm0 + band * 32 + pass * RPP + lr;
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int h = 0; h < NV; ++h) ev[pass][h] = z;
+      if (col_ok && (FULL || m < d.M)) {
+        const char* Ep = Ebase + ((long long)m * d.lde + wn0 + c8) * CSZ;
+#pragma unroll
+        for (int h = 0; h < NV; ++h) ev[pass][h] = ldg16(Ep + 16 * h);
       }
     }
   };
-  if (has_e) load_e(0);
+  if (HAS_E) load_e(0);
 #pragma unroll
   for (int i = 0; i < C::TMI; ++i) {
     {
@@ -269,85 +273,114 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
           *reinterpret_cast<float4*>(row + j * 32 + vq * 8) =
               make_float4(acc[i][j][vq * 4], acc[i][j][vq * 4 + 1], acc[i][j][vq * 4 + 2], acc[i][j][vq * 4 + 3]);
     }
-    __syncthreads();
+    wave_sync_lds();
     const int band_m = wm0 + i * 32;
-    uint4 ec[NPASS][2];
+    u32x4_t ec[NPASS][NV];
+    if (HAS_E) {
 #pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) { ec[pass][0] = ev[pass][0]; ec[pass][1] = ev[pass][1]; }
-    if (has_e && i + 1 < C::TMI) load_e(i + 1);
+      for (int pass = 0; pass < NPASS; ++pass)
+#pragma unroll
+        for (int h = 0; h < NV; ++h) ec[pass][h] = ev[pass][h];
+      if (i + 1 < C::TMI) load_e(i + 1);
+    }
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
-      const int r = pass * RPP + lane / CPR;
-      const int c8 = (lane % CPR) * 8;
-      const int m = band_m + r, n = wn0 + c8;
-      if (m < d.M && n < d.N) {
+      const int r = pass * RPP + lr;
+      const int m = band_m + r;
+      if (col_ok && (FULL || m < d.M)) {
         float* sp = stg + r * PITCH + c8;
         const float4 a0 = *reinterpret_cast<const float4*>(sp);
         const float4 a1 = *reinterpret_cast<const float4*>(sp + 4);
         float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
         float e[8];
-        const long long off = (long long)m * d.ldc + n;
-        if (ep.c_f32) {
-          const uint32_t w[8] = {ec[pass][0].x, ec[pass][0].y, ec[pass][0].z, ec[pass][0].w,
-                                 ec[pass][1].x, ec[pass][1].y, ec[pass][1].z, ec[pass][1].w};
+        char* Cp = Cbase + ((long long)m * d.ldc + wn0 + c8) * CSZ;
+        if (CF32) {
 #pragma unroll
-          for (int q = 0; q < 8; ++q) e[q] = __builtin_bit_cast(float, w[q]);
+          for (int q = 0; q < 8; ++q) {
+            const unsigned w = HAS_E ? ec[pass][q >> 2][q & 3] : 0u;  // (bit_cast of a vector element lvalue reads element 0)
+            e[q] = __builtin_bit_cast(float, w);
+          }
 #pragma unroll
-          for (int q = 0; q < 8; ++q) v[q] = epi_value(ep, v[q], e[q]);
-          float* Cp = reinterpret_cast<float*>(Cbase) + off;
-          *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
-          *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
+          for (int q = 0; q < 8; ++q) v[q] = epi_value<HAS_E, FAITHFUL, true>(s0, s1, v[q], e[q]);
+          const u32x4_t o0 = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
+                              __builtin_bit_cast(unsigned, v[2]), __builtin_bit_cast(unsigned, v[3])};
+          const u32x4_t o1 = {__builtin_bit_cast(unsigned, v[4]), __builtin_bit_cast(unsigned, v[5]),
+                              __builtin_bit_cast(unsigned, v[6]), __builtin_bit_cast(unsigned, v[7])};
+          stg16(Cp, o0);
+          stg16(Cp + 16, o1);
         } else {
-          const uint32_t w[4] = {ec[pass][0].x, ec[pass][0].y, ec[pass][0].z, ec[pass][0].w};
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            e[2 * q] = bf2f((bf16_t)(w[q] & 0xffffu));
-            e[2 * q + 1] = bf2f((bf16_t)(w[q] >> 16));
+            const unsigned w = HAS_E ? ec[pass][0][q] : 0u;
+            e[2 * q] = __builtin_bit_cast(float, w << 16);
+            e[2 * q + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
           }
-          uint32_t pk[4];
+          u32x4_t pk;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const bf16_t lo = f2bf(epi_value(ep, v[2 * q], e[2 * q]));
-            const bf16_t hi = f2bf(epi_value(ep, v[2 * q + 1], e[2 * q + 1]));
-            pk[q] = (uint32_t)lo | ((uint32_t)hi << 16);
-            v[2 * q] = bf2f(lo);
-            v[2 * q + 1] = bf2f(hi);
+            const bf16_t lo = f2bf(epi_value<HAS_E, FAITHFUL, false>(s0, s1, v[2 * q], e[2 * q]));
+            const bf16_t hi = f2bf(epi_value<HAS_E, FAITHFUL, false>(s0, s1, v[2 * q + 1], e[2 * q + 1]));
+            pk[q] = (unsigned)lo | ((unsigned)hi << 16);
+            if (SYM) {
+              v[2 * q] = bf2f(lo);
+              v[2 * q + 1] = bf2f(hi);
+            }
           }
-          *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(Cbase) + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+          stg16(Cp, pk);
         }
-        if (mirror) {  // keep the final values for the transposed store
+        if (SYM && mirror) {  // keep the final values for the transposed store
           *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
           *reinterpret_cast<float4*>(sp + 4) = make_float4(v[4], v[5], v[6], v[7]);
         }
       }
     }
-    if (mirror) {
-      __syncthreads();
+    if (SYM && mirror) {
+      wave_sync_lds();
       // C^T: row n of the mirrored tile holds 32 consecutive m of this band
+#pragma unroll
       for (int pass = 0; pass < (W / 64) * 4; ++pass) {
         const int nl = (pass >> 2) * 64 + lane;
         const int mg = (pass & 3) * 8;
         const int n = wn0 + nl, m = band_m + mg;
-        if (n < d.N && m < d.M) {  // M is a multiple of 8 for symmetric outputs
+        if (FULL || (n < d.N && m < d.M)) {  // M is a multiple of 8 for symmetric outputs
           float v[8];
 #pragma unroll
           for (int q = 0; q < 8; ++q) v[q] = stg[(mg + q) * PITCH + nl];
-          const long long off = (long long)n * d.ldc + m;
-          if (ep.c_f32) {
-            float* Cp = reinterpret_cast<float*>(Cbase) + off;
-            *reinterpret_cast<float4*>(Cp) = make_float4(v[0], v[1], v[2], v[3]);
-            *reinterpret_cast<float4*>(Cp + 4) = make_float4(v[4], v[5], v[6], v[7]);
+          char* Cp = Cbase + ((long long)n * d.ldc + m) * CSZ;
+          if (CF32) {
+            const u32x4_t o0 = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
+                                __builtin_bit_cast(unsigned, v[2]), __builtin_bit_cast(unsigned, v[3])};
+            const u32x4_t o1 = {__builtin_bit_cast(unsigned, v[4]), __builtin_bit_cast(unsigned, v[5]),
+                                __builtin_bit_cast(unsigned, v[6]), __builtin_bit_cast(unsigned, v[7])};
+            stg16(Cp, o0);
+            stg16(Cp + 16, o1);
           } else {
-            uint32_t pk[4];
+            u32x4_t pk;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) pk[q] = (uint32_t)f2bf(v[2 * q]) | ((uint32_t)f2bf(v[2 * q + 1]) << 16);
-            *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(Cbase) + off) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            for (int q = 0; q < 4; ++q) pk[q] = (unsigned)f2bf(v[2 * q]) | ((unsigned)f2bf(v[2 * q + 1]) << 16);
+            stg16(Cp, pk);
           }
         }
       }
     }
-    __syncthreads();
+    wave_sync_lds();
   }
+}
+
+template <typename C, bool SYM, bool FULL>
+__device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
+                                         int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
+  const bool mirror = SYM && (ti != tj);
+  const bool cf32 = d.c_dtype == DA_F32, has_e = d.epilogue == DA_EPI_AXPBY, fa = d.faithful != 0;
+#define DA_EPI(CF, HE, FA) epilogue_impl<C, SYM, FULL, CF, HE, FA>(acc, d, lds, b, mirror, m0, n0, wave, lane, wm, wn)
+  if (!cf32) {
+    if (has_e) { if (fa) DA_EPI(false, true, true); else DA_EPI(false, true, false); }
+    else       { if (fa) DA_EPI(false, false, true); else DA_EPI(false, false, false); }
+  } else {
+    if (has_e) { if (fa) DA_EPI(true, true, true); else DA_EPI(true, true, false); }
+    else       { if (fa) DA_EPI(true, false, true); else DA_EPI(true, false, false); }
+  }
+#undef DA_EPI
 }
 
 // ---------------------------------------------------------------------------------------
@@ -517,7 +550,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
 #undef DA_MMA
 #undef DA_FREAD2
 #undef DA_MMA2
-  epilogue<C, SYM>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
+  epilogue<C, SYM, FULL>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
 }
 
 template <typename C, bool A_KS, bool B_KS, bool SYM>
@@ -572,8 +605,18 @@ int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
   static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
   if (forced == 128) return dispatch_layout<Small>(d, stream);
   if (forced == 256) return dispatch_layout<Big>(d, stream);
-  // Large tiles once there are enough of them to cover the 256 CUs; small tiles otherwise.
-  const long long t256 = (long long)((d.M + 255) / 256) * ((d.N + 255) / 256) * d.batch / (d.symmetric ? 2 : 1);
-  if (d.M >= 1024 && d.N >= 1024 && t256 >= 200) return dispatch_layout<Big>(d, stream);
+  // Tile choice by a two-term cost model: rounds of workgroups over the chip (256 x 256 tiles run
+  // one per CU, 128 x 128 tiles two per CU) times the cost of one tile (a small tile does a quarter
+  // of the work on half a CU at about 0.8 of the large tile's MFMA efficiency).  Interior-only
+  // (direct-to-LDS) eligibility wins over either.
+  auto tiles = [&](int bt) {
+    const long long tm = (d.M + bt - 1) / bt, tn = (d.N + bt - 1) / bt;
+    return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch;
+  };
+  const bool full_big = d.M % 256 == 0 && d.N % 256 == 0 && d.K % BK == 0;
+  const bool full_small = d.M % 128 == 0 && d.N % 128 == 0 && d.K % BK == 0;
+  const double cost_big = (double)((tiles(256) + 255) / 256) * 4.0;
+  const double cost_small = (double)((tiles(128) + 511) / 512) * 2.5;
+  if (d.M >= 256 && d.N >= 256 && (full_big || !full_small) && cost_big <= cost_small) return dispatch_layout<Big>(d, stream);
   return dispatch_layout<Small>(d, stream);
 }
