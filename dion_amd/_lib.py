@@ -28,6 +28,16 @@ _vp, _i, _ll, _f, _sz = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_float, _c.c_s
 _fp = _c.POINTER(_c.c_float)
 _vpp = _c.POINTER(_c.c_void_p)
 
+
+
+class MuonBucket(ctypes.Structure):
+    """`dion_amd_muon_bucket` of include/dion_amd.h."""
+    _fields_ = [("X", _vpp), ("G", _vpp), ("M", _vpp), ("batch", _i), ("m", _i), ("n", _i),
+                ("decay", _f), ("adjusted_lr", _f)]
+
+
+_bkp = _c.POINTER(MuonBucket)
+
 _SIGNATURES = {
     "dion_amd_version": (_c.c_char_p, []),
     "dion_amd_ns_workspace_bytes": (_sz, [_i, _i, _i, _i]),
@@ -46,6 +56,8 @@ _SIGNATURES = {
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),
     "dion_amd_muon_step": (_i, [_vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _f, _i, _f, _f, _fp, _i, _f, _i, _vp, _sz, _vp]),
+    "dion_amd_muon_buckets_workspace_bytes": (_sz, [_bkp, _i]),
+    "dion_amd_muon_step_buckets": (_i, [_bkp, _i, _i, _i, _f, _i, _fp, _i, _f, _i, _vp, _sz, _vp]),
 }
 
 _lib = None

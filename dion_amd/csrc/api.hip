@@ -2,6 +2,7 @@
 // the kernels of one Newton-Schulz / Muon bucket on a stream.
 #include "../../include/dion_amd.h"
 #include "common.h"
+#include <cstdlib>
 #include "elementwise.h"
 #include "prof.h"
 #include "dion.h"
@@ -12,17 +13,20 @@ inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Workspace carve-up for one chunk of `cb` wide matrices (mw x nw).
 struct NsLayout {
-  int mw, nw, tiles;
-  size_t esz;
-  size_t x_bytes, a_bytes, part_bytes;  // per matrix
-  size_t per_matrix;
+  int mw = 0, nw = 0, tiles = 0;
+  size_t esz = 0;
+  size_t x_bytes = 0, a_bytes = 0, part_bytes = 0;  // per matrix
+  size_t per_matrix = 0;
+  NsLayout() {}
   NsLayout(int m, int n, int dtype) {
     mw = m < n ? m : n;
     nw = m < n ? n : m;
     tiles = da_stage_tiles(m, n);
     esz = dtype == DA_BF16 ? 2 : 4;
-    x_bytes = align_up((size_t)mw * nw * esz, 256);
-    a_bytes = align_up((size_t)mw * mw * esz, 256);
+    // unpadded: the staging kernels index the working matrices densely ([batch][mw][nw]); with
+    // m and n multiples of 8 every matrix still starts on a 128-byte boundary
+    x_bytes = (size_t)mw * nw * esz;
+    a_bytes = (size_t)mw * mw * esz;
     part_bytes = align_up((size_t)tiles * sizeof(float) + sizeof(float), 256);
     per_matrix = 2 * x_bytes + 2 * a_bytes + part_bytes;
   }
@@ -42,8 +46,9 @@ struct NsLayout {
 };
 
 struct NsBuffers {
-  char *x0, *x1, *a, *b;
-  float *partials, *divisor;
+  char *x0 = nullptr, *x1 = nullptr, *a = nullptr, *b = nullptr;
+  float *partials = nullptr, *divisor = nullptr;
+  NsBuffers() {}
   NsBuffers(const NsLayout& L, void* ws, int cb) {
     char* p = static_cast<char*>(ws);
     x0 = p; p += L.x_bytes * cb;
@@ -66,54 +71,100 @@ int gemm_any(const GemmDesc& d, int dtype, hipStream_t s, int kind = DA_PROF_GEM
   return dtype == DA_BF16 ? da_gemm_bf16(d, s) : da_gemm_f32(d, s);
 }
 
-// steps x { A = X X^T ; B = b A + c A A ; X' = a X + B X } on cb wide matrices.
-// Returns in *result which of x0 / x1 holds the final iterate.
-int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const float* coeffs, int steps,
-               int faithful, hipStream_t s, char** result) {
-  char* x = W.x0;
-  char* y = W.x1;
-  const long long sx = (long long)(L.x_bytes / L.esz), sa = (long long)(L.a_bytes / L.esz);
+// `n` products of the same form: one grouped launch in bf16, one launch each in fp32.
+int gemm_group(const GemmDesc* d, int n, int dtype, hipStream_t s, int kind) {
+  double flops = 0.0;
+  for (int i = 0; i < n; ++i) flops += gemm_flops(d[i]);
+  static const bool nogroup = getenv("DION_AMD_NO_GROUP") != nullptr;
+  if (dtype == DA_BF16 && !nogroup) {
+    DaProfScope prof(kind, flops, s);
+    return da_gemm_bf16_grouped(d, n, s);
+  }
+  for (int i = 0; i < n; ++i) {
+    const int rc = gemm_any(d[i], dtype, s, kind);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+// One set of wide matrices iterated together with others: `cb` matrices of layout L in buffers W.
+struct NsSet {
+  NsLayout L;
+  NsBuffers W;
+  int cb = 0;
+};
+
+// steps x { A = X X^T ; B = b A + c A A ; X' = a X + B X } on up to DA_MAX_GROUPS sets of wide
+// matrices at once (each of the three products is one grouped launch over all sets).
+// Returns in result[i] which of x0 / x1 of set i holds the final iterate.
+int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int steps, int faithful, hipStream_t s,
+               char** result) {
+  if (nsets < 1 || nsets > DA_MAX_GROUPS) return DA_ERR_ARG;
+  char *x[DA_MAX_GROUPS], *y[DA_MAX_GROUPS];
+  for (int i = 0; i < nsets; ++i) { x[i] = sets[i].W.x0; y[i] = sets[i].W.x1; }
   for (int it = 0; it < steps; ++it) {
     const float a = coeffs[3 * it], b = coeffs[3 * it + 1], c = coeffs[3 * it + 2];
-    GemmDesc g{};
-    g.batch = cb; g.c_dtype = dtype; g.faithful = faithful;
+    GemmDesc g[DA_MAX_GROUPS];
     // A = X X^T   (symmetric output, k = nw)
-    g.A = x; g.B = x; g.C = W.a; g.E = nullptr;
-    g.sA = sx; g.sB = sx; g.sC = sa; g.sE = 0;
-    g.lda = L.nw; g.ldb = L.nw; g.ldc = L.mw; g.lde = 0;
-    g.M = L.mw; g.N = L.mw; g.K = L.nw;
-    g.a_kstrided = 0; g.b_kstrided = 0; g.symmetric = 1;
-    g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
-    int rc = gemm_any(g, dtype, s, DA_PROF_NS_SYRK);
+    for (int i = 0; i < nsets; ++i) {
+      const NsLayout& L = sets[i].L;
+      const NsBuffers& W = sets[i].W;
+      const long long sx = (long long)(L.x_bytes / L.esz), sa = (long long)(L.a_bytes / L.esz);
+      g[i] = GemmDesc{};
+      g[i].batch = sets[i].cb; g[i].c_dtype = dtype; g[i].faithful = faithful;
+      g[i].A = x[i]; g[i].B = x[i]; g[i].C = W.a; g[i].E = nullptr;
+      g[i].sA = sx; g[i].sB = sx; g[i].sC = sa; g[i].sE = 0;
+      g[i].lda = L.nw; g[i].ldb = L.nw; g[i].ldc = L.mw; g[i].lde = 0;
+      g[i].M = L.mw; g[i].N = L.mw; g[i].K = L.nw;
+      g[i].a_kstrided = 0; g[i].b_kstrided = 0; g[i].symmetric = 1;
+      g[i].epilogue = DA_EPI_STORE; g[i].s0 = 0.f; g[i].s1 = 1.f;
+    }
+    int rc = gemm_group(g, nsets, dtype, s, DA_PROF_NS_SYRK);
     if (rc) return rc;
     // B = b A + c A A^T   (A symmetric, so A A = A A^T: both operands k-contiguous)
-    g.A = W.a; g.B = W.a; g.C = W.b; g.E = W.a;
-    g.sA = sa; g.sB = sa; g.sC = sa; g.sE = sa;
-    g.lda = L.mw; g.ldb = L.mw; g.ldc = L.mw; g.lde = L.mw;
-    g.M = L.mw; g.N = L.mw; g.K = L.mw;
-    g.epilogue = DA_EPI_AXPBY; g.s0 = b; g.s1 = c;
-    rc = gemm_any(g, dtype, s, DA_PROF_NS_POLY);
+    for (int i = 0; i < nsets; ++i) {
+      const NsLayout& L = sets[i].L;
+      const NsBuffers& W = sets[i].W;
+      const long long sa = (long long)(L.a_bytes / L.esz);
+      g[i].A = W.a; g[i].B = W.a; g[i].C = W.b; g[i].E = W.a;
+      g[i].sA = sa; g[i].sB = sa; g[i].sC = sa; g[i].sE = sa;
+      g[i].lda = L.mw; g[i].ldb = L.mw; g[i].ldc = L.mw; g[i].lde = L.mw;
+      g[i].M = L.mw; g[i].N = L.mw; g[i].K = L.mw;
+      g[i].epilogue = DA_EPI_AXPBY; g[i].s0 = b; g[i].s1 = c;
+    }
+    rc = gemm_group(g, nsets, dtype, s, DA_PROF_NS_POLY);
     if (rc) return rc;
     // X' = a X + B X   (B symmetric: k-contiguous; X is the k-strided operand)
-    g.A = W.b; g.B = x; g.C = y; g.E = x;
-    g.sA = sa; g.sB = sx; g.sC = sx; g.sE = sx;
-    g.lda = L.mw; g.ldb = L.nw; g.ldc = L.nw; g.lde = L.nw;
-    g.M = L.mw; g.N = L.nw; g.K = L.mw;
-    g.a_kstrided = 0; g.b_kstrided = 1; g.symmetric = 0;
-    g.epilogue = DA_EPI_AXPBY; g.s0 = a; g.s1 = 1.f;
-    rc = gemm_any(g, dtype, s, DA_PROF_NS_AXPY);
+    for (int i = 0; i < nsets; ++i) {
+      const NsLayout& L = sets[i].L;
+      const NsBuffers& W = sets[i].W;
+      const long long sx = (long long)(L.x_bytes / L.esz), sa = (long long)(L.a_bytes / L.esz);
+      g[i].A = W.b; g[i].B = x[i]; g[i].C = y[i]; g[i].E = x[i];
+      g[i].sA = sa; g[i].sB = sx; g[i].sC = sx; g[i].sE = sx;
+      g[i].lda = L.mw; g[i].ldb = L.nw; g[i].ldc = L.nw; g[i].lde = L.nw;
+      g[i].M = L.mw; g[i].N = L.nw; g[i].K = L.mw;
+      g[i].a_kstrided = 0; g[i].b_kstrided = 1; g[i].symmetric = 0;
+      g[i].epilogue = DA_EPI_AXPBY; g[i].s0 = a; g[i].s1 = 1.f;
+    }
+    rc = gemm_group(g, nsets, dtype, s, DA_PROF_NS_AXPY);
     if (rc) return rc;
-    char* t = x; x = y; y = t;
+    for (int i = 0; i < nsets; ++i) { char* t = x[i]; x[i] = y[i]; y[i] = t; }
   }
-  *result = x;
+  for (int i = 0; i < nsets; ++i) result[i] = x[i];
   return DA_OK;
+}
+
+int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const float* coeffs, int steps,
+               int faithful, hipStream_t s, char** result) {
+  NsSet one;
+  one.L = L; one.W = W; one.cb = cb;
+  return ns_iterate(&one, 1, dtype, coeffs, steps, faithful, s, result);
 }
 
 int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
   DaProfScope prof(DA_PROF_NORMALIZE, 2.0 * (double)L.mw * L.nw * L.esz * cb, s);
   int rc = da_norm_finish(W.partials, L.tiles, cb, eps, dtype == DA_BF16, W.divisor, s);
   if (rc) return rc;
-  // x_bytes is padded per matrix; the pad is never read by the GEMMs, normalising it is harmless.
   return da_normalize(W.x0, dtype, (long long)(L.x_bytes / L.esz), cb, W.divisor, s);
 }
 
@@ -275,6 +326,98 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
       rc = da_unstage(us, s);
     }
     if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+size_t dion_amd_muon_buckets_workspace_bytes(const dion_amd_muon_bucket* buckets, int nbuckets) {
+  if (!buckets || nbuckets <= 0) return 0;
+  size_t worst = 0;
+  for (int r0 = 0; r0 < nbuckets; r0 += DA_MAX_GROUPS) {
+    size_t need = 0;
+    for (int i = r0; i < nbuckets && i < r0 + DA_MAX_GROUPS; ++i) {
+      if (buckets[i].batch <= 0 || buckets[i].m <= 0 || buckets[i].n <= 0) return 0;
+      need += align_up(NsLayout(buckets[i].m, buckets[i].n, DA_BF16).per_matrix * (size_t)buckets[i].batch, 256);
+    }
+    if (need > worst) worst = need;
+  }
+  return worst;
+}
+
+int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets, int x_dtype, int g_dtype, float mu,
+                               int nesterov, const float* coeffs, int steps, float eps, int faithful,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+  if (!buckets || nbuckets <= 0 || !coeffs || !workspace || steps < 0) return DA_ERR_ARG;
+  if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype)) return DA_ERR_DTYPE;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
+  for (int i = 0; i < nbuckets; ++i) {
+    const dion_amd_muon_bucket& k = buckets[i];
+    if (!k.X || !k.G || !k.M || k.batch <= 0 || k.m <= 0 || k.n <= 0) return DA_ERR_ARG;
+    if ((k.m | k.n) & 7) return DA_ERR_ALIGN;
+    for (int j = 0; j < k.batch; ++j) {
+      if (!k.X[j] || !k.G[j] || !k.M[j]) return DA_ERR_ARG;
+      if (((uintptr_t)k.X[j] | (uintptr_t)k.G[j] | (uintptr_t)k.M[j]) & 15) return DA_ERR_ALIGN;
+    }
+  }
+  if (workspace_bytes < dion_amd_muon_buckets_workspace_bytes(buckets, nbuckets)) return DA_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const double xsz = x_dtype == DA_BF16 ? 2 : 4, gsz = g_dtype == DA_BF16 ? 2 : 4;
+  for (int r0 = 0; r0 < nbuckets; r0 += DA_MAX_GROUPS) {
+    const int nr = nbuckets - r0 < DA_MAX_GROUPS ? nbuckets - r0 : DA_MAX_GROUPS;
+    // carve the workspace: every bucket of this round keeps all of its matrices resident
+    NsSet sets[DA_MAX_GROUPS];
+    char* p = static_cast<char*>(workspace);
+    for (int i = 0; i < nr; ++i) {
+      const dion_amd_muon_bucket& k = buckets[r0 + i];
+      const NsLayout L(k.m, k.n, DA_BF16);
+      sets[i].L = L;
+      sets[i].W = NsBuffers(L, p, k.batch);
+      sets[i].cb = k.batch;
+      p += align_up(L.per_matrix * (size_t)k.batch, 256);
+    }
+    // momentum update, bf16 staging in wide orientation, Frobenius partial sums; then normalise
+    for (int i = 0; i < nr; ++i) {
+      const dion_amd_muon_bucket& k = buckets[r0 + i];
+      const NsLayout& L = sets[i].L;
+      const NsBuffers& W = sets[i].W;
+      for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {
+        const int c = k.batch - j0 < DA_MAX_PTRS ? k.batch - j0 : DA_MAX_PTRS;
+        DaStage st{};
+        for (int j = 0; j < c; ++j) {
+          st.g.p[j] = const_cast<void*>(k.G[j0 + j]);
+          st.mom.p[j] = k.M[j0 + j];
+        }
+        st.wide = W.x0 + (size_t)j0 * L.x_bytes;
+        st.partials = W.partials + (size_t)j0 * L.tiles;
+        st.batch = c; st.rows = k.m; st.cols = k.n; st.ld = k.n;
+        st.g_dtype = g_dtype; st.m_dtype = x_dtype; st.w_dtype = DA_BF16;
+        st.mu = mu; st.nesterov = nesterov; st.muon = 1;
+        DaProfScope prof(DA_PROF_STAGE, (double)k.m * k.n * (gsz + 2 * xsz + 2) * c, s);
+        const int rc = da_stage_wide(st, s);
+        if (rc) return rc;
+      }
+      const int rc = ns_normalize_chunk(L, W, k.batch, DA_BF16, eps, s);
+      if (rc) return rc;
+    }
+    char* res[DA_MAX_GROUPS];
+    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res);
+    if (rc) return rc;
+    for (int i = 0; i < nr; ++i) {
+      const dion_amd_muon_bucket& k = buckets[r0 + i];
+      const NsLayout& L = sets[i].L;
+      for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {
+        const int c = k.batch - j0 < DA_MAX_PTRS ? k.batch - j0 : DA_MAX_PTRS;
+        DaUnstage us{};
+        for (int j = 0; j < c; ++j) us.x.p[j] = k.X[j0 + j];
+        us.wide = res[i] + (size_t)j0 * L.x_bytes;
+        us.batch = c; us.rows = k.m; us.cols = k.n; us.ld = k.n;
+        us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
+        us.decay = k.decay; us.step = k.adjusted_lr; us.muon = 1;
+        DaProfScope prof(DA_PROF_UNSTAGE, (double)k.m * k.n * (2 * xsz + 2) * c, s);
+        rc = da_unstage(us, s);
+        if (rc) return rc;
+      }
+    }
   }
   return DA_OK;
 }

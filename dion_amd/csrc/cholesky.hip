@@ -1,9 +1,19 @@
-// Diagonal-block step of the batched, blocked fp64 Cholesky used by the CholeskyQR
-// orthonormalisation: one workgroup per matrix factors a (<= 64) x (<= 64) block held in
-// LDS and inverts the triangular factor, so that the panel solve and the triangular solve
-// of P become plain GEMMs (gemm_f64.hip).  No host synchronisation: a failed pivot is
-// recorded in a device-side info word, mirroring torch.linalg.cholesky_ex's `info`.
+// One block-column step of the batched, blocked fp64 Cholesky used by the CholeskyQR
+// orthonormalisation, fused into a single launch: every workgroup factors the (<= 64) x (<= 64)
+// diagonal block in registers and inverts the triangular factor (redundantly -- the factor is the
+// serial part, repeating it costs no time), then does one 64 x 64 piece of what depends on it:
+//   role 0            : stores L_jj and its inverse D_j (the diagonal block of W, see below),
+//   roles 1 .. below  : one 64-row tile of the panel   L[i, j] = A[i, j] D_j^T,
+//   roles above that  : one 64-column tile of          W[j, c] = -D_j L[j, c],  c < j,
+// where W is the block-lower-triangular matrix with which the triangular solve of P becomes one
+// in-place GEMM per block column:  P[:, j] <- P[:, 0 .. j] W[j, 0 .. j]^T.
+// No host synchronisation: a failed pivot is recorded in a device-side info word, mirroring
+// torch.linalg.cholesky_ex's `info`.
 #include "gemm_f64.h"
+
+// fp64 factorisation: fused multiply-adds are welcome here (the build disables contraction
+// globally for the kernels that reproduce the reference's bf16 rounding points)
+#pragma clang fp contract(fast)
 
 namespace {
 
@@ -15,15 +25,16 @@ constexpr int NB = DA_CHOL_NB;
 // in registers, the column owners form their L blocks (A_ic * L_cc^-T), the row owners of the
 // inverse form X_c = L_cc^-1 * Y_c, both are published through LDS, and every thread applies
 // the two rank-4 updates.  Two barriers per 4 columns.
-__global__ __launch_bounds__(256) void chol_diag_kernel(const double* __restrict__ G, double* __restrict__ Lmat,
-                                                        long long sG, int r, int o, int nb, double* __restrict__ Dinv,
-                                                        long long sD, int* __restrict__ info) {
+__global__ __launch_bounds__(256) void chol_step_kernel(const double* __restrict__ G, double* __restrict__ Lmat,
+                                                        double* __restrict__ Wmat, long long sG, int r, int o, int nb,
+                                                        int below, int* __restrict__ info) {
   __shared__ double dinv4[4][4];       // inverse of the current diagonal 4 x 4 factor (lower)
   __shared__ double dfac4[4][4];       // the factor itself
   __shared__ double lcol[NB][4];       // rows > 4cb+3: L[i][4cb .. 4cb+3]
   __shared__ double xrow[4][NB];       // rows 4cb .. 4cb+3 of L^-1
   __shared__ int first_bad;
-  const int b = blockIdx.x, tid = threadIdx.x;
+  extern __shared__ __attribute__((aligned(16))) double opnd[];   // two k-major 64 x 64 operand tiles
+  const int b = blockIdx.y, role = blockIdx.x, tid = threadIdx.x;
   const int bi = tid >> 4, bj = tid & 15;
   const double* g = G + (long long)b * sG + (long long)o * r + o;
   double a[4][4], y[4][4];
@@ -47,8 +58,14 @@ __global__ __launch_bounds__(256) void chol_diag_kernel(const double* __restrict
       for (int c = 0; c < 4; ++c) {
         const double p = a[c][c];
         const bool ok = p > 0.0 && p < 1.0e300;  // false for NaN as well
-        const double d = ok ? sqrt(p) : 0.0;
-        di[c] = ok ? 1.0 / d : 0.0;
+        // 1/sqrt(p) from the hardware estimate plus two Newton steps (full fp64 accuracy), then
+        // sqrt(p) = p * rsqrt(p): this thread is the critical path of the whole factorisation and
+        // the library sqrt + divide are four times as long
+        double rs = ok ? (double)__builtin_amdgcn_rsq(p) : 0.0;
+        rs = rs * (1.5 - 0.5 * p * rs * rs);
+        rs = rs * (1.5 - 0.5 * p * rs * rs);
+        const double d = ok ? p * rs : 0.0;
+        di[c] = ok ? rs : 0.0;
         if (!ok && cb * 4 + c < nb && first_bad == 0) first_bad = o + cb * 4 + c + 1;
         a[c][c] = d;
 #pragma unroll
@@ -147,24 +164,110 @@ __global__ __launch_bounds__(256) void chol_diag_kernel(const double* __restrict
     }
   }
 
-  double* l = Lmat + (long long)b * sG + (long long)o * r + o;
-  double* di_out = Dinv + (long long)b * sD;
+  if (role == 0) {
+    double* l = Lmat + (long long)b * sG + (long long)o * r + o;
+    double* w = Wmat + (long long)b * sG + (long long)o * r + o;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int i = bi * 4 + ii, j = bj * 4 + jj;
+        if (i < nb && j < nb) {
+          l[(long long)i * r + j] = j <= i ? a[ii][jj] : 0.0;
+          w[(long long)i * r + j] = j <= i ? y[ii][jj] : 0.0;
+        }
+      }
+    if (tid == 0 && first_bad != 0 && info[b] == 0) info[b] = first_bad;
+    return;
+  }
+
+  // 64 x 64 x 64 product on the matrix cores: C[m][n] = sum_k opa[k][m] * opb[k][n]
+  double* opa = opnd;
+  double* opb = opnd + NB * NB;
+  const bool panel = role <= below;
+  // D_j (zero outside its nb x nb lower triangle) goes in transposed: D^T[k][x] = D[x][k]
+  double* dt = panel ? opb : opa;
 #pragma unroll
   for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int i = bi * 4 + ii, j = bj * 4 + jj;
-      if (i < nb && j < nb) l[(long long)i * r + j] = j <= i ? a[ii][jj] : 0.0;
-      di_out[i * NB + j] = (i < nb && j <= i) ? y[ii][jj] : 0.0;
+      dt[j * NB + i] = (i < nb && j <= i) ? y[ii][jj] : 0.0;
     }
-  if (tid == 0 && first_bad != 0 && info[b] == 0) info[b] = first_bad;
+  int row0, col0, rows_ok, cols_ok;
+  if (panel) {
+    // opa[k][m] = A[row0 + m][o + k]
+    row0 = o + nb + (role - 1) * NB;
+    col0 = o;
+    rows_ok = r - row0 < NB ? r - row0 : NB;
+    cols_ok = nb;
+    const double* src = G + (long long)b * sG + (long long)row0 * r + o;
+    for (int e = tid; e < NB * NB; e += 256) {
+      const int m = e >> 6, k = e & 63;
+      opa[k * NB + m] = (m < rows_ok && k < nb) ? src[(long long)m * r + k] : 0.0;
+    }
+  } else {
+    // opb[k][n] = L[o + k][col0 + n]
+    row0 = o;
+    col0 = (role - 1 - below) * NB;
+    rows_ok = nb;
+    cols_ok = NB;   // col0 + 64 <= o
+    const double* src = Lmat + (long long)b * sG + (long long)o * r + col0;
+    for (int e = tid; e < NB * NB; e += 256) {
+      const int k = e >> 6, n = e & 63;
+      opb[k * NB + n] = k < nb ? src[(long long)k * r + n] : 0.0;
+    }
+  }
+  __syncthreads();
+  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+  f64x4_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+#pragma unroll 4
+  for (int ks = 0; ks < NB / 4; ++ks) {
+    const int k = ks * 4 + (lane >> 4);
+    double af[2], bfv[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = opa[k * NB + wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) bfv[j] = opb[k * NB + wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+  }
+  double* dst = (panel ? Lmat : Wmat) + (long long)b * sG + (long long)row0 * r + col0;
+  const double sign = panel ? 1.0 : -1.0;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = wm * 32 + i * 16 + v * 4 + (lane >> 4);
+        const int n = wn * 32 + j * 16 + (lane & 15);
+        if (m < rows_ok && n < cols_ok) dst[(long long)m * r + n] = sign * acc[i][j][v];
+      }
 }
 
 }  // namespace
 
-int da_chol_diag(const double* G, double* Lmat, long long sG, int r, int o, int nb, double* Dinv, long long sD,
-                 int* info, int batch, hipStream_t s) {
-  if (nb <= 0 || nb > NB || o < 0 || o + nb > r || batch <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(chol_diag_kernel, dim3(batch), dim3(256), 0, s, G, Lmat, sG, r, o, nb, Dinv, sD, info);
+int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
+                 int batch, hipStream_t s) {
+  if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  const int rest = r - o - nb;
+  if (rest > 0 && nb != NB) return DA_ERR_ARG;
+  const int below = (rest + NB - 1) / NB;
+  const int smem = 2 * NB * NB * (int)sizeof(double);
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(chol_step_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    configured = true;
+  }
+  hipLaunchKernelGGL(chol_step_kernel, dim3(1 + below + o / NB, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb,
+                     below, info);
   return da_launch_status();
 }

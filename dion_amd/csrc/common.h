@@ -94,4 +94,10 @@ struct GemmDesc {
 #define DA_EPI_AXPBY 1  // C = s0 * E + s1 * acc; E may alias C (in-place update)
 
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream);
+
+// Several independent batched bf16 GEMMs of the same form (operand layouts, symmetry, epilogue
+// kind and output dtype) in one launch: their tiles share the grid, so a product too small to
+// fill the chip runs beside the others instead of after them.
+constexpr int DA_MAX_GROUPS = 4;
+int da_gemm_bf16_grouped(const GemmDesc* d, int n, hipStream_t stream);
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream);

@@ -262,11 +262,8 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 // CholeskyQR2 in fp64
 // ---------------------------------------------------------------------------------------
 size_t da_orth_workspace_bytes(int batch, int rows, int r) {
-  const size_t nblk = (r + DA_CHOL_NB - 1) / DA_CHOL_NB;
-  size_t per = 2 * (size_t)rows * r * 8        // P0, P1
-               + (size_t)rows * DA_CHOL_NB * 8  // S
-               + 2 * (size_t)r * r * 8          // G, L
-               + nblk * DA_CHOL_NB * DA_CHOL_NB * 8;
+  size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place
+               + 3 * (size_t)r * r * 8;   // G, L, W
   return per * batch + 256;
 }
 
@@ -274,14 +271,11 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
                       int* info, hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
-  const long long pr = (long long)rows * r, rr = (long long)r * r, sS = (long long)rows * NB,
-                  sD = (long long)nblk * NB * NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
   double* P0 = static_cast<double*>(ws);
-  double* P1 = P0 + pr * batch;
-  double* S = P1 + pr * batch;
-  double* G = S + sS * batch;
+  double* G = P0 + pr * batch;
   double* L = G + rr * batch;
-  double* D = L + rr * batch;
+  double* W = L + rr * batch;
   int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
   if (rc) return rc;
   for (int pass = 0; pass < passes; ++pass) {
@@ -308,56 +302,39 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     }
     rc = da_gemm_f64(g, s);
     if (rc) return rc;
-    // blocked lower Cholesky G = L L^T
+    // blocked lower Cholesky G = L L^T (right-looking), building W alongside
     for (int j = 0; j < nblk; ++j) {
       const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-      rc = da_chol_diag(G, L, rr, r, o, nb, D + (long long)j * NB * NB, sD, info, batch, s);
+      rc = da_chol_step(G, L, W, rr, r, o, nb, info, batch, s);
       if (rc) return rc;
       if (rest <= 0) break;
-      Gemm64Desc t{};
-      t.batch = batch;
-      // L21 = A21 L11^-T
-      t.A = G + (long long)(o + nb) * r + o; t.sA = rr; t.lda = r; t.a_kstrided = 0;
-      t.B = D + (long long)j * NB * NB; t.sB = sD; t.ldb = NB; t.b_kstrided = 0;
-      t.C = L + (long long)(o + nb) * r + o; t.sC = rr; t.ldc = r;
-      t.M = rest; t.N = nb; t.K = nb; t.alpha = 1.0; t.beta = 0.0; t.E = nullptr;
-      rc = da_gemm_f64(t, s);
-      if (rc) return rc;
-      // A22 -= L21 L21^T
+      // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
       Gemm64Desc u{};
       u.batch = batch;
-      u.A = t.C; u.sA = rr; u.lda = r; u.a_kstrided = 0;
-      u.B = t.C; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+      u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
+      u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
       u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
       u.E = u.C; u.sE = rr; u.lde = r;
-      u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0;
+      u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
       rc = da_gemm_f64(u, s);
       if (rc) return rc;
     }
-    // P1 = P0 R^-1 with R = L^T, block column by block column
+    // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
+    //   P0[:, j] <- P0[:, 0 .. j] W[j, 0 .. j]^T
+    // (each workgroup owns 64 rows and the one 64-column output tile, and has read all it needs of
+    // those rows before it stores)
     for (int j = 0; j < nblk; ++j) {
       const int o = j * NB, nb = r - o < NB ? r - o : NB;
       Gemm64Desc a{};
       a.batch = batch;
-      // S = P0[:, blk] - P1[:, :o] L[blk, :o]^T
-      a.A = P1; a.sA = pr; a.lda = r; a.a_kstrided = 0;
-      a.B = L + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
-      a.C = S; a.sC = sS; a.ldc = NB;
-      a.E = P0 + o; a.sE = pr; a.lde = r;
-      a.M = rows; a.N = nb; a.K = o; a.alpha = -1.0; a.beta = 1.0;
+      a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+      a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
+      a.C = P0 + o; a.sC = pr; a.ldc = r;
+      a.E = nullptr;
+      a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
       rc = da_gemm_f64(a, s);
       if (rc) return rc;
-      // P1[:, blk] = S L_jj^-T
-      Gemm64Desc c{};
-      c.batch = batch;
-      c.A = S; c.sA = sS; c.lda = NB; c.a_kstrided = 0;
-      c.B = D + (long long)j * NB * NB; c.sB = sD; c.ldb = NB; c.b_kstrided = 0;
-      c.C = P1 + o; c.sC = pr; c.ldc = r;
-      c.M = rows; c.N = nb; c.K = nb; c.alpha = 1.0; c.beta = 0.0; c.E = nullptr;
-      rc = da_gemm_f64(c, s);
-      if (rc) return rc;
     }
-    double* tmp = P0; P0 = P1; P1 = tmp;
   }
   return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
 }

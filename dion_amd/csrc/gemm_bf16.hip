@@ -37,6 +37,13 @@ typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BK = 64;       // k elements per stage
 
+// Kernel argument: up to DA_MAX_GROUPS products; group g owns blocks start[g] .. start[g+1]-1.
+struct GemmArgs {
+  GemmDesc d[DA_MAX_GROUPS];
+  int start[DA_MAX_GROUPS + 1];
+  int n;
+};
+
 template <int BT_, int WGM_, int WGN_>
 struct Cfg {
   static constexpr int BT = BT_, WGM = WGM_, WGN = WGN_;
@@ -185,13 +192,11 @@ __device__ __forceinline__ void stg16(char* p, u32x4_t v) { *(global_u32x4_t*)p 
 struct TileId { int b, ti, tj; };
 
 template <int BT, bool SYM>
-__device__ __forceinline__ TileId decode_tile(const GemmDesc& d) {
+__device__ __forceinline__ TileId decode_tile(const GemmDesc& d, int bid, int nblk, bool xcd_aligned) {
   const int tiles_m = (d.M + BT - 1) / BT;
   const int tiles_n = (d.N + BT - 1) / BT;
   const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
-  int bid = blockIdx.x;
-  const int nblk = gridDim.x;
-  if ((nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  if (xcd_aligned && (nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
   TileId r;
   r.b = bid / per_batch;
   int t = bid - r.b * per_batch;
@@ -392,7 +397,14 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
 //     written to LDS after the stage's MFMAs.
 // ---------------------------------------------------------------------------------------
 template <typename C, bool A_KS, bool B_KS, bool SYM, bool FULL>
-__global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
+__global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
+  // which of the grouped products this workgroup belongs to (groups own contiguous block ranges)
+  int grp = 0;
+#pragma unroll
+  for (int q = 1; q < DA_MAX_GROUPS; ++q)
+    if (q < args.n && (int)blockIdx.x >= args.start[q]) grp = q;
+  const GemmDesc& d = args.d[grp];
+  const int blk0 = args.start[grp];
   constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ, NCH = C::NCH, NW = C::NT / 64;
   constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
   constexpr int B_BYTES = Tile<BT, B_KS>::bytes;
@@ -403,7 +415,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
   const int lane = tid & 63;
   const int wave = wave_uniform(tid >> 6);
   const int wm = wave / C::WGN, wn = wave % C::WGN;
-  const TileId tile = decode_tile<BT, SYM>(d);
+  const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0);
   const int b = tile.b, ti = tile.ti, tj = tile.tj;
   const int m0 = ti * BT, n0 = tj * BT;
   const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
@@ -553,13 +565,18 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmDesc d) {
   epilogue<C, SYM, FULL>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
 }
 
+template <typename C>
+long long tiles_of(const GemmDesc& d) {
+  const long long tm = (d.M + C::BT - 1) / C::BT, tn = (d.N + C::BT - 1) / C::BT;
+  return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch;
+}
+
 template <typename C, bool A_KS, bool B_KS, bool SYM>
-int launch(const GemmDesc& d, hipStream_t stream) {
+int launch(const GemmDesc* d, int n, hipStream_t stream) {
   constexpr int BT = C::BT;
   constexpr int stage2 = 2 * (Tile<BT, A_KS>::bytes + Tile<BT, B_KS>::bytes);
   constexpr int epi = (C::NT / 64) * 32 * (C::WCOLS + 4) * 4;
   constexpr int smem = stage2 > epi ? stage2 : epi;
-  const bool full = (d.M % BT == 0) && (d.N % BT == 0) && (d.K % BK == 0);
   auto kfull = gemm_bf16_kernel<C, A_KS, B_KS, SYM, true>;
   auto kgen = gemm_bf16_kernel<C, A_KS, B_KS, SYM, false>;
   static bool configured = false;  // benign race: the attribute calls are idempotent
@@ -568,28 +585,35 @@ int launch(const GemmDesc& d, hipStream_t stream) {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kgen), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
-  const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
-  const long long blocks = per_batch * d.batch;
-  if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
-  hipLaunchKernelGGL(full ? kfull : kgen, dim3((unsigned)blocks), dim3(C::NT), smem, stream, d);
+  GemmArgs args{};
+  args.n = n;
+  bool full = true;
+  long long blocks = 0;
+  for (int g = 0; g < n; ++g) {
+    args.d[g] = d[g];
+    args.start[g] = (int)blocks;
+    full = full && (d[g].M % BT == 0) && (d[g].N % BT == 0) && (d[g].K % BK == 0);
+    const long long t = tiles_of<C>(d[g]);
+    if (t <= 0) return DA_ERR_LIMIT;
+    blocks += t;
+    if (blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
+  }
+  for (int g = n; g <= DA_MAX_GROUPS; ++g) args.start[g] = (int)blocks;
+  hipLaunchKernelGGL(full ? kfull : kgen, dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
   return da_launch_status();
 }
 
 template <typename C>
-int dispatch_layout(const GemmDesc& d, hipStream_t stream) {
-  if (d.symmetric) return launch<C, false, false, true>(d, stream);
-  if (!d.a_kstrided && !d.b_kstrided) return launch<C, false, false, false>(d, stream);
-  if (!d.a_kstrided && d.b_kstrided) return launch<C, false, true, false>(d, stream);
-  if (d.a_kstrided && !d.b_kstrided) return launch<C, true, false, false>(d, stream);
-  return launch<C, true, true, false>(d, stream);
+int dispatch_layout(const GemmDesc* d, int n, hipStream_t stream) {
+  const GemmDesc& f = d[0];
+  if (f.symmetric) return launch<C, false, false, true>(d, n, stream);
+  if (!f.a_kstrided && !f.b_kstrided) return launch<C, false, false, false>(d, n, stream);
+  if (!f.a_kstrided && f.b_kstrided) return launch<C, false, true, false>(d, n, stream);
+  if (f.a_kstrided && !f.b_kstrided) return launch<C, true, false, false>(d, n, stream);
+  return launch<C, true, true, false>(d, n, stream);
 }
 
-}  // namespace
-
-// Alignment contract: K, N, every leading dimension and every batch stride are multiples
-// of 8 elements (16-byte chunks); M too when A is k-strided; pointers 16-byte aligned.
-int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
+int check_desc(const GemmDesc& d) {
   if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0)
     return DA_ERR_ARG;
   if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
@@ -600,23 +624,71 @@ int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) {
   if (d.a_kstrided && (d.M & 7)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;
   if (d.symmetric && (d.M != d.N || d.a_kstrided || d.b_kstrided)) return DA_ERR_ARG;
+  return DA_OK;
+}
+
+// Estimated duration of the launch with tile configuration C, in units of "one 64-deep stage of a
+// 256 x 256 tile on a whole CU": groups are taken longest-K first (the order they are launched
+// in), `slots` tiles run at a time, the last group's partial round is rounded up, and no launch
+// is shorter than its longest tile.
+template <typename C>
+double launch_cost(const GemmDesc* d, int n, int slots, double unit) {
+  double level = 0.0, longest = 0.0;
+  for (int g = 0; g < n; ++g) {
+    const double kt = (double)((d[g].K + BK - 1) / BK);
+    const double rounds = (double)tiles_of<C>(d[g]) / slots;
+    if (g + 1 < n) {
+      level += rounds * kt;
+    } else {
+      // the last group first fills what the earlier ones left of their final round
+      const double frac = level > 0.0 ? 0.5 : 0.0;
+      double r = rounds - frac;
+      if (r < 0.0) r = 0.0;
+      level += ((double)(long long)(r + 0.999999)) * kt;
+    }
+    if (kt > longest) longest = kt;
+  }
+  return unit * (level > longest ? level : longest);
+}
+
+}  // namespace
+
+// Alignment contract: K, N, every leading dimension and every batch stride are multiples
+// of 8 elements (16-byte chunks); M too when A is k-strided; pointers 16-byte aligned.
+int da_gemm_bf16_grouped(const GemmDesc* din, int n, hipStream_t stream) {
+  if (!din || n <= 0 || n > DA_MAX_GROUPS) return DA_ERR_ARG;
+  GemmDesc d[DA_MAX_GROUPS];
+  for (int g = 0; g < n; ++g) {
+    const int rc = check_desc(din[g]);
+    if (rc) return rc;
+    const GemmDesc &a = din[g], &f = din[0];
+    if (a.symmetric != f.symmetric || a.a_kstrided != f.a_kstrided || a.b_kstrided != f.b_kstrided ||
+        a.epilogue != f.epilogue || a.c_dtype != f.c_dtype || a.faithful != f.faithful)
+      return DA_ERR_ARG;
+    // insertion sort, longest K first: long tiles start early, short ones fill the tail
+    int pos = g;
+    while (pos > 0 && d[pos - 1].K < a.K) { d[pos] = d[pos - 1]; --pos; }
+    d[pos] = a;
+  }
   typedef Cfg<256, 2, 4> Big;
   typedef Cfg<128, 2, 2> Small;
   static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
-  if (forced == 128) return dispatch_layout<Small>(d, stream);
-  if (forced == 256) return dispatch_layout<Big>(d, stream);
-  // Tile choice by a two-term cost model: rounds of workgroups over the chip (256 x 256 tiles run
-  // one per CU, 128 x 128 tiles two per CU) times the cost of one tile (a small tile does a quarter
-  // of the work on half a CU at about 0.8 of the large tile's MFMA efficiency).  Interior-only
-  // (direct-to-LDS) eligibility wins over either.
-  auto tiles = [&](int bt) {
-    const long long tm = (d.M + bt - 1) / bt, tn = (d.N + bt - 1) / bt;
-    return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch;
-  };
-  const bool full_big = d.M % 256 == 0 && d.N % 256 == 0 && d.K % BK == 0;
-  const bool full_small = d.M % 128 == 0 && d.N % 128 == 0 && d.K % BK == 0;
-  const double cost_big = (double)((tiles(256) + 255) / 256) * 4.0;
-  const double cost_small = (double)((tiles(128) + 511) / 512) * 2.5;
-  if (d.M >= 256 && d.N >= 256 && (full_big || !full_small) && cost_big <= cost_small) return dispatch_layout<Big>(d, stream);
-  return dispatch_layout<Small>(d, stream);
+  if (forced == 128) return dispatch_layout<Small>(d, n, stream);
+  if (forced == 256) return dispatch_layout<Big>(d, n, stream);
+  // Tile choice by cost model: 256 x 256 tiles run one per CU, 128 x 128 tiles two per CU; a small
+  // tile does a quarter of the work on half a CU at about 2/3 of the large tile's MFMA efficiency
+  // (measured on grouped Newton-Schulz products of 768-wide matrices).
+  // Interior-only (direct-to-LDS) eligibility wins over either.
+  bool full_big = true, full_small = true, fits_big = true;
+  for (int g = 0; g < n; ++g) {
+    full_big = full_big && d[g].M % 256 == 0 && d[g].N % 256 == 0 && d[g].K % BK == 0;
+    full_small = full_small && d[g].M % 128 == 0 && d[g].N % 128 == 0 && d[g].K % BK == 0;
+    fits_big = fits_big && d[g].M >= 256 && d[g].N >= 256;
+  }
+  const double cost_big = launch_cost<Big>(d, n, 256, 4.0);
+  const double cost_small = launch_cost<Small>(d, n, 512, 3.0);
+  if (fits_big && (full_big || !full_small) && cost_big <= cost_small) return dispatch_layout<Big>(d, n, stream);
+  return dispatch_layout<Small>(d, n, stream);
 }
+
+int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) { return da_gemm_bf16_grouped(&d, 1, stream); }

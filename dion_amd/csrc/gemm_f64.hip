@@ -56,16 +56,18 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
-  const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  const bool tri = SYM || d.lower_only;
+  const int per_batch = tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
   const int split = blockIdx.y;  // split-K slice
   const int b = blockIdx.x / per_batch;
   int t = blockIdx.x - b * per_batch;
   int ti, tj;
-  if (SYM) {
+  if (tri) {
     ti = 0;
     int len = tiles_m;
     while (t >= len) { t -= len; ++ti; --len; }
     tj = ti + t;
+    if (!SYM) { const int x = ti; ti = tj; tj = x; }   // lower triangle: row tile >= column tile
   } else {
     ti = t / tiles_n;
     tj = t - ti * tiles_n;
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
 template <bool A_KS, bool B_KS, bool SYM>
 int launch(const Gemm64Desc& d, hipStream_t s) {
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
-  const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
+  const long long per_batch = (SYM || d.lower_only) ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
   const long long blocks = per_batch * d.batch;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
   int split = d.split_k > 1 ? d.split_k : 1;
@@ -187,6 +189,7 @@ inline unsigned cvt_blocks(long long n) {
 
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) {
   if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K < 0 || d.batch <= 0) return DA_ERR_ARG;
+  if (d.lower_only && (d.M != d.N || d.symmetric)) return DA_ERR_ARG;
   if (d.symmetric) {
     if (d.M != d.N || !d.a_kstrided || !d.b_kstrided) return DA_ERR_ARG;  // only the Gram form A^T A
     return launch<true, true, true>(d, s);

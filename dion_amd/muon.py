@@ -15,6 +15,8 @@ import math
 from collections import defaultdict
 from typing import Callable, List, Optional, Tuple
 
+import ctypes
+
 import torch
 from torch import Tensor
 from torch.optim.optimizer import Optimizer, ParamsT
@@ -172,6 +174,10 @@ class Muon(Optimizer):
         for p in params:
             buckets[(p.shape, p.dtype, p.grad.dtype, p.device)].append(p)
 
+        # Buckets of one (dtype, grad dtype, device) go to the library together: their Newton-Schulz
+        # products are grouped launches, so small buckets share the GPU instead of queueing
+        # (the reference overlaps them as async tasks, dion/muon.py:185-270).
+        fused = defaultdict(list)
         for (shape, dtype, gdtype, device), plist in buckets.items():
             states = [self._get_or_initialize_state(p, "muon") for p in plist]
             adjusted_lr = lr if adjust is None else _ADJUST[adjust](lr, shape)
@@ -180,20 +186,31 @@ class Muon(Optimizer):
                 continue
             _lib.require_gpu(plist[0], "Muon.step")
             X, G, M = self._matrix_views(plist, states, group["flatten"])
-            m, n = X[0].shape
+            fused[(dtype, gdtype, device)].append((X, G, M, float(adjusted_lr)))
+
+        decay = 1 - lr * weight_decay
+        for (dtype, gdtype, device), items in fused.items():
             lib = _lib.load()
-            ws = self._workspace.get(lib.dion_amd_muon_workspace_bytes(len(X), m, n), device)
-            decay = 1 - lr * weight_decay
+            arr = (_lib.MuonBucket * len(items))()
+            keep = []  # pointer arrays (and contiguous gradient copies) must outlive the call
+            for b, (X, G, M, alr) in zip(arr, items):
+                px, pg, pm = _lib.ptr_array(X), _lib.ptr_array(G), _lib.ptr_array(M)
+                keep.append((px, pg, pm, G))
+                b.X, b.G, b.M = (ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p)) for a in (px, pg, pm))
+                b.batch = len(X)
+                b.m, b.n = X[0].shape
+                b.decay = decay.item()
+                b.adjusted_lr = alr
+            ws = self._workspace.get(lib.dion_amd_muon_buckets_workspace_bytes(arr, len(items)), device)
             with torch.cuda.device(device):
-                rc = lib.dion_amd_muon_step(
-                    _lib.ptr_array(X), _lib.ptr_array(G), _lib.ptr_array(M), len(X), m, n,
-                    _lib.dtype_code(dtype), _lib.dtype_code(gdtype),
-                    mu.item(), int(bool(group["nesterov"])), decay.item(), float(adjusted_lr),
+                rc = lib.dion_amd_muon_step_buckets(
+                    arr, len(items), _lib.dtype_code(dtype), _lib.dtype_code(gdtype),
+                    mu.item(), int(bool(group["nesterov"])),
                     self._coeffs, len(NS_SCHEDULE_COEFFS), epsilon.item(), 1,
                     ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
                 )
-            _lib.check(rc, "dion_amd_muon_step")
-            del G  # keeps contiguous gradient copies alive until the launches are enqueued
+            _lib.check(rc, "dion_amd_muon_step_buckets")
+            del keep
 
     @staticmethod
     def _matrix_views(plist: List[Tensor], states: List[dict], flatten: bool):

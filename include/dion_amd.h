@@ -120,6 +120,31 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
                        const float* coeffs, int steps, float eps, int faithful,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* Several buckets (each of one shape) in one call.  Replaces the task generator and the task
+ * runtime around muon_update_batch_async (reference dion/muon.py:185-270 _create_muon_tasks,
+ * 134-183 step; dion/opt_utils.py AsyncRuntime): where the reference overlaps buckets as
+ * concurrent async tasks, here the buckets advance through Newton-Schulz in lock step and
+ * each of its three products is ONE grouped launch over up to four buckets, so that a bucket
+ * too small to fill the GPU shares it with the others.  Results per matrix are those of
+ * dion_amd_muon_step.  Every bucket keeps all its matrices resident in the workspace
+ * (no chunking): workspace_bytes must be at least dion_amd_muon_buckets_workspace_bytes(),
+ * else DA_ERR_WORKSPACE and nothing is launched. */
+typedef struct dion_amd_muon_bucket {
+  void* const* X;        /* HOST arrays of `batch` device pointers, as in dion_amd_muon_step */
+  const void* const* G;
+  void* const* M;
+  int batch, m, n;
+  float decay;           /* 1 - lr * weight_decay */
+  float adjusted_lr;     /* adjust_lr_* (m, n) applied to lr */
+} dion_amd_muon_bucket;
+
+size_t dion_amd_muon_buckets_workspace_bytes(const dion_amd_muon_bucket* buckets, int nbuckets);
+
+int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets,
+                               int x_dtype, int g_dtype, float mu, int nesterov,
+                               const float* coeffs, int steps, float eps, int faithful,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Dion step for one bucket of same-shape matrices
  * ------------------------------------------------------------------------------------- */

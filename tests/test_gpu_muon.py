@@ -155,3 +155,64 @@ def test_muon_custom_newton_schulz_hook(dev):
     assert calls and calls[0][0] == torch.bfloat16 and calls[0][1] == (64, 32)
     assert abs(calls[0][2] - 1e-8) < 1e-12
     assert torch.allclose(p.detach(), torch.full_like(p, 1 - 0.1 * 0.5), atol=1e-3)  # U * lr rounds in bf16
+
+
+def test_muon_step_buckets_equals_per_bucket_calls(dev):
+    """The multi-bucket entry (grouped launches, more buckets than one grouped launch takes, a bucket
+    of more matrices than one staging launch takes, shapes that are not multiples of the tile) gives
+    per matrix what dion_amd_muon_step gives for each bucket on its own."""
+    import ctypes
+
+    from dion_amd import _lib
+    from dion_amd.newton_schulz import NS_SCHEDULE_COEFFS, flat_coeffs
+
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(11)
+    specs = [((256, 256), 5), ((128, 512), 3), ((512, 128), 3), ((40, 24), 2), ((16, 32), 70), ((8, 24), 1)]
+    coeffs = flat_coeffs(NS_SCHEDULE_COEFFS)
+    steps = len(NS_SCHEDULE_COEFFS)
+
+    def fresh():
+        g2 = torch.Generator().manual_seed(12)
+        out = []
+        for shape, nb in specs:
+            X = [(torch.randn(shape, generator=g2) * 0.02).bfloat16().to(dev) for _ in range(nb)]
+            G = [(torch.randn(shape, generator=g2) * 1e-3).bfloat16().to(dev) for _ in range(nb)]
+            M = [(torch.randn(shape, generator=g2) * 1e-3).bfloat16().to(dev) for _ in range(nb)]
+            out.append((X, G, M))
+        return out
+
+    single = fresh()
+    for (shape, nb), (X, G, M) in zip(specs, single):
+        m, n = shape
+        ws = torch.empty(lib.dion_amd_muon_workspace_bytes(nb, m, n), dtype=torch.uint8, device=dev)
+        rc = lib.dion_amd_muon_step(_lib.ptr_array(X), _lib.ptr_array(G), _lib.ptr_array(M), nb, m, n, _lib.BF16,
+                                    _lib.BF16, 0.95, 1, 0.9998, 0.02 * (m / n) ** 0.5, coeffs, steps, 1e-8, 1,
+                                    ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+        _lib.check(rc, "dion_amd_muon_step")
+
+    multi = fresh()
+    arr = (_lib.MuonBucket * len(specs))()
+    keep = []
+    for b, (shape, nb), (X, G, M) in zip(arr, specs, multi):
+        ptrs = [_lib.ptr_array(t) for t in (X, G, M)]
+        keep.append(ptrs)
+        b.X, b.G, b.M = (ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p)) for a in ptrs)
+        b.batch, b.m, b.n = nb, shape[0], shape[1]
+        b.decay, b.adjusted_lr = 0.9998, 0.02 * (shape[0] / shape[1]) ** 0.5
+    need = lib.dion_amd_muon_buckets_workspace_bytes(arr, len(specs))
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    # one byte short: refused before anything is launched
+    assert lib.dion_amd_muon_step_buckets(arr, len(specs), _lib.BF16, _lib.BF16, 0.95, 1, coeffs, steps, 1e-8, 1,
+                                          ws.data_ptr(), need - 1, _lib.stream_ptr(dev)) == -3
+    rc = lib.dion_amd_muon_step_buckets(arr, len(specs), _lib.BF16, _lib.BF16, 0.95, 1, coeffs, steps, 1e-8, 1,
+                                        ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+    _lib.check(rc, "dion_amd_muon_step_buckets")
+    torch.cuda.synchronize()
+    for (shape, nb), (Xs, _, Ms), (Xm, _, Mm) in zip(specs, single, multi):
+        for j in range(nb):
+            assert torch.equal(Ms[j], Mm[j]), f"momentum differs: {shape} #{j}"
+            # tile configuration may differ between a grouped and a single launch; accumulation order
+            # per output element does not, so the weights agree to the last bit
+            assert torch.equal(Xs[j], Xm[j]), f"weights differ: {shape} #{j}"
