@@ -105,6 +105,10 @@ def measure(wl, dev, steps, warmup):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
 
+    # Second pass for the per-launch figures.  Dion runs its buckets on up to three streams; for this
+    # pass they run one at a time so that a launch's duration is that of the kernel alone.
+    if hasattr(opt, "_max_concurrent_tasks"):
+        opt._max_concurrent_tasks = 1
     lib = _lib.load()
     lib.dion_amd_profile_reset()
     lib.dion_amd_profile_enable(1)

@@ -1,7 +1,8 @@
 // One block-column step of the batched, blocked fp64 Cholesky used by the CholeskyQR
 // orthonormalisation, fused into a single launch: every workgroup factors the (<= 64) x (<= 64)
 // diagonal block in registers and inverts the triangular factor (redundantly -- the factor is the
-// serial part, repeating it costs no time), then does one 64 x 64 piece of what depends on it:
+// serial part; a few workgroups per matrix repeat it rather than wait for one), then they share
+// the 64 x 64 pieces of what depends on it:
 //   role 0            : stores L_jj and its inverse D_j (the diagonal block of W, see below),
 //   roles 1 .. below  : one 64-row tile of the panel   L[i, j] = A[i, j] D_j^T,
 //   roles above that  : one 64-column tile of          W[j, c] = -D_j L[j, c],  c < j,
@@ -18,6 +19,7 @@
 namespace {
 
 constexpr int NB = DA_CHOL_NB;
+constexpr int LP = NB + 1;   // LDS pitch of the operand tiles (doubles): transposed stores stay nearly conflict-free
 
 // 256 threads as a 16 x 16 grid; thread (bi, bj) keeps the 4 x 4 blocks of the working matrix
 // and of the inverse-in-progress at block position (bi, bj) in registers.  Right-looking with
@@ -34,7 +36,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const double* __restrict
   __shared__ double xrow[4][NB];       // rows 4cb .. 4cb+3 of L^-1
   __shared__ int first_bad;
   extern __shared__ __attribute__((aligned(16))) double opnd[];   // two k-major 64 x 64 operand tiles
-  const int b = blockIdx.y, role = blockIdx.x, tid = threadIdx.x;
+  const int b = blockIdx.y, tid = threadIdx.x;
   const int bi = tid >> 4, bj = tid & 15;
   const double* g = G + (long long)b * sG + (long long)o * r + o;
   double a[4][4], y[4][4];
@@ -164,92 +166,98 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const double* __restrict
     }
   }
 
-  if (role == 0) {
-    double* l = Lmat + (long long)b * sG + (long long)o * r + o;
-    double* w = Wmat + (long long)b * sG + (long long)o * r + o;
-#pragma unroll
-    for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int i = bi * 4 + ii, j = bj * 4 + jj;
-        if (i < nb && j < nb) {
-          l[(long long)i * r + j] = j <= i ? a[ii][jj] : 0.0;
-          w[(long long)i * r + j] = j <= i ? y[ii][jj] : 0.0;
-        }
-      }
-    if (tid == 0 && first_bad != 0 && info[b] == 0) info[b] = first_bad;
-    return;
-  }
-
-  // 64 x 64 x 64 product on the matrix cores: C[m][n] = sum_k opa[k][m] * opb[k][n]
-  double* opa = opnd;
-  double* opb = opnd + NB * NB;
-  const bool panel = role <= below;
-  // D_j (zero outside its nb x nb lower triangle) goes in transposed: D^T[k][x] = D[x][k]
-  double* dt = panel ? opb : opa;
+  // D_j (zero outside its nb x nb lower triangle), transposed: dT[k][x] = D[x][k]
+  double* dT = opnd;
+  double* op = opnd + NB * LP;
 #pragma unroll
   for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int i = bi * 4 + ii, j = bj * 4 + jj;
-      dt[j * NB + i] = (i < nb && j <= i) ? y[ii][jj] : 0.0;
+      dT[j * LP + i] = (i < nb && j <= i) ? y[ii][jj] : 0.0;
     }
-  int row0, col0, rows_ok, cols_ok;
-  if (panel) {
-    // opa[k][m] = A[row0 + m][o + k]
-    row0 = o + nb + (role - 1) * NB;
-    col0 = o;
-    rows_ok = r - row0 < NB ? r - row0 : NB;
-    cols_ok = nb;
-    const double* src = G + (long long)b * sG + (long long)row0 * r + o;
-    for (int e = tid; e < NB * NB; e += 256) {
-      const int m = e >> 6, k = e & 63;
-      opa[k * NB + m] = (m < rows_ok && k < nb) ? src[(long long)m * r + k] : 0.0;
-    }
-  } else {
-    // opb[k][n] = L[o + k][col0 + n]
-    row0 = o;
-    col0 = (role - 1 - below) * NB;
-    rows_ok = nb;
-    cols_ok = NB;   // col0 + 64 <= o
-    const double* src = Lmat + (long long)b * sG + (long long)o * r + col0;
-    for (int e = tid; e < NB * NB; e += 256) {
-      const int k = e >> 6, n = e & 63;
-      opb[k * NB + n] = k < nb ? src[(long long)k * r + n] : 0.0;
-    }
-  }
-  __syncthreads();
   const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-  f64x4_t acc[2][2];
+  const int nroles = 1 + below + o / NB;
+  // the workgroups of one matrix share its roles round-robin
+  for (int role = blockIdx.x; role < nroles; role += gridDim.x) {
+    if (role == 0) {
+      double* l = Lmat + (long long)b * sG + (long long)o * r + o;
+      double* w = Wmat + (long long)b * sG + (long long)o * r + o;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+      for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
-#pragma unroll 4
-  for (int ks = 0; ks < NB / 4; ++ks) {
-    const int k = ks * 4 + (lane >> 4);
-    double af[2], bfv[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) af[i] = opa[k * NB + wm * 32 + i * 16 + (lane & 15)];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) bfv[j] = opb[k * NB + wn * 32 + j * 16 + (lane & 15)];
+        for (int jj = 0; jj < 4; ++jj) {
+          const int i = bi * 4 + ii, j = bj * 4 + jj;
+          if (i < nb && j < nb) {
+            l[(long long)i * r + j] = j <= i ? a[ii][jj] : 0.0;
+            w[(long long)i * r + j] = j <= i ? y[ii][jj] : 0.0;
+          }
+        }
+      if (tid == 0 && first_bad != 0 && info[b] == 0) info[b] = first_bad;
+      continue;
+    }
+    // 64 x 64 x 64 product on the matrix cores: C[m][n] = sum_k opa[k][m] * opb[k][n]
+    const bool panel = role <= below;
+    int row0, col0, rows_ok, cols_ok;
+    __syncthreads();   // `op` may still be read by the previous role's MFMAs; dT is complete after it
+    if (panel) {
+      // L[i, j] = A[i, j] D^T :  opa[k][m] = A[row0 + m][o + k],  opb = dT
+      row0 = o + nb + (role - 1) * NB;
+      col0 = o;
+      rows_ok = r - row0 < NB ? r - row0 : NB;
+      cols_ok = nb;
+      const double* src = G + (long long)b * sG + (long long)row0 * r + o;
+      for (int e = tid; e < NB * NB; e += 256) {
+        const int m = e >> 6, k = e & 63;
+        op[k * LP + m] = (m < rows_ok && k < nb) ? src[(long long)m * r + k] : 0.0;
+      }
+    } else {
+      // W[j, c] = -D L[j, c] :  opa = dT,  opb[k][n] = L[o + k][col0 + n]
+      row0 = o;
+      col0 = (role - 1 - below) * NB;   // col0 + 64 <= o
+      rows_ok = nb;
+      cols_ok = NB;
+      const double* src = Lmat + (long long)b * sG + (long long)o * r + col0;
+      for (int e = tid; e < NB * NB; e += 256) {
+        const int k = e >> 6, n = e & 63;
+        op[k * LP + n] = k < nb ? src[(long long)k * r + n] : 0.0;
+      }
+    }
+    __syncthreads();
+    const double* opa = panel ? op : dT;
+    const double* opb = panel ? dT : op;
+    f64x4_t acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+#pragma unroll 4
+    for (int ks = 0; ks < NB / 4; ++ks) {
+      const int k = ks * 4 + (lane >> 4);
+      double af[2], bfv[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = opa[k * LP + wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bfv[j] = opb[k * LP + wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+    }
+    double* dst = (panel ? Lmat : Wmat) + (long long)b * sG + (long long)row0 * r + col0;
+    const double sign = panel ? 1.0 : -1.0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = wm * 32 + i * 16 + v * 4 + (lane >> 4);
+          const int n = wn * 32 + j * 16 + (lane & 15);
+          if (m < rows_ok && n < cols_ok) dst[(long long)m * r + n] = sign * acc[i][j][v];
+        }
   }
-  double* dst = (panel ? Lmat : Wmat) + (long long)b * sG + (long long)row0 * r + col0;
-  const double sign = panel ? 1.0 : -1.0;
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int m = wm * 32 + i * 16 + v * 4 + (lane >> 4);
-        const int n = wn * 32 + j * 16 + (lane & 15);
-        if (m < rows_ok && n < cols_ok) dst[(long long)m * r + n] = sign * acc[i][j][v];
-      }
 }
 
 }  // namespace
@@ -260,14 +268,19 @@ int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int 
   const int rest = r - o - nb;
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
   const int below = (rest + NB - 1) / NB;
-  const int smem = 2 * NB * NB * (int)sizeof(double);
+  const int smem = 2 * NB * LP * (int)sizeof(double);
+  // workgroups per matrix: enough for ~384 in flight over the batch, never more than there are roles
+  const int nroles = 1 + below + o / NB;
+  int per = 384 / batch;
+  if (per < 1) per = 1;
+  if (per > nroles) per = nroles;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(chol_step_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  hipLaunchKernelGGL(chol_step_kernel, dim3(1 + below + o / NB, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb,
+  hipLaunchKernelGGL(chol_step_kernel, dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb,
                      below, info);
   return da_launch_status();
 }

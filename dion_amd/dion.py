@@ -107,7 +107,13 @@ class Dion(Optimizer):
         if mixed_precision_config is None:
             mixed_precision_config = DionMixedPrecisionConfig()
         self._mixed_precision_config = mixed_precision_config
-        self._workspace = _lib.Workspace()
+        # Buckets are independent tasks; like the reference's AsyncRuntime(max_concurrent_tasks=3)
+        # (dion/dion.py:268) up to three of them are in flight, here on HIP streams of their own
+        # (default priority), each with its own workspace.  The orthonormaliser is a chain of short
+        # launches that cannot fill the GPU, so buckets overlap nearly for free.
+        self._max_concurrent_tasks = 3
+        self._workspaces = [_lib.Workspace() for _ in range(self._max_concurrent_tasks)]
+        self._streams = {}
         self._info = {}
 
     @torch.no_grad()
@@ -210,25 +216,44 @@ class Dion(Optimizer):
         for p in params:
             buckets[(p.shape, p.dtype, p.grad.dtype, p.device)].append(p)
         lib = _lib.load()
+        # optimizer state and status words are created on the caller's stream, before any fork
         for (shape, dtype, gdtype, device), plist in buckets.items():
             _lib.require_gpu(plist[0], "Dion.step")
+            for p in plist:
+                self._get_or_initialize_state(p, group)
+            info = self._info.get((shape, dtype, device))
+            if info is None or info.numel() != len(plist):
+                self._info[(shape, dtype, device)] = torch.zeros(len(plist), dtype=torch.int32, device=device)
+        slots = min(len(buckets), self._max_concurrent_tasks)
+        forked = {}
+        for index, ((shape, dtype, gdtype, device), plist) in enumerate(buckets.items()):
+            slot = index % slots
+            main = torch.cuda.current_stream(device)
+            if slots == 1:
+                stream = main
+            else:
+                pool = self._streams.setdefault(device, [])
+                while len(pool) < slots:
+                    pool.append(torch.cuda.Stream(device=device))
+                stream = pool[slot]
+                if (device, slot) not in forked:
+                    stream.wait_stream(main)   # gradients and earlier updates were produced on `main`
+                    forked[(device, slot)] = (main, stream)
             states = [self._get_or_initialize_state(p, group) for p in plist]
             m, n = shape
             Ms = [s["momentum"] for s in states]
             Qs = [s["Q"] for s in states]
             r = Qs[0].size(1)
-            Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
             for t in (*plist, *Ms, *Qs):
                 if not t.is_contiguous():
                     raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
             scaled_lr = ((m / n) ** 0.5) * lr
             mcode = _lib.dtype_code(Ms[0].dtype)
-            ws = self._workspace.get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
-            info = self._info.get((shape, dtype, device))
-            if info is None or info.numel() != len(plist):
-                info = torch.zeros(len(plist), dtype=torch.int32, device=device)
-                self._info[(shape, dtype, device)] = info
-            with torch.cuda.device(device):
+            info = self._info[(shape, dtype, device)]
+            with torch.cuda.device(device), torch.cuda.stream(stream):
+                # contiguous gradient copies and the workspace belong to this stream
+                Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
+                ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
                 rc = lib.dion_amd_dion_step(
                     _lib.ptr_array(plist), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
                     len(plist), m, n, r,
@@ -236,8 +261,10 @@ class Dion(Optimizer):
                     ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1,
                     info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
                 )
-            _lib.check(rc, "dion_amd_dion_step")
-            del Gs
+                _lib.check(rc, "dion_amd_dion_step")
+                del Gs
+        for main, stream in forked.values():
+            main.wait_stream(stream)
 
     # ------------------------------------------------------------------ element-wise groups
     def _lion_group_step(self, group: dict):
