@@ -8,7 +8,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdion_amd.so")
+# DION_AMD_LIB names another build of the same library (kernel experiments); default: in-tree
+LIB_PATH = os.environ.get("DION_AMD_LIB") or os.path.join(_HERE, "libdion_amd.so")
 
 BF16, F32, F64 = 0, 1, 2
 EPI_STORE, EPI_AXPBY = 0, 1

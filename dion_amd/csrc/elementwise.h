@@ -11,9 +11,10 @@ struct DaPtrTable {
 struct DaStage {
   DaPtrTable g;      // source matrices (rows x cols, row pitch ld)
   DaPtrTable mom;    // momentum buffers (contiguous rows x cols), Muon mode only
-  void* wide;        // [batch][min(rows,cols)][max(rows,cols)] working matrices
+  void* wide;        // [batch][min(rows,cols)][ldw] working matrices, max(rows,cols) columns used
   float* partials;   // [batch][da_stage_tiles(rows, cols)]
   int batch, rows, cols, ld;
+  int ldw;           // row pitch of the working matrices (elements, multiple of 8, >= max(rows,cols))
   int g_dtype, m_dtype, w_dtype;
   float mu;
   int nesterov;
@@ -24,6 +25,7 @@ struct DaUnstage {
   DaPtrTable x;      // destinations (rows x cols, row pitch ld)
   const void* wide;
   int batch, rows, cols, ld;
+  int ldw;           // row pitch of the working matrices
   int x_dtype, w_dtype;
   float decay, step;
   int muon;

@@ -71,10 +71,11 @@ template <typename TG, typename TM, typename TW>
 struct StageArgs {
   DaPtrTable g;       // sources (gradients), one pointer per matrix
   DaPtrTable mom;     // momentum buffers (Muon mode), modified in place; unused for plain
-  TW* wide;           // [batch][mw][nw]
+  TW* wide;           // [batch][mw][ldw], columns < nw used
   float* partials;    // [batch][tiles]
   int rows, cols;     // source shape
   int ld;             // source row pitch (elements)
+  int ldw;            // row pitch of the wide matrices (elements)
   float mu;
   int nesterov;
   int muon;           // 1: momentum update, 0: plain cast
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
   const TG* G = static_cast<const TG*>(a.g.p[b]);
   TM* M = a.muon ? static_cast<TM*>(a.mom.p[b]) : nullptr;
   const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
-  TW* W = a.wide + (long long)b * mw * nw;
+  TW* W = a.wide + (long long)b * mw * a.ldw;
 
   float ss = 0.f;
 #pragma unroll
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss += u[e] * u[e];
-      if (!TALL) Vec8<TW>::store(W + (long long)i * nw + j, u);
+      if (!TALL) Vec8<TW>::store(W + (long long)i * a.ldw + j, u);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) u[e] = 0.f;
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
         float u[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) u[e] = tile[p][qq + e];
-        Vec8<TW>::store(W + (long long)wi * nw + wj, u);
+        Vec8<TW>::store(W + (long long)wi * a.ldw + wj, u);
       }
     }
   }
@@ -201,8 +202,8 @@ __global__ __launch_bounds__(256) void normalize_kernel(TW* W, long long per_mat
 template <typename TX, typename TW>
 struct UnstageArgs {
   DaPtrTable x;       // destinations, one pointer per matrix (rows x cols, row-major, pitch ld)
-  const TW* wide;     // [batch][mw][nw]
-  int rows, cols, ld;
+  const TW* wide;     // [batch][mw][ldw], columns < nw used
+  int rows, cols, ld, ldw;
   float decay;        // 1 - lr * weight_decay
   float step;         // adjusted learning rate
   int muon;           // 1: X <- X*decay - wide*step ; 0: X <- wide
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
   const int tid = threadIdx.x;
   TX* X = static_cast<TX*>(a.x.p[b]);
   const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
-  const TW* W = a.wide + (long long)b * mw * nw;
+  const TW* W = a.wide + (long long)b * mw * a.ldw;
 
   if (TALL) {
 #pragma unroll
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
       const int p = c >> 3, qq = (c & 7) * 8;
       const int wi = tj * TS + p, wj = ti * TS + qq;
       float u[8];
-      if (wi < mw && wj < nw) Vec8<TW>::load(W + (long long)wi * nw + wj, u);
+      if (wi < mw && wj < nw) Vec8<TW>::load(W + (long long)wi * a.ldw + wj, u);
       else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) u[e] = 0.f;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) u[e] = tile[r][cc + e];
     } else {
-      Vec8<TW>::load(W + (long long)i * nw + j, u);
+      Vec8<TW>::load(W + (long long)i * a.ldw + j, u);
     }
     TX* xp = X + (long long)i * a.ld + j;
     if (a.muon) {
@@ -278,16 +279,16 @@ int stage_launch(const StageArgs<TG, TM, TW>& a, int batch, bool tall, hipStream
 template <typename TG, typename TM>
 int stage_dispatch_w(const DaStage& d, hipStream_t s) {
   if (d.w_dtype == DA_BF16) {
-    StageArgs<TG, TM, bf16_t> a{d.g, d.mom, static_cast<bf16_t*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.mu, d.nesterov, d.muon};
+    StageArgs<TG, TM, bf16_t> a{d.g, d.mom, static_cast<bf16_t*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon};
     return stage_launch(a, d.batch, d.rows > d.cols, s);
   }
-  StageArgs<TG, TM, float> a{d.g, d.mom, static_cast<float*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.mu, d.nesterov, d.muon};
+  StageArgs<TG, TM, float> a{d.g, d.mom, static_cast<float*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon};
   return stage_launch(a, d.batch, d.rows > d.cols, s);
 }
 
 template <typename TX, typename TW>
 int unstage_launch(const DaUnstage& d, hipStream_t s) {
-  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.decay, d.step, d.muon};
+  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon};
   const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
   dim3 grid(tiles, d.batch);
   if (d.rows > d.cols) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
