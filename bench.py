@@ -151,7 +151,13 @@ def summarize(name, wl, res):
     return out
 
 
-def roofline_of(res, kind):
+# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.000 and
+# WRITE_SIZE x 1.000, in KiB, the factors being what the same counters read for a plain 512 MiB copy);
+# the summary of those runs is profiles/muon_gpt_small_hbm_traffic.md.  Keyed by (workload, kernel).
+MEASURED_TRAFFIC_BYTES = {("muon_gpt_small", "ns_axpy"): 683634 * 1024}
+
+
+def roofline_of(res, kind, workload=None):
     """Dominant GEMM kernel of the run: algorithmic flops per launch / average launch duration."""
     prof = res["prof"]
     cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
@@ -160,7 +166,8 @@ def roofline_of(res, kind):
     n, ms, work = prof[dom]
     achieved = work / (ms * 1e-3) / 1e12
     return dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=PEAK_BF16_FLOPS / 1e12, unit="TFLOP/s",
-                frac=round(achieved * 1e12 / PEAK_BF16_FLOPS, 4), traffic=None,
+                frac=round(achieved * 1e12 / PEAK_BF16_FLOPS, 4),
+                traffic=MEASURED_TRAFFIC_BYTES.get((workload, dom)),
                 avg_launch_ms=round(ms / n, 5), flops_per_launch=work / n)
 
 
@@ -251,7 +258,7 @@ def main():
                    "optimizer": res["optimizer"], "grad": f"N(0,1e-3) seed {wl['seed']}", "parallelism": "single GPU"},
         "event_ms_per_step": round(res["event_ms"], 4),
         "wall_ms_per_step": round(res["wall_ms"], 4),
-        "roofline": roofline_of(res, wl["kind"]),
+        "roofline": roofline_of(res, wl["kind"], args.workload),
     }
     out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
     if not args.no_extra:
@@ -263,7 +270,7 @@ def main():
             big = "llama" in name
             r = measure(w, dev, 3 if big else 10, 1 if big else 2)
             s = summarize(name, w, r)
-            s["roofline"] = roofline_of(r, w["kind"])
+            s["roofline"] = roofline_of(r, w["kind"], name)
             extra[name] = s
         out["extra"] = extra
     if not args.no_cpu_baseline:
