@@ -128,7 +128,7 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
  * too small to fill the GPU shares it with the others.  Results per matrix are those of
  * dion_amd_muon_step.  Every bucket keeps all its matrices resident in the workspace
  * (no chunking): workspace_bytes must be at least dion_amd_muon_buckets_workspace_bytes(),
- * else DA_ERR_WORKSPACE and nothing is launched. */
+ * else DION_AMD_ERR_WORKSPACE and nothing is launched. */
 typedef struct dion_amd_muon_bucket {
   void* const* X;        /* HOST arrays of `batch` device pointers, as in dion_amd_muon_step */
   const void* const* G;
