@@ -15,6 +15,7 @@ Workloads (BASELINE.json `configs`):
   dion_gpt_small_r1     rank fraction 1.0; bf16 weights / momentum, fp32 Q, G seed 3.
   muon_llama8b_layer    (configs[3], one of the 32 layers) Muon on 7 bf16 matrices incl. 4096x14336.
   dion_llama70b_layer   (configs[4], one of the 8 layers) Dion r=512 on 2 x 28672x8192 + 8192x28672.
+  scalar_gpt_small      the non-matrix groups of GPT-small: Lion / AdamW on embedding, lm_head, norms.
 """
 import argparse
 import json
@@ -43,6 +44,8 @@ WORKLOADS = {
                                desc="Muon step, one Llama-3-8B layer: 7 bf16 matrices incl. 4096x14336"),
     "dion_llama70b_layer": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER, seed=5, rank_fraction=1.0 / 16,
                                 desc="Dion step, one Llama-3-70B MLP layer (28672x8192 x2, 8192x28672), r=512"),
+    "scalar_gpt_small": dict(kind="scalar", shapes=[(50304, 768)] * 2 + [(768,)] * 25, seed=6,
+                             desc="Lion on the GPT-small embedding and norms, AdamW on lm_head (50304x768 each), bf16"),
 }
 GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd")
 
@@ -74,6 +77,11 @@ def build_optimizer(wl, dev):
     params = [torch.nn.Parameter(x.to(dev)) for x in X]
     for p, g in zip(params, G):
         p.grad = g.to(dev)
+    if wl["kind"] == "scalar":
+        opt = Muon([dict(params=[params[0]] + params[2:], algorithm="lion"),
+                    dict(params=[params[1]], algorithm="adamw")], lr=0.01, weight_decay=0.01)
+        desc = "Muon(param groups: lion [embedding, 25 norm vectors], adamw [lm_head]; lr=0.01, betas=(0.9, 0.95), wd=0.01)"
+        return opt, params, desc
     if wl["kind"] == "muon":
         opt = Muon(params, lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True, adjust_lr="spectral_norm")
         desc = "Muon(lr=0.02, mu=0.95, nesterov=True, weight_decay=0.01, adjust_lr=spectral_norm)"
@@ -158,8 +166,15 @@ MEASURED_TRAFFIC_BYTES = {("muon_gpt_small", "ns_axpy"): 683634 * 1024}
 
 
 def roofline_of(res, kind, workload=None):
-    """Dominant GEMM kernel of the run: algorithmic flops per launch / average launch duration."""
+    """Dominant kernel of the run: algorithmic flops (bytes for the HBM-bound passes) per launch / average launch
+    duration."""
     prof = res["prof"]
+    if kind == "scalar":
+        n, ms, work = prof["scalar_opt"]
+        achieved = work / (ms * 1e-3) / 1e9
+        return dict(bound="hbm", kernel="scalar_opt", achieved=round(achieved, 1), peak=PEAK_HBM_BPS / 1e9, unit="GB/s",
+                    frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4), traffic=None, avg_launch_ms=round(ms / n, 5),
+                    bytes_per_launch=work / n)
     cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
                          else ("dion_bq", "dion_btp", "dion_ef", "dion_upd")) if k in prof]
     dom = max(cands, key=lambda k: prof[k][1])
@@ -263,7 +278,8 @@ def main():
     out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
     if not args.no_extra:
         extra = {}
-        for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "dion_llama70b_layer"):
+        for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "dion_llama70b_layer",
+                     "scalar_gpt_small"):
             if name == args.workload:
                 continue
             w = WORKLOADS[name]

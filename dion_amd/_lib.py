@@ -57,6 +57,9 @@ _SIGNATURES = {
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),
     "dion_amd_muon_step": (_i, [_vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _f, _i, _f, _f, _fp, _i, _f, _i, _vp, _sz, _vp]),
+    "dion_amd_lion_step": (_i, [_vpp, _vpp, _vpp, _c.POINTER(_ll), _i, _i, _i, _i, _f, _f, _f, _f, _vp]),
+    "dion_amd_adamw_step": (_i, [_vpp, _vpp, _vpp, _vpp, _c.POINTER(_ll), _i, _i, _i, _i, _i,
+                                 _f, _f, _f, _f, _f, _f, _vp]),
     "dion_amd_muon_buckets_workspace_bytes": (_sz, [_bkp, _i]),
     "dion_amd_muon_step_buckets": (_i, [_bkp, _i, _i, _i, _f, _i, _fp, _i, _f, _i, _vp, _sz, _vp]),
 }
@@ -140,7 +143,7 @@ class Workspace:
 
 
 PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
-              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem")
+              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt")
 
 
 def profile_read():

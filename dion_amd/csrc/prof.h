@@ -17,7 +17,8 @@ enum DaProfKind {
   DA_PROF_DION_UPD = 10,  // X <- (1 - lr wd) X - lr' P Q^T
   DA_PROF_DION_ORTH = 11, // orthonormalisation of P (all of its launches)
   DA_PROF_DION_ELEM = 12, // B = M + G, column norms, guards
-  DA_PROF_KINDS = 13
+  DA_PROF_SCALAR_OPT = 13,// fused Lion / AdamW pass over non-matrix parameters
+  DA_PROF_KINDS = 14
 };
 
 struct DaProfScope {

@@ -1,0 +1,218 @@
+// Lion and AdamW for the parameter groups that are not matrices (embeddings, lm_head, norms,
+// biases): one fused multi-tensor pass each, in place, HBM-bound.  Replaces the reference's
+// lion_update_foreach / adamw_update_foreach (dion/scalar_opts.py:152-187, 89-149), whose every
+// tensor op is a separate pass over memory; the rounding points of those ops (each result is
+// rounded to the dtype of the tensor that holds it) are reproduced in registers.
+//
+//   Lion :  g = r_M(G);  U = sign(r_M(lerp(M, g, r_M(1-b1))));  M <- r_M(lerp(M, g, r_M(1-b2)));
+//           X <- r_X(X * (1 - lr wd));  X <- r_X(X - r_M(U * lr))
+//   AdamW:  g = r_M(G);  M <- r_M(lerp(M, g, r_M(1-b1)));  V <- r_V(lerp(V, r_V(r_M(g g)), r_V(1-b2)));
+//           den = r_V(r_V(r_V(sqrt V) / sqrt(1-b2^t)) + eps);  X <- r_X(X * (1 - lr wd));
+//           X <- r_X(X - r_D(r_D(M / den) * lr / (1-b1^t)))          (D = the wider of M's and V's dtype)
+//
+// Tensors of one call share their dtypes; each has its own length.  A tensor whose pointers are
+// all 16-byte aligned moves as 8-element vectors (plus a scalar tail), any other element by element.
+#include "../../include/dion_amd.h"
+#include "common.h"
+#include "prof.h"
+
+namespace {
+
+constexpr int MAX_TENSORS = 48;   // per launch: the table travels as a kernel argument
+
+struct ScalarTable {
+  void* x[MAX_TENSORS];
+  const void* g[MAX_TENSORS];
+  void* m[MAX_TENSORS];
+  void* v[MAX_TENSORS];
+  long long n[MAX_TENSORS];
+  unsigned char vec[MAX_TENSORS];   // 1: every pointer of the tensor is 16-byte aligned
+};
+
+struct ScalarArgs {
+  float w1, w2;        // 1 - beta1, 1 - beta2 (lerp weights)
+  float decay;         // 1 - lr * weight_decay
+  float lr;            // Lion: lr;  AdamW: lr / (1 - beta1^step)
+  float bc2_sqrt;      // AdamW: sqrt(1 - beta2^step)
+  float eps;           // AdamW
+  int x_dtype, g_dtype, m_dtype, v_dtype;
+};
+
+__device__ __forceinline__ float rnd(float x, int dtype) { return dtype == DA_BF16 ? rbf(x) : x; }
+
+// torch.lerp with a 0-dim tensor weight: the weight is first cast to the dtype of the tensors (so in
+// bf16 1 - 0.95 becomes 0.050048828125), then start + w (end - start) for |w| < 0.5, else
+// end - (end - start)(1 - w); one rounding of the fused multiply-add in fp32, then the store's rounding
+__device__ __forceinline__ float lerp_f(float s, float e, float w_in, int dtype) {
+  const float w = rnd(w_in, dtype);
+  const float d = e - s;
+  return fabsf(w) < 0.5f ? fmaf(w, d, s) : fmaf(-(1.0f - w), d, e);
+}
+
+__device__ __forceinline__ float ld1(const void* p, int dtype, long long i) {
+  return dtype == DA_BF16 ? bf2f(static_cast<const bf16_t*>(p)[i]) : static_cast<const float*>(p)[i];
+}
+__device__ __forceinline__ void st1(void* p, int dtype, long long i, float v) {
+  if (dtype == DA_BF16) static_cast<bf16_t*>(p)[i] = f2bf(v);
+  else static_cast<float*>(p)[i] = v;
+}
+__device__ __forceinline__ void ld8(const void* p, int dtype, long long i, float (&v)[8]) {
+  if (dtype == DA_BF16) {
+    const uint4 r = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(p) + i);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v[2 * q] = __builtin_bit_cast(float, w[q] << 16);
+      v[2 * q + 1] = __builtin_bit_cast(float, w[q] & 0xffff0000u);
+    }
+  } else {
+    const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+    const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+}
+__device__ __forceinline__ void st8(void* p, int dtype, long long i, const float (&v)[8]) {
+  if (dtype == DA_BF16) {
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) w[q] = (uint32_t)f2bf(v[2 * q]) | ((uint32_t)f2bf(v[2 * q + 1]) << 16);
+    *reinterpret_cast<uint4*>(static_cast<bf16_t*>(p) + i) = make_uint4(w[0], w[1], w[2], w[3]);
+  } else {
+    *reinterpret_cast<float4*>(static_cast<float*>(p) + i) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(static_cast<float*>(p) + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
+
+__device__ __forceinline__ void lion_one(float& x, float gin, float& m, const ScalarArgs& a) {
+  const float g = rnd(gin, a.m_dtype);
+  const float u0 = rnd(lerp_f(m, g, a.w1, a.m_dtype), a.m_dtype);
+  const float u = u0 > 0.f ? 1.f : (u0 < 0.f ? -1.f : u0);   // sign keeps 0 and NaN
+  m = rnd(lerp_f(m, g, a.w2, a.m_dtype), a.m_dtype);
+  const float xd = rnd(x * a.decay, a.x_dtype);
+  const float step = rnd(u * a.lr, a.m_dtype);
+  x = xd - step;   // rounded by the store
+}
+
+__device__ __forceinline__ void adamw_one(float& x, float gin, float& m, float& v, const ScalarArgs& a) {
+  const int d_dtype = (a.m_dtype == DA_F32 || a.v_dtype == DA_F32) ? DA_F32 : DA_BF16;
+  const float g = rnd(gin, a.m_dtype);
+  m = rnd(lerp_f(m, g, a.w1, a.m_dtype), a.m_dtype);
+  const float g2 = rnd(rnd(g * g, a.m_dtype), a.v_dtype);
+  v = rnd(lerp_f(v, g2, a.w2, a.v_dtype), a.v_dtype);
+  float den = rnd(sqrtf(v), a.v_dtype);
+  den = rnd(den / a.bc2_sqrt, a.v_dtype);
+  den = rnd(den + a.eps, a.v_dtype);
+  const float xd = rnd(x * a.decay, a.x_dtype);
+  float q = rnd(m / den, d_dtype);
+  q = rnd(q * a.lr, d_dtype);
+  x = xd - q;      // rounded by the store
+}
+
+template <bool ADAMW>
+__global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarArgs a) {
+  const int b = blockIdx.y;
+  void* X = t.x[b];
+  const void* G = t.g[b];
+  void* M = t.m[b];
+  void* V = ADAMW ? t.v[b] : nullptr;
+  const long long n = t.n[b];
+  const long long nvec = t.vec[b] ? n / 8 * 8 : 0;
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < nvec; i += stride * 8) {
+    float x[8], g[8], m[8], v[8];
+    ld8(X, a.x_dtype, i, x);
+    ld8(G, a.g_dtype, i, g);
+    ld8(M, a.m_dtype, i, m);
+    if (ADAMW) ld8(V, a.v_dtype, i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (ADAMW) adamw_one(x[e], g[e], m[e], v[e], a);
+      else lion_one(x[e], g[e], m[e], a);
+    }
+    st8(X, a.x_dtype, i, x);
+    st8(M, a.m_dtype, i, m);
+    if (ADAMW) st8(V, a.v_dtype, i, v);
+  }
+  // unaligned tensors entirely, aligned ones for their last n % 8 elements
+  for (long long i = nvec + (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    float x = ld1(X, a.x_dtype, i), m = ld1(M, a.m_dtype, i), v = ADAMW ? ld1(V, a.v_dtype, i) : 0.f;
+    const float g = ld1(G, a.g_dtype, i);
+    if (ADAMW) adamw_one(x, g, m, v, a);
+    else lion_one(x, g, m, a);
+    st1(X, a.x_dtype, i, x);
+    st1(M, a.m_dtype, i, m);
+    if (ADAMW) st1(V, a.v_dtype, i, v);
+  }
+}
+
+inline bool dtype_ok(int d) { return d == DA_BF16 || d == DA_F32; }
+inline size_t esize(int d) { return d == DA_BF16 ? 2 : 4; }
+
+int run(bool adamw, void* const* X, const void* const* G, void* const* M, void* const* V, const long long* numel,
+        int count, const ScalarArgs& a, hipStream_t s) {
+  if (!X || !G || !M || (adamw && !V) || !numel || count <= 0) return DA_ERR_ARG;
+  if (!dtype_ok(a.x_dtype) || !dtype_ok(a.g_dtype) || !dtype_ok(a.m_dtype) || (adamw && !dtype_ok(a.v_dtype)))
+    return DA_ERR_DTYPE;
+  for (int i = 0; i < count; ++i) {
+    if (!X[i] || !G[i] || !M[i] || (adamw && !V[i]) || numel[i] < 0) return DA_ERR_ARG;
+    // element alignment is the least a tensor of that dtype has
+    if (((uintptr_t)X[i] % esize(a.x_dtype)) || ((uintptr_t)G[i] % esize(a.g_dtype)) ||
+        ((uintptr_t)M[i] % esize(a.m_dtype)) || (adamw && ((uintptr_t)V[i] % esize(a.v_dtype))))
+      return DA_ERR_ALIGN;
+  }
+  for (int i0 = 0; i0 < count; i0 += MAX_TENSORS) {
+    const int c = count - i0 < MAX_TENSORS ? count - i0 : MAX_TENSORS;
+    ScalarTable t{};
+    long long longest = 0;
+    double bytes = 0.0;
+    for (int i = 0; i < c; ++i) {
+      t.x[i] = X[i0 + i];
+      t.g[i] = G[i0 + i];
+      t.m[i] = M[i0 + i];
+      t.v[i] = adamw ? V[i0 + i] : nullptr;
+      t.n[i] = numel[i0 + i];
+      const uintptr_t all = (uintptr_t)t.x[i] | (uintptr_t)t.g[i] | (uintptr_t)t.m[i] | (uintptr_t)t.v[i];
+      t.vec[i] = (all & 15) == 0;
+      if (t.n[i] > longest) longest = t.n[i];
+      // algorithmic bytes: read X, G, M (, V); write X, M (, V)
+      bytes += (double)t.n[i] * (2.0 * esize(a.x_dtype) + esize(a.g_dtype) + 2.0 * esize(a.m_dtype) +
+                                 (adamw ? 2.0 * esize(a.v_dtype) : 0.0));
+    }
+    if (longest == 0) continue;
+    long long bx = (longest / 8 + 255) / 256;
+    if (bx < 1) bx = 1;
+    if (bx > 2048) bx = 2048;
+    DaProfScope prof(DA_PROF_SCALAR_OPT, bytes, s);
+    if (adamw) hipLaunchKernelGGL(scalar_opt_kernel<true>, dim3((unsigned)bx, c), dim3(256), 0, s, t, a);
+    else hipLaunchKernelGGL(scalar_opt_kernel<false>, dim3((unsigned)bx, c), dim3(256), 0, s, t, a);
+    const int rc = da_launch_status();
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dion_amd_lion_step(void* const* X, const void* const* G, void* const* M, const long long* numel, int count,
+                       int x_dtype, int g_dtype, int m_dtype, float lr, float one_minus_beta1,
+                       float one_minus_beta2, float decay, void* stream) {
+  ScalarArgs a{};
+  a.w1 = one_minus_beta1; a.w2 = one_minus_beta2; a.decay = decay; a.lr = lr;
+  a.x_dtype = x_dtype; a.g_dtype = g_dtype; a.m_dtype = m_dtype; a.v_dtype = m_dtype;
+  return run(false, X, G, M, nullptr, numel, count, a, static_cast<hipStream_t>(stream));
+}
+
+int dion_amd_adamw_step(void* const* X, const void* const* G, void* const* M, void* const* V,
+                        const long long* numel, int count, int x_dtype, int g_dtype, int m_dtype, int v_dtype,
+                        float adjusted_lr, float one_minus_beta1, float one_minus_beta2, float decay,
+                        float bias_correction2_sqrt, float epsilon, void* stream) {
+  ScalarArgs a{};
+  a.w1 = one_minus_beta1; a.w2 = one_minus_beta2; a.decay = decay; a.lr = adjusted_lr;
+  a.bc2_sqrt = bias_correction2_sqrt; a.eps = epsilon;
+  a.x_dtype = x_dtype; a.g_dtype = g_dtype; a.m_dtype = m_dtype; a.v_dtype = v_dtype;
+  return run(true, X, G, M, V, numel, count, a, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

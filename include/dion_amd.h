@@ -146,6 +146,39 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
                                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Lion / AdamW for the non-matrix parameter groups (embeddings, lm_head, norms, biases)
+ * ------------------------------------------------------------------------------------- */
+
+/* Replaces lion_update_foreach (reference dion/scalar_opts.py:152-187; callers
+ * dion/muon.py:275-312, dion/dion.py:387-428): one fused in-place pass over `count` tensors.
+ * X, G, M: HOST arrays of `count` device pointers (weights, gradients, momentum); numel: HOST
+ * array of their lengths (any length; tensors whose pointers are 16-byte aligned move as
+ * vectors).  All X share x_dtype, all G g_dtype, all M m_dtype (bf16 or f32).  Per element,
+ * with the reference's rounding after every tensor op:
+ *   g = G.to(M.dtype); U = sign(lerp(M, g, 1-beta1)); M <- lerp(M, g, 1-beta2);
+ *   X <- X * decay; X <- X - U * lr.
+ * lr, one_minus_beta1/2 and decay = 1 - lr*weight_decay are passed as already-evaluated fp32
+ * values (the reference evaluates them on 0-dim fp32 tensors). */
+int dion_amd_lion_step(void* const* X, const void* const* G, void* const* M,
+                       const long long* numel, int count,
+                       int x_dtype, int g_dtype, int m_dtype,
+                       float lr, float one_minus_beta1, float one_minus_beta2, float decay,
+                       void* stream);
+
+/* Replaces adamw_update_foreach (reference dion/scalar_opts.py:89-149; callers
+ * dion/muon.py:314-353, dion/dion.py:430-473).  V: variance buffers (v_dtype).  Per element:
+ *   g = G.to(M.dtype); M <- lerp(M, g, 1-beta1); V <- lerp(V, (g*g).to(V.dtype), 1-beta2);
+ *   den = sqrt(V) / bias_correction2_sqrt + epsilon; X <- X * decay;
+ *   X <- X - (M / den) * adjusted_lr,
+ * with adjusted_lr = lr / (1 - beta1^step) and bias_correction2_sqrt = sqrt(1 - beta2^step)
+ * evaluated by the caller in fp32. */
+int dion_amd_adamw_step(void* const* X, const void* const* G, void* const* M, void* const* V,
+                        const long long* numel, int count,
+                        int x_dtype, int g_dtype, int m_dtype, int v_dtype,
+                        float adjusted_lr, float one_minus_beta1, float one_minus_beta2, float decay,
+                        float bias_correction2_sqrt, float epsilon, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Dion step for one bucket of same-shape matrices
  * ------------------------------------------------------------------------------------- */
 
@@ -205,7 +238,8 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
 #define DION_AMD_PROF_DION_UPD 10
 #define DION_AMD_PROF_DION_ORTH 11
 #define DION_AMD_PROF_DION_ELEM 12
-#define DION_AMD_PROF_KINDS 13
+#define DION_AMD_PROF_SCALAR_OPT 13
+#define DION_AMD_PROF_KINDS 14
 int dion_amd_profile_enable(int on);
 int dion_amd_profile_reset(void);
 /* Waits for the recorded events of `kind`; returns launch count, summed milliseconds and

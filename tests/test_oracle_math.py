@@ -168,3 +168,61 @@ def test_orthogonalize_variants_agree():
     wide = torch.randn(1, 16, 24)
     Qw = O.orthogonalize(wide)                 # rows <= cols: Householder branch
     assert (Qw[0].T @ Qw[0]).shape == (16, 16) or Qw.shape == (1, 16, 16)
+
+
+def test_scalar_opts_match_closed_forms():
+    """Lion / AdamW oracle (reference dion/scalar_opts.py:89-187) against the textbook forms in fp64."""
+    from oracle.scalar_opts import adamw_update_foreach, lion_update_foreach
+
+    torch.manual_seed(0)
+    x, g = torch.randn(50, dtype=torch.float64), torch.randn(50, dtype=torch.float64)
+    m, v = torch.randn(50, dtype=torch.float64) * 0.1, torch.rand(50, dtype=torch.float64) * 0.1
+    lr, b1, b2, wd, eps, step = 0.01, 0.9, 0.95, 0.1, 1e-8, 3
+    m1 = b1 * m + (1 - b1) * g
+    v1 = b2 * v + (1 - b2) * g * g
+    want = x * (1 - lr * wd) - lr * (m1 / (1 - b1**step)) / ((v1 / (1 - b2**step)).sqrt() + eps)
+    X, M, V = [x.clone()], [m.clone()], [v.clone()]
+    t = lambda z: torch.tensor(z, dtype=torch.float64)  # noqa: E731
+    adamw_update_foreach(X, [g], M, V, t(lr), t(b1), t(b2), t(wd), t(step), t(eps))
+    assert torch.allclose(X[0], want, rtol=1e-9) and torch.allclose(M[0], m1) and torch.allclose(V[0], v1)
+    want = x * (1 - lr * wd) - lr * torch.sign(b1 * m + (1 - b1) * g)
+    X, M = [x.clone()], [m.clone()]
+    lion_update_foreach(X, [g], M, t(lr), t(b1), t(b2), t(wd))
+    assert torch.allclose(X[0], want, rtol=1e-12) and torch.allclose(M[0], b2 * m + (1 - b2) * g)
+
+
+def test_scalar_opts_bf16_rounding_points():
+    """In bf16 every tensor op of the reference rounds once; the oracle must equal an fp32 evaluation of the same
+    sequence with an explicit bf16 rounding after each op (the 0-dim lerp weights 0.1 / 0.05 are cast to bf16 first
+    and use the `start + w*(end-start)` branch with a fused multiply-add, as ATen's kernel does)."""
+    from oracle.scalar_opts import adamw_update_foreach, lion_update_foreach
+
+    r = lambda z: z.to(torch.bfloat16).to(torch.float32)  # noqa: E731
+    torch.manual_seed(1)
+    n = 4096
+    x0, g0 = r(torch.randn(n)), r(torch.randn(n) * 0.1)
+    m0, v0 = r(torch.randn(n) * 0.1), r(torch.rand(n) * 0.01)
+    f = lambda z: torch.tensor(z, dtype=torch.float32)  # noqa: E731
+    lr, b1, b2, wd, eps, step = f(0.01), f(0.9), f(0.95), f(0.1), 1e-8, 2
+    w1, w2, decay = 1 - b1, 1 - b2, 1 - lr * wd
+
+    def lerp(s, e, w):
+        return r(torch.addcmul(s.double(), (e - s).double(), r(w).double()).float())  # one rounding of the fma in fp32
+
+    # Lion
+    u = torch.sign(lerp(m0, g0, w1))
+    m1 = lerp(m0, g0, w2)
+    x1 = r(r(x0 * decay) - r(u * lr))
+    X, M = [x0.bfloat16()], [m0.bfloat16()]
+    lion_update_foreach(X, [g0.bfloat16()], M, lr, b1, b2, wd)
+    assert torch.equal(M[0].float(), m1)
+    assert (X[0].float() != x1).float().mean() < 1e-3  # double-rounding ties of the fp64 stand-in for the fma
+    # AdamW
+    m1 = lerp(m0, g0, w1)
+    v1 = lerp(v0, r(g0 * g0), w2)
+    den = r(r(r(v1.sqrt()) / (1 - b2**step).sqrt()) + eps)
+    x1 = r(r(x0 * decay) - r(r(m1 / den) * (lr / (1 - b1**step))))
+    X, M, V = [x0.bfloat16()], [m0.bfloat16()], [v0.bfloat16()]
+    adamw_update_foreach(X, [g0.bfloat16()], M, V, lr, b1, b2, wd, step, eps)
+    assert torch.equal(M[0].float(), m1) and torch.equal(V[0].float(), v1)
+    assert (X[0].float() != x1).float().mean() < 1e-3
