@@ -192,7 +192,20 @@ def cpu_baseline(wl, budget_s=20.0):
 
     shapes = wl["shapes"]
     X, G = make_problem(shapes, wl["seed"], torch.bfloat16)
-    if wl["kind"] == "muon":
+    if wl["kind"] == "scalar":
+        from oracle import scalar_opts as O
+
+        M = [torch.zeros_like(x) for x in X]
+        V = [torch.zeros_like(X[1])]
+        t = torch.tensor
+        lion = [0] + list(range(2, len(X)))
+
+        def step():
+            O.lion_update_foreach([X[i] for i in lion], [G[i] for i in lion], [M[i] for i in lion],
+                                  t(0.01), t(0.9), t(0.95), t(0.01))
+            O.adamw_update_foreach([X[1]], [G[1]], [M[1]], V, t(0.01), t(0.9), t(0.95), t(0.01), t(1), t(1e-8))
+        what = "eager PyTorch CPU foreach ops, bf16"
+    elif wl["kind"] == "muon":
         from oracle import muon_step as O
 
         M = [torch.zeros_like(x) for x in X]

@@ -26,8 +26,12 @@ struct ScalarTable {
   void* m[MAX_TENSORS];
   void* v[MAX_TENSORS];
   long long n[MAX_TENSORS];
+  int first_block[MAX_TENSORS + 1]; // tensor i owns blocks first_block[i] .. first_block[i+1]-1
   unsigned char vec[MAX_TENSORS];   // 1: every pointer of the tensor is 16-byte aligned
+  int count;
 };
+
+constexpr int BLOCK_ELEMS = 256 * 8 * 4;   // elements per workgroup: four 8-element vectors per lane
 
 struct ScalarArgs {
   float w1, w2;        // 1 - beta1, 1 - beta2 (lerp weights)
@@ -56,30 +60,43 @@ __device__ __forceinline__ void st1(void* p, int dtype, long long i, float v) {
   if (dtype == DA_BF16) static_cast<bf16_t*>(p)[i] = f2bf(v);
   else static_cast<float*>(p)[i] = v;
 }
+// 8 elements per lane with non-temporal hints: every operand is touched once per step
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void ld8(const void* p, int dtype, long long i, float (&v)[8]) {
   if (dtype == DA_BF16) {
-    const uint4 r = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(p) + i);
-    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+    const u32x4_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(static_cast<const bf16_t*>(p) + i));
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       v[2 * q] = __builtin_bit_cast(float, w[q] << 16);
       v[2 * q + 1] = __builtin_bit_cast(float, w[q] & 0xffff0000u);
     }
   } else {
-    const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
-    const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i + 4);
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    const u32x4_t* src = reinterpret_cast<const u32x4_t*>(static_cast<const float*>(p) + i);
+    const u32x4_t a = __builtin_nontemporal_load(src), b = __builtin_nontemporal_load(src + 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const unsigned ua = a[q], ub = b[q];   // (bit_cast applied directly to a vector element reads element 0)
+      v[q] = __builtin_bit_cast(float, ua);
+      v[4 + q] = __builtin_bit_cast(float, ub);
+    }
   }
 }
 __device__ __forceinline__ void st8(void* p, int dtype, long long i, const float (&v)[8]) {
   if (dtype == DA_BF16) {
-    uint32_t w[4];
+    u32x4_t w;
 #pragma unroll
     for (int q = 0; q < 4; ++q) w[q] = (uint32_t)f2bf(v[2 * q]) | ((uint32_t)f2bf(v[2 * q + 1]) << 16);
-    *reinterpret_cast<uint4*>(static_cast<bf16_t*>(p) + i) = make_uint4(w[0], w[1], w[2], w[3]);
+    __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t*>(static_cast<bf16_t*>(p) + i));
   } else {
-    *reinterpret_cast<float4*>(static_cast<float*>(p) + i) = make_float4(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<float4*>(static_cast<float*>(p) + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    u32x4_t a, b;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      a[q] = __builtin_bit_cast(unsigned, v[q]);
+      b[q] = __builtin_bit_cast(unsigned, v[4 + q]);
+    }
+    u32x4_t* dst = reinterpret_cast<u32x4_t*>(static_cast<float*>(p) + i);
+    __builtin_nontemporal_store(a, dst);
+    __builtin_nontemporal_store(b, dst + 1);
   }
 }
 
@@ -110,15 +127,23 @@ __device__ __forceinline__ void adamw_one(float& x, float gin, float& m, float& 
 
 template <bool ADAMW>
 __global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarArgs a) {
-  const int b = blockIdx.y;
+  // which tensor this workgroup works on: bisection over the block ranges
+  int lo = 0, hi = t.count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int)blockIdx.x >= t.first_block[mid]) lo = mid; else hi = mid - 1;
+  }
+  const int b = lo;
   void* X = t.x[b];
   const void* G = t.g[b];
   void* M = t.m[b];
   void* V = ADAMW ? t.v[b] : nullptr;
   const long long n = t.n[b];
   const long long nvec = t.vec[b] ? n / 8 * 8 : 0;
-  const long long stride = (long long)gridDim.x * 256;
-  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < nvec; i += stride * 8) {
+  const long long begin = (long long)((int)blockIdx.x - t.first_block[b]) * BLOCK_ELEMS;
+  const long long end = begin + BLOCK_ELEMS < n ? begin + BLOCK_ELEMS : n;
+  const long long vend = end < nvec ? end : nvec;
+  for (long long i = begin + threadIdx.x * 8; i < vend; i += 256 * 8) {
     float x[8], g[8], m[8], v[8];
     ld8(X, a.x_dtype, i, x);
     ld8(G, a.g_dtype, i, g);
@@ -134,7 +159,7 @@ __global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarAr
     if (ADAMW) st8(V, a.v_dtype, i, v);
   }
   // unaligned tensors entirely, aligned ones for their last n % 8 elements
-  for (long long i = nvec + (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+  for (long long i = (begin > nvec ? begin : nvec) + threadIdx.x; i < end; i += 256) {
     float x = ld1(X, a.x_dtype, i), m = ld1(M, a.m_dtype, i), v = ADAMW ? ld1(V, a.v_dtype, i) : 0.f;
     const float g = ld1(G, a.g_dtype, i);
     if (ADAMW) adamw_one(x, g, m, v, a);
@@ -154,7 +179,9 @@ int run(bool adamw, void* const* X, const void* const* G, void* const* M, void* 
   if (!dtype_ok(a.x_dtype) || !dtype_ok(a.g_dtype) || !dtype_ok(a.m_dtype) || (adamw && !dtype_ok(a.v_dtype)))
     return DA_ERR_DTYPE;
   for (int i = 0; i < count; ++i) {
-    if (!X[i] || !G[i] || !M[i] || (adamw && !V[i]) || numel[i] < 0) return DA_ERR_ARG;
+    if (numel[i] < 0) return DA_ERR_ARG;
+    if (numel[i] == 0) continue;   // empty tensors may come without storage
+    if (!X[i] || !G[i] || !M[i] || (adamw && !V[i])) return DA_ERR_ARG;
     // element alignment is the least a tensor of that dtype has
     if (((uintptr_t)X[i] % esize(a.x_dtype)) || ((uintptr_t)G[i] % esize(a.g_dtype)) ||
         ((uintptr_t)M[i] % esize(a.m_dtype)) || (adamw && ((uintptr_t)V[i] % esize(a.v_dtype))))
@@ -163,28 +190,32 @@ int run(bool adamw, void* const* X, const void* const* G, void* const* M, void* 
   for (int i0 = 0; i0 < count; i0 += MAX_TENSORS) {
     const int c = count - i0 < MAX_TENSORS ? count - i0 : MAX_TENSORS;
     ScalarTable t{};
-    long long longest = 0;
+    long long blocks = 0;
     double bytes = 0.0;
+    int k = 0;
     for (int i = 0; i < c; ++i) {
-      t.x[i] = X[i0 + i];
-      t.g[i] = G[i0 + i];
-      t.m[i] = M[i0 + i];
-      t.v[i] = adamw ? V[i0 + i] : nullptr;
-      t.n[i] = numel[i0 + i];
-      const uintptr_t all = (uintptr_t)t.x[i] | (uintptr_t)t.g[i] | (uintptr_t)t.m[i] | (uintptr_t)t.v[i];
-      t.vec[i] = (all & 15) == 0;
-      if (t.n[i] > longest) longest = t.n[i];
+      if (numel[i0 + i] == 0) continue;
+      t.x[k] = X[i0 + i];
+      t.g[k] = G[i0 + i];
+      t.m[k] = M[i0 + i];
+      t.v[k] = adamw ? V[i0 + i] : nullptr;
+      t.n[k] = numel[i0 + i];
+      const uintptr_t all = (uintptr_t)t.x[k] | (uintptr_t)t.g[k] | (uintptr_t)t.m[k] | (uintptr_t)t.v[k];
+      t.vec[k] = (all & 15) == 0;
+      t.first_block[k] = (int)blocks;
+      blocks += (t.n[k] + BLOCK_ELEMS - 1) / BLOCK_ELEMS;
+      if (blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
       // algorithmic bytes: read X, G, M (, V); write X, M (, V)
-      bytes += (double)t.n[i] * (2.0 * esize(a.x_dtype) + esize(a.g_dtype) + 2.0 * esize(a.m_dtype) +
+      bytes += (double)t.n[k] * (2.0 * esize(a.x_dtype) + esize(a.g_dtype) + 2.0 * esize(a.m_dtype) +
                                  (adamw ? 2.0 * esize(a.v_dtype) : 0.0));
+      ++k;
     }
-    if (longest == 0) continue;
-    long long bx = (longest / 8 + 255) / 256;
-    if (bx < 1) bx = 1;
-    if (bx > 2048) bx = 2048;
+    if (k == 0) continue;
+    t.count = k;
+    for (int i = k; i <= MAX_TENSORS; ++i) t.first_block[i] = (int)blocks;
     DaProfScope prof(DA_PROF_SCALAR_OPT, bytes, s);
-    if (adamw) hipLaunchKernelGGL(scalar_opt_kernel<true>, dim3((unsigned)bx, c), dim3(256), 0, s, t, a);
-    else hipLaunchKernelGGL(scalar_opt_kernel<false>, dim3((unsigned)bx, c), dim3(256), 0, s, t, a);
+    if (adamw) hipLaunchKernelGGL(scalar_opt_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, t, a);
+    else hipLaunchKernelGGL(scalar_opt_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, t, a);
     const int rc = da_launch_status();
     if (rc) return rc;
   }
