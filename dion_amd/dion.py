@@ -154,6 +154,20 @@ class Dion(Optimizer):
         0 = success, k > 0 = pivot k-1 was not positive (the analogue of `torch.linalg.cholesky_ex`'s info)."""
         return dict(self._info)
 
+    def load_state_dict(self, state_dict):
+        """`Optimizer.load_state_dict` casts every floating-point state tensor to its parameter's dtype, which would
+        turn an fp32 `Q` or variance of bf16 weights into bf16.  The saved dtypes are those of the
+        `DionMixedPrecisionConfig` the state was created with (reference dion/dion.py:636-647, 684-688, 718), and a
+        checkpoint restore in the reference's trainer loads into the existing tensors and keeps them
+        (train.py:566-571): keep them here as well."""
+        super().load_state_dict(state_dict)
+        saved_ids = [i for g in state_dict["param_groups"] for i in g["params"]]
+        params = [p for g in self.param_groups for p in g["params"]]
+        for pid, p in zip(saved_ids, params):
+            for key, value in state_dict["state"].get(pid, {}).items():
+                if torch.is_tensor(value) and value.is_floating_point() and self.state[p][key].dtype != value.dtype:
+                    self.state[p][key] = value.detach().to(device=p.device, copy=True)
+
     # ------------------------------------------------------------------ state
     def _get_or_initialize_state(self, param: Tensor, group: dict) -> dict:
         state = self.state[param]
