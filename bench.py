@@ -5,10 +5,10 @@
 
 A "step" is one full optimizer step over every matrix of the workload, with synthetic
 Gaussian gradients already resident in HBM.  Prints ONE JSON line whose `value` is the
-milliseconds per step of the selected workload; the other BASELINE configurations that fit
+milliseconds per step of the selected workload; the other benchmark configurations that fit
 in a short run are reported under `extra`.
 
-Workloads (BASELINE.json `configs`):
+Workloads (numbered as the benchmark's configurations):
   muon_gpt_small        (default, configs[1]) full Muon step, GPT-small: 72 bf16 matrices
                         (48 x 768^2, 12 x 3072x768, 12 x 768x3072), G ~ N(0,1e-3) seed 1, Nesterov.
   dion_gpt_small_r025   (configs[2]) full Dion step on the same matrices, rank fraction 0.25,
@@ -161,7 +161,7 @@ def summarize(name, wl, res):
 
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.000 and
 # WRITE_SIZE x 1.000, in KiB, the factors being what the same counters read for a plain 512 MiB copy);
-# the summary of those runs is profiles/muon_gpt_small_hbm_traffic.md.  Keyed by (workload, kernel).
+# the runs used the default workload with three 512 MiB copies first (--calibrate-copy).  Keyed by (workload, kernel).
 MEASURED_TRAFFIC_BYTES = {("muon_gpt_small", "ns_axpy"): 683634 * 1024}
 
 

@@ -102,7 +102,7 @@ def _run_dion(dev, shapes, rank_fraction, steps, x_dtype, m_dtype, q_dtype, seed
     ([(512, 1024), (1024, 512), (256, 256)], 0.5),
 ])
 def test_dion_fp32_matches_oracle_10_steps(dev, shapes, rank_fraction):
-    """BASELINE config 3 (low rank) in all-fp32 state: M, Q (sign-aligned), X within 1e-4 after every step."""
+    """GPT-small Dion configuration (low rank) in all-fp32 state: M, Q (sign-aligned), X within 1e-4 after every step."""
     def check(step, params, opt, Xo, Mo, Qo):
         for i, p in enumerate(params):
             st = opt.state[p]
@@ -134,7 +134,7 @@ def test_dion_fp32_full_rank(dev):
 
 
 def test_dion_bf16_momentum(dev):
-    """BASELINE config 3/5 storage: bf16 weights and momentum, fp32 Q.  Every product rounds to bf16, so the
+    """Storage of the bf16 Dion configurations: bf16 weights and momentum, fp32 Q.  Every product rounds to bf16, so the
     bar is bf16-level (1e-2) on M and X; P's invariants are checked on the GPU result itself."""
     def check(step, params, opt, Xo, Mo, Qo):
         for i, p in enumerate(params):

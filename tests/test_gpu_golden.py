@@ -1,5 +1,5 @@
 """The HIP path against the golden vectors produced by the reference implementation itself
-(tests/golden/reference_vectors.npz), plus size-independent properties at the full BASELINE shapes."""
+(tests/golden/reference_vectors.npz), plus size-independent properties at the full benchmark shapes."""
 import os
 
 import numpy as np

@@ -39,7 +39,7 @@ def test_ns_bf16_schedule_vs_oracle(dev, m, n):
 
 
 def test_ns_config1_keller(dev):
-    """BASELINE config 1: one 768x3072 fp32 N(0,1) seed-0 matrix, Keller coefficients, eps 1e-7."""
+    """CPU-runnable configuration: one 768x3072 fp32 N(0,1) seed-0 matrix, Keller coefficients, eps 1e-7."""
     from dion_amd.newton_schulz import zeropower_via_newtonschulz5_keller
     from oracle import newton_schulz as O
 
@@ -92,7 +92,7 @@ def test_ns_batched_and_input_dtypes(dev):
 
 
 def test_ns_invariants_large(dev):
-    """Size-independent properties at a BASELINE shape too large for the CPU oracle in a test:
+    """Size-independent properties at a benchmark shape too large for the CPU oracle in a test:
     NS(G^T) = NS(G)^T, NS(2^k G) = NS(G) exactly, singular values pulled into ~[0.9, 1.1]."""
     from dion_amd import zeropower_via_newtonschulz5
 
