@@ -36,6 +36,24 @@ template <> struct Vec8<bf16_t> {
     for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(v[2 * i]) | ((uint32_t)f2bf(v[2 * i + 1]) << 16);
     *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  // streaming variants: data that is not touched again before it would fall out of the caches anyway
+  static __device__ __forceinline__ void load_nt(const bf16_t* p, float (&v)[8]) {
+    typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+    const u4_t w = __builtin_nontemporal_load(reinterpret_cast<const u4_t*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned x = w[i];
+      v[2 * i] = __builtin_bit_cast(float, x << 16);
+      v[2 * i + 1] = __builtin_bit_cast(float, x & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store_nt(bf16_t* p, const float (&v)[8]) {
+    typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+    u4_t w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f2bf(v[2 * i]) | ((uint32_t)f2bf(v[2 * i + 1]) << 16);
+    __builtin_nontemporal_store(w, reinterpret_cast<u4_t*>(p));
+  }
   static __device__ __forceinline__ float round(float x) { return rbf(x); }
 };
 template <> struct Vec8<float> {
@@ -48,6 +66,23 @@ template <> struct Vec8<float> {
   static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
     *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+  static __device__ __forceinline__ void load_nt(const float* p, float (&v)[8]) {
+    typedef float f4_t __attribute__((ext_vector_type(4)));
+    const f4_t a = __builtin_nontemporal_load(reinterpret_cast<const f4_t*>(p));
+    const f4_t b = __builtin_nontemporal_load(reinterpret_cast<const f4_t*>(p) + 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float x = a[i], y = b[i];
+      v[i] = x;
+      v[4 + i] = y;
+    }
+  }
+  static __device__ __forceinline__ void store_nt(float* p, const float (&v)[8]) {
+    typedef float f4_t __attribute__((ext_vector_type(4)));
+    const f4_t a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+    __builtin_nontemporal_store(a, reinterpret_cast<f4_t*>(p));
+    __builtin_nontemporal_store(b, reinterpret_cast<f4_t*>(p) + 1);
   }
   static __device__ __forceinline__ float round(float x) { return x; }
 };
@@ -106,10 +141,10 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
     const bool ok = i < a.rows && j < a.cols;  // cols is a multiple of 8
     if (ok) {
       float g[8];
-      Vec8<TG>::load(G + (long long)i * a.ld + j, g);
+      Vec8<TG>::load_nt(G + (long long)i * a.ld + j, g);
       if (a.muon) {
         float m[8];
-        Vec8<TM>::load(M + (long long)i * a.cols + j, m);
+        Vec8<TM>::load_nt(M + (long long)i * a.cols + j, m);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float ge = Vec8<TM>::round(g[e]);                 // G.to(M.dtype)
@@ -120,7 +155,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
           if (a.nesterov) ue = Vec8<TM>::round(Vec8<TM>::round(me * a.mu) + ge);  // U = M*mu; U += G
           u[e] = Vec8<TW>::round(ue);                             // U.to(bf16)
         }
-        Vec8<TM>::store(M + (long long)i * a.cols + j, m);
+        Vec8<TM>::store_nt(M + (long long)i * a.cols + j, m);
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) u[e] = Vec8<TW>::round(g[e]);
@@ -253,14 +288,14 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
     TX* xp = X + (long long)i * a.ld + j;
     if (a.muon) {
       float x[8];
-      Vec8<TX>::load(xp, x);
+      Vec8<TX>::load_nt(xp, x);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float xd = Vec8<TX>::round(x[e] * a.decay);    // X *= 1 - lr*wd
         const float t = Vec8<TW>::round(u[e] * a.step);      // U * adjusted_lr (U's dtype)
         x[e] = xd - t;                                       // X -= U ; rounded by the store
       }
-      Vec8<TX>::store(xp, x);
+      Vec8<TX>::store_nt(xp, x);
     } else {
       Vec8<TX>::store(xp, u);
     }
