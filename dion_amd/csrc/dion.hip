@@ -262,79 +262,115 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 // CholeskyQR2 in fp64
 // ---------------------------------------------------------------------------------------
 size_t da_orth_workspace_bytes(int batch, int rows, int r) {
-  size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place
-               + 3 * (size_t)r * r * 8;   // G, L, W
+  size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place (first pass)
+               + 3 * (size_t)r * r * 8    // G, L, W (fp64; reused in fp32 by the later passes)
+               + (size_t)rows * r * 4;    // P in fp32 (later passes)
   return per * batch + 256;
 }
 
-int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
-                      int* info, hipStream_t s) {
+namespace {
+
+inline int chol_step_any(const double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info,
+                         int batch, hipStream_t s) { return da_chol_step(G, L, W, sG, r, o, nb, info, batch, s); }
+inline int chol_step_any(const float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info,
+                         int batch, hipStream_t s) { return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, s); }
+inline int gemm_any_real(const Gemm64Desc& d, hipStream_t s) { return da_gemm_f64(d, s); }
+inline int gemm_any_real(const Gemm32Desc& d, hipStream_t s) { return da_gemm_f32s(d, s); }
+inline int fill_any(double* p, long long n, hipStream_t s) { return da_fill_f64(p, n, 0.0, s); }
+inline int fill_any(float* p, long long n, hipStream_t s) { return da_fill_f32(p, n, 0.f, s); }
+
+// One CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
+template <typename T>
+int cholqr_pass(T* P0, T* G, T* L, T* W, int batch, int rows, int r, int* info, hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  RealGemmDesc<T> g{};
+  g.batch = batch;
+  // G = P0^T P0
+  g.A = P0; g.B = P0; g.C = G; g.E = nullptr;
+  g.sA = pr; g.sB = pr; g.sC = rr;
+  g.lda = r; g.ldb = r; g.ldc = r;
+  g.M = r; g.N = r; g.K = rows;
+  g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
+  int rc;
+  {
+    // few output tiles, long K: slice K until ~512 workgroups exist
+    const int t = (r + 63) / 64;
+    const long long blocks = (long long)t * (t + 1) / 2 * batch;
+    int split = (int)((512 + blocks - 1) / blocks);
+    const int max_split = rows / 256 > 0 ? rows / 256 : 1;
+    if (split > max_split) split = max_split;
+    g.split_k = split;
+    if (split > 1) {
+      rc = fill_any(G, rr * batch, s);
+      if (rc) return rc;
+    }
+  }
+  rc = gemm_any_real(g, s);
+  if (rc) return rc;
+  // blocked lower Cholesky G = L L^T (right-looking), building W alongside
+  for (int j = 0; j < nblk; ++j) {
+    const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
+    rc = chol_step_any(G, L, W, rr, r, o, nb, info, batch, s);
+    if (rc) return rc;
+    if (rest <= 0) break;
+    // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
+    RealGemmDesc<T> u{};
+    u.batch = batch;
+    u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
+    u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+    u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
+    u.E = u.C; u.sE = rr; u.lde = r;
+    u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
+    rc = gemm_any_real(u, s);
+    if (rc) return rc;
+  }
+  // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
+  //   P0[:, j] <- P0[:, 0 .. j] W[j, 0 .. j]^T
+  // (each workgroup owns 64 rows and the one 64-column output tile, and has read all it needs of
+  // those rows before it stores)
+  for (int j = 0; j < nblk; ++j) {
+    const int o = j * NB, nb = r - o < NB ? r - o : NB;
+    RealGemmDesc<T> a{};
+    a.batch = batch;
+    a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+    a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
+    a.C = P0 + o; a.sC = pr; a.ldc = r;
+    a.E = nullptr;
+    a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
+    rc = gemm_any_real(a, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+}  // namespace
+
+// The first pass runs in fp64: the Gram matrix squares P's condition number (up to 4e12 on the
+// optimizer's inputs).  Its result is orthonormal to about eps64 * cond(P)^2 <= 1e-4, so the later
+// passes, which only polish it, run in fp32 -- twice the MFMA rate, half the bytes, and a serial
+// Cholesky chain of half the latency -- and still end at fp32 round-off, which is also all the
+// output dtype (fp32 or bf16) can hold.
+int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
+                      int* info, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   double* P0 = static_cast<double*>(ws);
   double* G = P0 + pr * batch;
   double* L = G + rr * batch;
   double* W = L + rr * batch;
+  float* P0f = reinterpret_cast<float*>(W + rr * batch);
   int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
   if (rc) return rc;
-  for (int pass = 0; pass < passes; ++pass) {
-    Gemm64Desc g{};
-    g.batch = batch;
-    // G = P0^T P0
-    g.A = P0; g.B = P0; g.C = G; g.E = nullptr;
-    g.sA = pr; g.sB = pr; g.sC = rr;
-    g.lda = r; g.ldb = r; g.ldc = r;
-    g.M = r; g.N = r; g.K = rows;
-    g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
-    {
-      // few output tiles, long K: slice K until ~512 workgroups exist
-      const int t = (r + 63) / 64;
-      const long long blocks = (long long)t * (t + 1) / 2 * batch;
-      int split = (int)((512 + blocks - 1) / blocks);
-      const int max_split = rows / 256 > 0 ? rows / 256 : 1;
-      if (split > max_split) split = max_split;
-      g.split_k = split;
-      if (split > 1) {
-        rc = da_fill_f64(G, rr * batch, 0.0, s);
-        if (rc) return rc;
-      }
-    }
-    rc = da_gemm_f64(g, s);
+  rc = cholqr_pass<double>(P0, G, L, W, batch, rows, r, info, s);
+  if (rc) return rc;
+  if (passes <= 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+  rc = da_cvt_f64_to_f32(P0, P0f, pr * batch, s);
+  if (rc) return rc;
+  for (int pass = 1; pass < passes; ++pass) {
+    rc = cholqr_pass<float>(P0f, reinterpret_cast<float*>(G), reinterpret_cast<float*>(L), reinterpret_cast<float*>(W),
+                            batch, rows, r, info, s);
     if (rc) return rc;
-    // blocked lower Cholesky G = L L^T (right-looking), building W alongside
-    for (int j = 0; j < nblk; ++j) {
-      const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-      rc = da_chol_step(G, L, W, rr, r, o, nb, info, batch, s);
-      if (rc) return rc;
-      if (rest <= 0) break;
-      // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
-      Gemm64Desc u{};
-      u.batch = batch;
-      u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
-      u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
-      u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
-      u.E = u.C; u.sE = rr; u.lde = r;
-      u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
-      rc = da_gemm_f64(u, s);
-      if (rc) return rc;
-    }
-    // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
-    //   P0[:, j] <- P0[:, 0 .. j] W[j, 0 .. j]^T
-    // (each workgroup owns 64 rows and the one 64-column output tile, and has read all it needs of
-    // those rows before it stores)
-    for (int j = 0; j < nblk; ++j) {
-      const int o = j * NB, nb = r - o < NB ? r - o : NB;
-      Gemm64Desc a{};
-      a.batch = batch;
-      a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
-      a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
-      a.C = P0 + o; a.sC = pr; a.ldc = r;
-      a.E = nullptr;
-      a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
-      rc = da_gemm_f64(a, s);
-      if (rc) return rc;
-    }
   }
-  return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+  return da_cvt_from_f32(P0f, out, dtype, pr * batch, s);
 }

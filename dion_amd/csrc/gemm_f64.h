@@ -2,13 +2,14 @@
 #pragma once
 #include "common.h"
 
-// C[b] (M x N) = alpha * sum_k Aop[b](i,k) Bop[b](j,k) + beta * E[b]   (all fp64, row-major)
+// C[b] (M x N) = alpha * sum_k Aop[b](i,k) Bop[b](j,k) + beta * E[b]   (all of one real type, row-major)
 // Operand layouts as in GemmDesc.  E may alias C.  K == 0 is allowed (C = beta * E).
-struct Gemm64Desc {
-  const double* A;
-  const double* B;
-  double* C;
-  const double* E;
+template <typename T>
+struct RealGemmDesc {
+  const T* A;
+  const T* B;
+  T* C;
+  const T* E;
   long long sA, sB, sC, sE;
   int lda, ldb, ldc, lde;
   int M, N, K, batch;
@@ -18,7 +19,16 @@ struct Gemm64Desc {
   int split_k;   // > 1: K is cut into that many slices whose partial products are added atomically into a
                  // zeroed C (no E term); the summation order, and so the last bits, vary run to run
 };
+typedef RealGemmDesc<double> Gemm64Desc;
+typedef RealGemmDesc<float> Gemm32Desc;
 
+// The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the second CholeskyQR pass, whose input is already
+// orthonormal to 1e-4 or better, does not need fp64.
+int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s);
+int da_fill_f32(float* p, long long n, float v, hipStream_t s);
+int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s);
+int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long n, hipStream_t s);
+int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long n, hipStream_t s);
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
 int da_fill_f64(double* p, long long n, double v, hipStream_t s);
 
@@ -34,5 +44,26 @@ int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hi
 // L_jj and of D_j) and records (o + column + 1) in info[b] if it is the matrix's first failure.
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
                  int batch, hipStream_t s);
+int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
+                     int batch, hipStream_t s);
 
 #define DA_CHOL_NB 64
+
+// The 16 x 16 x 4 MFMA of either precision: operands are one scalar per lane (A: row = lane % 16,
+// k = lane / 16; B: k = lane / 16, column = lane % 16); the four results of a lane are in column
+// lane % 16 and rows 4 v + lane / 16 (fp64) resp. 4 (lane / 16) + v (fp32).
+template <typename T> struct Mfma;
+template <> struct Mfma<double> {
+  typedef f64x4_t acc_t;
+  static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int v, int lane) { return 4 * v + (lane >> 4); }
+};
+template <> struct Mfma<float> {
+  typedef f32x4_t acc_t;
+  static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int v, int lane) { return 4 * (lane >> 4) + v; }
+};
+
+// One 64 x 16 operand tile: 4 elements per thread, fetched into registers (zero filled out of
+// range) and later written to lds[k][row].
+

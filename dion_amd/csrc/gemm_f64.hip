@@ -16,28 +16,27 @@ namespace {
 constexpr int BT = 64;
 constexpr int BK = 16;
 
-// One 64 x 16 operand tile: 4 elements per thread, fetched into registers (zero filled out of
-// range) and later written to lds[k][row].
-template <bool KS>
-__device__ __forceinline__ void fetch(double (&v)[4], const double* __restrict__ base, int ld, int row0, int k0,
+template <bool KS, typename T>
+__device__ __forceinline__ void fetch(T (&v)[4], const T* __restrict__ base, int ld, int row0, int k0,
                                       int rows, int K, int tid) {
   // the thread's 4 elements are contiguous in memory in either layout
   const int outer = KS ? k0 + (tid >> 4) : row0 + (tid >> 2);
   const int inner = KS ? row0 + (tid & 15) * 4 : k0 + (tid & 3) * 4;
   const int outer_n = KS ? K : rows, inner_n = KS ? rows : K;
-  const double* p = base + (long long)outer * ld + inner;
+  const T* p = base + (long long)outer * ld + inner;
   if (outer < outer_n && inner + 3 < inner_n && ((reinterpret_cast<uintptr_t>(p) & 15) == 0)) {
-    const double2 lo = *reinterpret_cast<const double2*>(p);
-    const double2 hi = *reinterpret_cast<const double2*>(p + 2);
+    typedef T pair_t __attribute__((ext_vector_type(2)));   // 16 bytes (fp64) / 8 bytes (fp32) per access
+    const pair_t lo = *reinterpret_cast<const pair_t*>(p);
+    const pair_t hi = *reinterpret_cast<const pair_t*>(p + 2);
     v[0] = lo.x; v[1] = lo.y; v[2] = hi.x; v[3] = hi.y;
   } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = (outer < outer_n && inner + e < inner_n) ? p[e] : 0.0;
+    for (int e = 0; e < 4; ++e) v[e] = (outer < outer_n && inner + e < inner_n) ? p[e] : T(0);
   }
 }
 
-template <bool KS>
-__device__ __forceinline__ void put(double* lds, const double (&v)[4], int tid) {
+template <bool KS, typename T>
+__device__ __forceinline__ void put(T* lds, const T (&v)[4], int tid) {
   if (!KS) {
     const int r = tid >> 2, k4 = (tid & 3) * 4;
 #pragma unroll
@@ -49,10 +48,11 @@ __device__ __forceinline__ void put(double* lds, const double (&v)[4], int tid) 
   }
 }
 
-template <bool A_KS, bool B_KS, bool SYM>
-__global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
-  __shared__ double lds_a[2][BK * BT];
-  __shared__ double lds_b[2][BK * BT];
+template <typename T, bool A_KS, bool B_KS, bool SYM>
+__global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
+  typedef typename Mfma<T>::acc_t acc_t;
+  __shared__ T lds_a[2][BK * BT];
+  __shared__ T lds_b[2][BK * BT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
@@ -73,21 +73,21 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
     tj = t - ti * tiles_n;
   }
   const int m0 = ti * BT, n0 = tj * BT;
-  const double* A = d.A + (long long)b * d.sA;
-  const double* B = d.B + (long long)b * d.sB;
+  const T* A = d.A + (long long)b * d.sA;
+  const T* B = d.B + (long long)b * d.sB;
 
-  f64x4_t acc[2][2];
+  acc_t acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+    for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
   // double buffered: the global loads of stage s+1 are in flight while stage s is multiplied
   const int KT_all = (d.K + BK - 1) / BK;
   const int per_split = (KT_all + (int)gridDim.y - 1) / (int)gridDim.y;
   const int kt0 = split * per_split;
   const int KT = KT_all - kt0 < per_split ? KT_all - kt0 : per_split;   // may be <= 0 for the last slices
-  double pa[4], pb[4];
+  T pa[4], pb[4];
   if (KT > 0) {
     fetch<A_KS>(pa, A, d.lda, m0, kt0 * BK, d.M, d.K, tid);
     fetch<B_KS>(pb, B, d.ldb, n0, kt0 * BK, d.N, d.K, tid);
@@ -96,8 +96,8 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
   }
   __syncthreads();
   for (int kt = 0; kt < KT; ++kt) {
-    const double* sa = lds_a[kt & 1];
-    const double* sb = lds_b[kt & 1];
+    const T* sa = lds_a[kt & 1];
+    const T* sb = lds_b[kt & 1];
     const bool more = kt + 1 < KT;
     if (more) {
       fetch<A_KS>(pa, A, d.lda, m0, (kt0 + kt + 1) * BK, d.M, d.K, tid);
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       const int k = ks * 4 + (lane >> 4);
-      double af[2], bfv[2];
+      T af[2], bfv[2];
 #pragma unroll
       for (int i = 0; i < 2; ++i) af[i] = sa[k * BT + wm * 32 + i * 16 + (lane & 15)];
 #pragma unroll
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[i], bfv[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
     }
     if (more) {
       put<A_KS>(lds_a[(kt + 1) & 1], pa, tid);
@@ -123,9 +123,8 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
     __syncthreads();
   }
 
-  // D layout: lane l, register v -> row 4 v + (l >> 4), column (l & 15)
-  double* C = d.C + (long long)b * d.sC;
-  const double* E = d.E ? d.E + (long long)b * d.sE : nullptr;
+  T* C = d.C + (long long)b * d.sC;
+  const T* E = d.E ? d.E + (long long)b * d.sE : nullptr;
   const bool mirror = SYM && (ti != tj);
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -133,15 +132,15 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int m = m0 + wm * 32 + i * 16 + v * 4 + (lane >> 4);
+        const int m = m0 + wm * 32 + i * 16 + Mfma<T>::row(v, lane);
         const int n = n0 + wn * 32 + j * 16 + (lane & 15);
         if (m < d.M && n < d.N) {
-          double o = d.alpha * acc[i][j][v];
+          T o = (T)d.alpha * acc[i][j][v];
           if (gridDim.y > 1) {  // split-K: partial sums meet in a zeroed C
             atomicAdd(C + (long long)m * d.ldc + n, o);
             if (mirror) atomicAdd(C + (long long)n * d.ldc + m, o);
           } else {
-            if (E) o += d.beta * E[(long long)m * d.lde + n];
+            if (E) o += (T)d.beta * E[(long long)m * d.lde + n];
             C[(long long)m * d.ldc + n] = o;
             if (mirror) C[(long long)n * d.ldc + m] = o;
           }
@@ -149,33 +148,40 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(Gemm64Desc d) {
       }
 }
 
-template <bool A_KS, bool B_KS, bool SYM>
-int launch(const Gemm64Desc& d, hipStream_t s) {
+template <typename T, bool A_KS, bool B_KS, bool SYM>
+int launch(const RealGemmDesc<T>& d, hipStream_t s) {
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
   const long long per_batch = (SYM || d.lower_only) ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
   const long long blocks = per_batch * d.batch;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
   int split = d.split_k > 1 ? d.split_k : 1;
   if (d.E) split = 1;
-  hipLaunchKernelGGL((gemm_f64_kernel<A_KS, B_KS, SYM>), dim3((unsigned)blocks, split), dim3(256), 0, s, d);
+  hipLaunchKernelGGL((gemm_f64_kernel<T, A_KS, B_KS, SYM>), dim3((unsigned)blocks, split), dim3(256), 0, s, d);
   return da_launch_status();
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void cvt_to_f64_kernel(const T* __restrict__ src, double* __restrict__ dst,
+template <typename T, typename R>
+__global__ __launch_bounds__(256) void cvt_to_f64_kernel(const T* __restrict__ src, R* __restrict__ dst,
                                                          long long n) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
-    dst[i] = (double)ld_as_float<T>(src + i);
+    dst[i] = (R)ld_as_float<T>(src + i);
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void cvt_from_f64_kernel(const double* __restrict__ src, T* __restrict__ dst,
+template <typename T, typename R>
+__global__ __launch_bounds__(256) void cvt_from_f64_kernel(const R* __restrict__ src, T* __restrict__ dst,
                                                            long long n) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
     st_from_float<T>(dst + i, (float)src[i]);
 }
 
-__global__ void fill_f64_kernel(double* p, long long n, double v) {
+__global__ __launch_bounds__(256) void cvt_f64_to_f32_kernel(const double* __restrict__ src, float* __restrict__ dst,
+                                                              long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    dst[i] = (float)src[i];
+}
+
+template <typename R>
+__global__ void fill_f64_kernel(R* p, long long n, R v) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
 }
@@ -185,45 +191,66 @@ inline unsigned cvt_blocks(long long n) {
   return (unsigned)(b > 8192 ? 8192 : (b < 1 ? 1 : b));
 }
 
-}  // namespace
-
-int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) {
+template <typename T>
+int gemm_real(const RealGemmDesc<T>& d, hipStream_t s) {
   if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K < 0 || d.batch <= 0) return DA_ERR_ARG;
   if (d.lower_only && (d.M != d.N || d.symmetric)) return DA_ERR_ARG;
   if (d.symmetric) {
     if (d.M != d.N || !d.a_kstrided || !d.b_kstrided) return DA_ERR_ARG;  // only the Gram form A^T A
-    return launch<true, true, true>(d, s);
+    return launch<T, true, true, true>(d, s);
   }
-  if (!d.a_kstrided && !d.b_kstrided) return launch<false, false, false>(d, s);
-  if (!d.a_kstrided && d.b_kstrided) return launch<false, true, false>(d, s);
-  if (d.a_kstrided && !d.b_kstrided) return launch<true, false, false>(d, s);
-  return launch<true, true, false>(d, s);
+  if (!d.a_kstrided && !d.b_kstrided) return launch<T, false, false, false>(d, s);
+  if (!d.a_kstrided && d.b_kstrided) return launch<T, false, true, false>(d, s);
+  if (d.a_kstrided && !d.b_kstrided) return launch<T, true, false, false>(d, s);
+  return launch<T, true, true, false>(d, s);
 }
+
+template <typename R>
+int cvt_to(const void* src, int src_dtype, R* dst, long long n, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  if (src_dtype == DA_BF16)
+    hipLaunchKernelGGL((cvt_to_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n);
+  else if (src_dtype == DA_F32)
+    hipLaunchKernelGGL((cvt_to_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+template <typename R>
+int cvt_from(const R* src, void* dst, int dst_dtype, long long n, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  if (dst_dtype == DA_BF16)
+    hipLaunchKernelGGL((cvt_from_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
+  else if (dst_dtype == DA_F32)
+    hipLaunchKernelGGL((cvt_from_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<float*>(dst), n);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
+}  // namespace
+
+int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) { return gemm_real<double>(d, s); }
+int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s) { return gemm_real<float>(d, s); }
 
 int da_fill_f64(double* p, long long n, double v, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
+  hipLaunchKernelGGL(fill_f64_kernel<double>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
+  return da_launch_status();
+}
+int da_fill_f32(float* p, long long n, float v, hipStream_t s) {
+  if (n <= 0) return DA_ERR_ARG;
+  hipLaunchKernelGGL(fill_f64_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
   return da_launch_status();
 }
 
-int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) {
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) { return cvt_to<double>(src, src_dtype, dst, n, s); }
+int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<double>(src, dst, dst_dtype, n, s); }
+int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long n, hipStream_t s) { return cvt_to<float>(src, src_dtype, dst, n, s); }
+int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<float>(src, dst, dst_dtype, n, s); }
+int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
-  if (src_dtype == DA_BF16)
-    hipLaunchKernelGGL(cvt_to_f64_kernel<bf16_t>, dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n);
-  else if (src_dtype == DA_F32)
-    hipLaunchKernelGGL(cvt_to_f64_kernel<float>, dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n);
-  else
-    return DA_ERR_DTYPE;
-  return da_launch_status();
-}
-
-int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
-  if (dst_dtype == DA_BF16)
-    hipLaunchKernelGGL(cvt_from_f64_kernel<bf16_t>, dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
-  else if (dst_dtype == DA_F32)
-    hipLaunchKernelGGL(cvt_from_f64_kernel<float>, dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<float*>(dst), n);
-  else
-    return DA_ERR_DTYPE;
+  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, n);
   return da_launch_status();
 }
