@@ -140,3 +140,16 @@ def test_dion_constructor_contract():
         bad.step()
 
 
+
+
+def test_reference_import_paths_exist():
+    """The reference exposes the orthogonalisation under three module paths (dion/muon.py:620,
+    dion/newton_schulz_triton.py:305-337, dion/muon_reference.py:10); the same names import here."""
+    import inspect
+
+    from dion_amd import muon, muon_reference, newton_schulz_triton as nst
+    assert list(inspect.signature(muon.zeropower_via_newtonschulz5).parameters) == ["G", "epsilon"]
+    assert list(inspect.signature(nst.zeropower_via_newtonschulz5).parameters) == ["G", "epsilon"]
+    assert list(inspect.signature(nst.newton_schulz_triton).parameters) == ["G", "epsilon"]
+    assert list(inspect.signature(muon_reference.zeropower_via_newtonschulz5).parameters) == ["G", "steps", "eps"]
+    assert callable(nst.ns_line_1) and callable(nst.ns_line_2)

@@ -111,3 +111,28 @@ def test_ns_zero_matrix(dev):
     Z = torch.zeros(256, 512, device=dev)
     out = zeropower_via_newtonschulz5(Z)
     assert torch.count_nonzero(out) == 0 and torch.isfinite(out.float()).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n", [(256, 256), (256, 1024)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_newton_schulz_triton_matches_eager_rounding(dev, m, n, dtype):
+    """The reference's own relational test (tests/test_newton_shultz.py:77-88): the fused-epilogue variant against
+    the op-by-op variant, atol = rtol = 5e-2, 2-D and batch of 4, through the reference's import path."""
+    from dion_amd.newton_schulz_triton import newton_schulz_triton, zeropower_via_newtonschulz5
+    g = torch.Generator().manual_seed(11)
+    for shape in ((m, n), (4, m, n)):
+        G = torch.randn(*shape, generator=g).to(dtype).to(dev)
+        a, b = newton_schulz_triton(G), zeropower_via_newtonschulz5(G)
+        assert a.dtype == b.dtype == torch.bfloat16 and a.shape == b.shape == G.shape
+        assert torch.allclose(a.float(), b.float(), atol=5e-2, rtol=5e-2), (a.float() - b.float()).abs().max()
+
+
+@pytest.mark.gpu
+def test_muon_reference_import_path(dev):
+    from dion_amd.muon_reference import zeropower_via_newtonschulz5 as keller
+    from dion_amd.newton_schulz import NS_KELLER_COEFFS, newton_schulz
+    G = torch.randn(128, 256, generator=torch.Generator().manual_seed(12)).to(dev)
+    assert torch.equal(keller(G, steps=3), newton_schulz(G, epsilon=1e-7, coeffs=(NS_KELLER_COEFFS,) * 3))
+    with pytest.raises(AssertionError):
+        keller(G.unsqueeze(0))
