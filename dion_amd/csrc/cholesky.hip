@@ -293,7 +293,3 @@ int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int 
                  int batch, hipStream_t s) {
   return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, s);
 }
-int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
-                     int batch, hipStream_t s) {
-  return chol_step<float>(G, Lmat, Wmat, sG, r, o, nb, info, batch, s);
-}

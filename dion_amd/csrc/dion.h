@@ -14,8 +14,9 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
                int batch, double* sums, hipStream_t s);
 
 // CholeskyQR (passes = 1) / CholeskyQR2 (passes = 2) of `batch` contiguous matrices P[b]
-// (rows x r, dtype bf16 or f32) with fp64 Gram, Cholesky and triangular solve; result in
-// `out` (same dtype and layout, may alias P).  info[b] receives 1 + the first failed pivot
+// (rows x r, dtype bf16 or f32): one pass with fp64 Gram, Cholesky and triangular solve, then
+// passes - 1 first-order polishing passes in fp32; result in `out` (same dtype and layout, may
+// alias P).  info[b] receives 1 + the first failed pivot
 // column (0 = success); failed columns come out as zeros.
 size_t da_orth_workspace_bytes(int batch, int rows, int r);
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,

@@ -263,29 +263,19 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 // ---------------------------------------------------------------------------------------
 size_t da_orth_workspace_bytes(int batch, int rows, int r) {
   size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place (first pass)
-               + 3 * (size_t)r * r * 8    // G, L, W (fp64; reused in fp32 by the later passes)
-               + (size_t)rows * r * 4;    // P in fp32 (later passes)
+               + 3 * (size_t)r * r * 8    // G, L, W (fp64; the polishing passes keep their fp32 G and V there)
+               + (size_t)rows * r * 4;    // fp32 iterate between polishing passes (three or more passes)
   return per * batch + 256;
 }
 
 namespace {
 
-inline int chol_step_any(const double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info,
-                         int batch, hipStream_t s) { return da_chol_step(G, L, W, sG, r, o, nb, info, batch, s); }
-inline int chol_step_any(const float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info,
-                         int batch, hipStream_t s) { return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, s); }
-inline int gemm_any_real(const Gemm64Desc& d, hipStream_t s) { return da_gemm_f64(d, s); }
-inline int gemm_any_real(const Gemm32Desc& d, hipStream_t s) { return da_gemm_f32s(d, s); }
-inline int fill_any(double* p, long long n, hipStream_t s) { return da_fill_f64(p, n, 0.0, s); }
-inline int fill_any(float* p, long long n, hipStream_t s) { return da_fill_f32(p, n, 0.f, s); }
-
-// One CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
-template <typename T>
-int cholqr_pass(T* P0, T* G, T* L, T* W, int batch, int rows, int r, int* info, hipStream_t s) {
+// One blocked CholeskyQR pass in fp64, in place:  P <- P R^-1  with  P^T P = R^T R.
+int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int* info, hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
-  RealGemmDesc<T> g{};
+  Gemm64Desc g{};
   g.batch = batch;
   // G = P0^T P0
   g.A = P0; g.B = P0; g.C = G; g.E = nullptr;
@@ -293,37 +283,24 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, int batch, int rows, int r, int* info, 
   g.lda = r; g.ldb = r; g.ldc = r;
   g.M = r; g.N = r; g.K = rows;
   g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
-  int rc;
-  {
-    // few output tiles, long K: slice K until ~512 workgroups exist
-    const int t = (r + 63) / 64;
-    const long long blocks = (long long)t * (t + 1) / 2 * batch;
-    int split = (int)((512 + blocks - 1) / blocks);
-    const int max_split = rows / 256 > 0 ? rows / 256 : 1;
-    if (split > max_split) split = max_split;
-    g.split_k = split;
-    if (split > 1) {
-      rc = fill_any(G, rr * batch, s);
-      if (rc) return rc;
-    }
-  }
-  rc = gemm_any_real(g, s);
+  g.split_k = -1;   // few output tiles, long K: the launcher slices K until the GPU is full
+  int rc = da_gemm_f64(g, s);
   if (rc) return rc;
   // blocked lower Cholesky G = L L^T (right-looking), building W alongside
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-    rc = chol_step_any(G, L, W, rr, r, o, nb, info, batch, s);
+    rc = da_chol_step(G, L, W, rr, r, o, nb, info, batch, s);
     if (rc) return rc;
     if (rest <= 0) break;
     // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
-    RealGemmDesc<T> u{};
+    Gemm64Desc u{};
     u.batch = batch;
     u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
     u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
     u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
     u.E = u.C; u.sE = rr; u.lde = r;
     u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
-    rc = gemm_any_real(u, s);
+    rc = da_gemm_f64(u, s);
     if (rc) return rc;
   }
   // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
@@ -332,28 +309,74 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, int batch, int rows, int r, int* info, 
   // those rows before it stores)
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB;
-    RealGemmDesc<T> a{};
+    Gemm64Desc a{};
     a.batch = batch;
     a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
     a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
     a.C = P0 + o; a.sC = pr; a.ldc = r;
     a.E = nullptr;
     a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
-    rc = gemm_any_real(a, s);
+    rc = da_gemm_f64(a, s);
     if (rc) return rc;
   }
   return DA_OK;
 }
 
+// V = I - up(G - I) for each r x r Gram matrix G of an almost orthonormal P, where up() keeps the strict
+// upper triangle and half of the diagonal: the Cholesky factor of G = I + E is R = I + up(E) + O(E^2), so
+// P V = P R^-1 + O(E^2).
+__global__ __launch_bounds__(256) void polish_factor_kernel(const float* __restrict__ G, float* __restrict__ V,
+                                                            long long rr, int r) {
+  const long long b = blockIdx.y;
+  const int i = blockIdx.x;
+  const float* g = G + b * rr + (long long)i * r;
+  float* v = V + b * rr + (long long)i * r;
+  for (int j = threadIdx.x; j < r; j += 256) {
+    const float x = g[j];
+    v[j] = i < j ? -x : (i == j ? 1.5f - 0.5f * x : 0.f);
+  }
+}
+
+// One polishing pass in fp32:  out <- in V(in^T in).  `in` (fp64 or fp32) and `out` (fp32, or the caller's
+// dtype for the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one
+// product with the triangular V -- no serial chain.
+int polish_pass(const void* in, int in_store, void* out, int out_store, float* G, float* V, int batch, int rows,
+                int r, hipStream_t s) {
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  Gemm32Desc g{};
+  g.batch = batch;
+  g.A = static_cast<const float*>(in); g.B = g.A; g.C = G;
+  g.a_store = in_store; g.b_store = in_store;
+  g.sA = pr; g.sB = pr; g.sC = rr;
+  g.lda = r; g.ldb = r; g.ldc = r;
+  g.M = r; g.N = r; g.K = rows;
+  g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
+  g.split_k = -1;
+  int rc = da_gemm_f32s(g, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(polish_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, V, rr, r);
+  rc = da_launch_status();
+  if (rc) return rc;
+  // out = in V: V is upper triangular, so column tile j only sums k < 64 (j + 1)
+  Gemm32Desc a{};
+  a.batch = batch;
+  a.A = static_cast<const float*>(in); a.a_store = in_store; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+  a.B = V; a.sB = rr; a.ldb = r; a.b_kstrided = 1;
+  a.C = static_cast<float*>(out); a.c_store = out_store; a.sC = pr; a.ldc = r;
+  a.M = rows; a.N = r; a.K = r; a.alpha = 1.0; a.beta = 0.0; a.k_tri = 1;
+  return da_gemm_f32s(a, s);
+}
+
 }  // namespace
 
-// The first pass runs in fp64: the Gram matrix squares P's condition number (up to 4e12 on the
-// optimizer's inputs).  Its result is orthonormal to about eps64 * cond(P)^2 <= 1e-4, so the later
-// passes, which only polish it, run in fp32 -- twice the MFMA rate, half the bytes, and a serial
-// Cholesky chain of half the latency -- and still end at fp32 round-off, which is also all the
-// output dtype (fp32 or bf16) can hold.
+// The first pass is a blocked CholeskyQR in fp64: the Gram matrix squares P's condition number (up to
+// 4e12 on the optimizer's inputs).  Its result is orthonormal to E = eps64 * cond(P)^2 <= 1e-4, and for
+// such a matrix the second CholeskyQR pass has a closed form to O(E^2) <= 1e-8 -- below fp32 round-off,
+// which is all the output dtype (fp32 or bf16) can hold: R^-1 = I - up(P^T P - I).  So the later passes
+// are two fp32 products and no factorisation at all; the last one stores the output dtype.
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
                       int* info, hipStream_t s) {
+  if (passes < 1 || batch > 65535) return DA_ERR_ARG;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   double* P0 = static_cast<double*>(ws);
   double* G = P0 + pr * batch;
@@ -362,15 +385,23 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   float* P0f = reinterpret_cast<float*>(W + rr * batch);
   int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
   if (rc) return rc;
-  rc = cholqr_pass<double>(P0, G, L, W, batch, rows, r, info, s);
+  rc = cholqr_pass(P0, G, L, W, batch, rows, r, info, s);
   if (rc) return rc;
-  if (passes <= 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+  if (passes == 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+  // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products
   rc = da_cvt_f64_to_f32(P0, P0f, pr * batch, s);
   if (rc) return rc;
+  const float* cur = P0f;
+  float* Gf = reinterpret_cast<float*>(G);
+  float* Vf = reinterpret_cast<float*>(L);
   for (int pass = 1; pass < passes; ++pass) {
-    rc = cholqr_pass<float>(P0f, reinterpret_cast<float*>(G), reinterpret_cast<float*>(L), reinterpret_cast<float*>(W),
-                            batch, rows, r, info, s);
+    const bool last = pass + 1 == passes;
+    // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
+    float* other = cur == P0f ? reinterpret_cast<float*>(P0) : P0f;
+    rc = polish_pass(cur, DA_STORE_NATIVE, last ? out : static_cast<void*>(other),
+                     last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf, Vf, batch, rows, r, s);
     if (rc) return rc;
+    cur = other;
   }
-  return da_cvt_from_f32(P0f, out, dtype, pr * batch, s);
+  return DA_OK;
 }

@@ -17,20 +17,28 @@ struct RealGemmDesc {
   int lower_only;  // 1 (M == N): only tiles on or below the diagonal are computed and stored
   double alpha, beta;
   int split_k;   // > 1: K is cut into that many slices whose partial products are added atomically into a
-                 // zeroed C (no E term); the summation order, and so the last bits, vary run to run
+                 // zeroed C (no E term); the summation order, and so the last bits, vary run to run.
+                 // < 0: the launcher picks the slice count for the tile it chooses and clears C itself
+  // Storage of A, B and C when it is not T (DA_STORE_*): the pointers then address elements of that dtype
+  // (cast to T* by the caller), leading dimensions and strides count its elements, operands are widened as
+  // they are fetched and the result is rounded once at the store.  A converted C excludes E, split_k and the
+  // symmetric form.
+  int a_store, b_store, c_store;
+  int k_tri;     // 1: B is block lower triangular -- output column tile j only sums k < 64 (j + 1)
 };
+#define DA_STORE_NATIVE 0
+#define DA_STORE_BF16 1
+#define DA_STORE_F32 2
+#define DA_STORE_F64 3   // operands only (an fp64 matrix read by the fp32 kernel)
+inline int da_store_of(int dtype) { return dtype == DA_BF16 ? DA_STORE_BF16 : DA_STORE_F32; }
 typedef RealGemmDesc<double> Gemm64Desc;
 typedef RealGemmDesc<float> Gemm32Desc;
 
-// The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the second CholeskyQR pass, whose input is already
-// orthonormal to 1e-4 or better, does not need fp64.
+// The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the products of the polishing passes, whose input is
+// already orthonormal to 1e-4 or better, do not need fp64.
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s);
-int da_fill_f32(float* p, long long n, float v, hipStream_t s);
 int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s);
-int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long n, hipStream_t s);
-int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long n, hipStream_t s);
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
-int da_fill_f64(double* p, long long n, double v, hipStream_t s);
 
 // dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.
 int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s);
@@ -44,8 +52,6 @@ int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hi
 // L_jj and of D_j) and records (o + column + 1) in info[b] if it is the matrix's first failure.
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
                  int batch, hipStream_t s);
-int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
-                     int batch, hipStream_t s);
 
 #define DA_CHOL_NB 64
 

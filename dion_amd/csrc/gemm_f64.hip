@@ -9,11 +9,13 @@
 // 32 x 32 as 2 x 2 accumulators of 16 x 16.  LDS tiles are k-major [16][64] doubles for
 // either operand layout, so the one-double-per-lane MFMA operands are conflict-free reads.
 // Double buffered: the global loads of the next stage are in flight during the MFMAs.
+// Operands may be stored narrower (bf16, fp32) or wider (fp64 into the fp32 instance) than the
+// compute type and the result may be stored as fp32 or bf16; a block-triangular B operand
+// shortens the sum per column tile.
 #include "gemm_f64.h"
 
 namespace {
 
-constexpr int BT = 64;
 constexpr int BK = 16;
 
 template <bool KS, typename T>
@@ -24,8 +26,8 @@ __device__ __forceinline__ void fetch(T (&v)[4], const T* __restrict__ base, int
   const int inner = KS ? row0 + (tid & 15) * 4 : k0 + (tid & 3) * 4;
   const int outer_n = KS ? K : rows, inner_n = KS ? rows : K;
   const T* p = base + (long long)outer * ld + inner;
-  if (outer < outer_n && inner + 3 < inner_n && ((reinterpret_cast<uintptr_t>(p) & 15) == 0)) {
-    typedef T pair_t __attribute__((ext_vector_type(2)));   // 16 bytes (fp64) / 8 bytes (fp32) per access
+  if (outer < outer_n && inner + 3 < inner_n && ((reinterpret_cast<uintptr_t>(p) & (2 * sizeof(T) - 1)) == 0)) {
+    typedef T pair_t __attribute__((ext_vector_type(2)));   // 16 bytes (fp64) / 8 (fp32) / 4 (bf16) per access
     const pair_t lo = *reinterpret_cast<const pair_t*>(p);
     const pair_t hi = *reinterpret_cast<const pair_t*>(p + 2);
     v[0] = lo.x; v[1] = lo.y; v[2] = hi.x; v[3] = hi.y;
@@ -35,27 +37,57 @@ __device__ __forceinline__ void fetch(T (&v)[4], const T* __restrict__ base, int
   }
 }
 
+// The same for an operand stored as `store` (DA_STORE_*), widened to T.
 template <bool KS, typename T>
+__device__ __forceinline__ void fetch_as(T (&v)[4], const T* __restrict__ base, int store, int ld, int row0, int k0,
+                                         int rows, int K, int tid) {
+  if (store == DA_STORE_NATIVE) {
+    fetch<KS>(v, base, ld, row0, k0, rows, K, tid);
+  } else if (store == DA_STORE_F32) {
+    float t[4];
+    fetch<KS>(t, reinterpret_cast<const float*>(base), ld, row0, k0, rows, K, tid);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (T)t[e];
+  } else if (store == DA_STORE_F64) {
+    double t[4];
+    fetch<KS>(t, reinterpret_cast<const double*>(base), ld, row0, k0, rows, K, tid);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (T)t[e];
+  } else {
+    bf16_t t[4];
+    fetch<KS>(t, reinterpret_cast<const bf16_t*>(base), ld, row0, k0, rows, K, tid);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (T)bf2f(t[e]);
+  }
+}
+
+// One 64-row slice of a stage goes to the k-major LDS tile lds[k][row] (row pitch BTt).
+template <bool KS, int BTt, typename T>
 __device__ __forceinline__ void put(T* lds, const T (&v)[4], int tid) {
   if (!KS) {
     const int r = tid >> 2, k4 = (tid & 3) * 4;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) lds[(k4 + e) * BT + r] = v[e];
+    for (int e = 0; e < 4; ++e) lds[(k4 + e) * BTt + r] = v[e];
   } else {
     const int k = tid >> 4, r4 = (tid & 15) * 4;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) lds[k * BT + r4 + e] = v[e];
+    for (int e = 0; e < 4; ++e) lds[k * BTt + r4 + e] = v[e];
   }
 }
 
-template <typename T, bool A_KS, bool B_KS, bool SYM>
+// BTt x BTt output tile (64 or 128), 256 threads as 2 x 2 wavefronts of (BTt / 2) x (BTt / 2) each.  The larger
+// tile halves the operand bytes per flop: the 64-wide one is bound by the L2 -> LDS path on large products.
+template <typename T, bool A_KS, bool B_KS, bool SYM, int BTt>
 __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
   typedef typename Mfma<T>::acc_t acc_t;
-  __shared__ T lds_a[2][BK * BT];
-  __shared__ T lds_b[2][BK * BT];
+  constexpr int H = BTt / 64;        // 64-row slices per operand stage
+  constexpr int WT = BTt / 2;        // wavefront tile
+  constexpr int TI = WT / 16;        // 16 x 16 accumulators per wavefront and direction
+  __shared__ T lds_a[2][BK * BTt];
+  __shared__ T lds_b[2][BK * BTt];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
+  const int tiles_m = (d.M + BTt - 1) / BTt, tiles_n = (d.N + BTt - 1) / BTt;
   const bool tri = SYM || d.lower_only;
   const int per_batch = tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
   const int split = blockIdx.y;  // split-K slice
@@ -68,72 +100,107 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
     while (t >= len) { t -= len; ++ti; --len; }
     tj = ti + t;
     if (!SYM) { const int x = ti; ti = tj; tj = x; }   // lower triangle: row tile >= column tile
+  } else if (d.k_tri) {
+    // longest sums (last column tiles) first
+    tj = tiles_n - 1 - t / tiles_m;
+    ti = t - (tiles_n - 1 - tj) * tiles_m;
   } else {
     ti = t / tiles_n;
     tj = t - ti * tiles_n;
   }
-  const int m0 = ti * BT, n0 = tj * BT;
-  const T* A = d.A + (long long)b * d.sA;
-  const T* B = d.B + (long long)b * d.sB;
+  const int m0 = ti * BTt, n0 = tj * BTt;
+  // batch offsets in bytes of the operand's storage dtype
+  const int asz = d.a_store == DA_STORE_NATIVE ? (int)sizeof(T) : d.a_store == DA_STORE_F64 ? 8 : d.a_store == DA_STORE_F32 ? 4 : 2;
+  const int bsz = d.b_store == DA_STORE_NATIVE ? (int)sizeof(T) : d.b_store == DA_STORE_F64 ? 8 : d.b_store == DA_STORE_F32 ? 4 : 2;
+  const T* A = reinterpret_cast<const T*>(reinterpret_cast<const char*>(d.A) + (long long)b * d.sA * asz);
+  const T* B = reinterpret_cast<const T*>(reinterpret_cast<const char*>(d.B) + (long long)b * d.sB * bsz);
+  const int Keff = d.k_tri && n0 + BTt < d.K ? n0 + BTt : d.K;
 
-  acc_t acc[2][2];
+  acc_t acc[TI][TI];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+    for (int j = 0; j < TI; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
   // double buffered: the global loads of stage s+1 are in flight while stage s is multiplied
-  const int KT_all = (d.K + BK - 1) / BK;
+  const int KT_all = (Keff + BK - 1) / BK;
   const int per_split = (KT_all + (int)gridDim.y - 1) / (int)gridDim.y;
   const int kt0 = split * per_split;
   const int KT = KT_all - kt0 < per_split ? KT_all - kt0 : per_split;   // may be <= 0 for the last slices
-  T pa[4], pb[4];
+  T pa[H][4], pb[H][4];
+#define DA_RFETCH(kt)                                                                               \
+  do {                                                                                              \
+    _Pragma("unroll") for (int h = 0; h < H; ++h) {                                                 \
+      fetch_as<A_KS>(pa[h], A, d.a_store, d.lda, m0 + 64 * h, (kt) * BK, d.M, Keff, tid);           \
+      fetch_as<B_KS>(pb[h], B, d.b_store, d.ldb, n0 + 64 * h, (kt) * BK, d.N, Keff, tid);           \
+    }                                                                                               \
+  } while (0)
+#define DA_RPUT(buf)                                                                                \
+  do {                                                                                              \
+    _Pragma("unroll") for (int h = 0; h < H; ++h) {                                                 \
+      put<A_KS, BTt>(lds_a[buf] + 64 * h, pa[h], tid);                                              \
+      put<B_KS, BTt>(lds_b[buf] + 64 * h, pb[h], tid);                                              \
+    }                                                                                               \
+  } while (0)
   if (KT > 0) {
-    fetch<A_KS>(pa, A, d.lda, m0, kt0 * BK, d.M, d.K, tid);
-    fetch<B_KS>(pb, B, d.ldb, n0, kt0 * BK, d.N, d.K, tid);
-    put<A_KS>(lds_a[0], pa, tid);
-    put<B_KS>(lds_b[0], pb, tid);
+    DA_RFETCH(kt0);
+    DA_RPUT(0);
   }
   __syncthreads();
   for (int kt = 0; kt < KT; ++kt) {
     const T* sa = lds_a[kt & 1];
     const T* sb = lds_b[kt & 1];
     const bool more = kt + 1 < KT;
-    if (more) {
-      fetch<A_KS>(pa, A, d.lda, m0, (kt0 + kt + 1) * BK, d.M, d.K, tid);
-      fetch<B_KS>(pb, B, d.ldb, n0, (kt0 + kt + 1) * BK, d.N, d.K, tid);
-    }
+    if (more) DA_RFETCH(kt0 + kt + 1);
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       const int k = ks * 4 + (lane >> 4);
-      T af[2], bfv[2];
+      T af[TI], bfv[TI];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) af[i] = sa[k * BT + wm * 32 + i * 16 + (lane & 15)];
+      for (int i = 0; i < TI; ++i) af[i] = sa[k * BTt + wm * WT + i * 16 + (lane & 15)];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) bfv[j] = sb[k * BT + wn * 32 + j * 16 + (lane & 15)];
+      for (int j = 0; j < TI; ++j) bfv[j] = sb[k * BTt + wn * WT + j * 16 + (lane & 15)];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
+        for (int j = 0; j < TI; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
     }
-    if (more) {
-      put<A_KS>(lds_a[(kt + 1) & 1], pa, tid);
-      put<B_KS>(lds_b[(kt + 1) & 1], pb, tid);
-    }
+    if (more) DA_RPUT((kt + 1) & 1);
     __syncthreads();
   }
+#undef DA_RFETCH
+#undef DA_RPUT
 
+  if (d.c_store != DA_STORE_NATIVE) {   // rounded once to the storage dtype; no E, no split, no mirror (checked on the host)
+    char* Cc = reinterpret_cast<char*>(d.C) + (long long)b * d.sC * (d.c_store == DA_STORE_F32 ? 4 : 2);
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TI; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = m0 + wm * WT + i * 16 + Mfma<T>::row(v, lane);
+          const int n = n0 + wn * WT + j * 16 + (lane & 15);
+          if (m < d.M && n < d.N) {
+            const float o = (float)((T)d.alpha * acc[i][j][v]);
+            const long long at = (long long)m * d.ldc + n;
+            if (d.c_store == DA_STORE_F32) reinterpret_cast<float*>(Cc)[at] = o;
+            else reinterpret_cast<bf16_t*>(Cc)[at] = f2bf(o);
+          }
+        }
+    return;
+  }
   T* C = d.C + (long long)b * d.sC;
   const T* E = d.E ? d.E + (long long)b * d.sE : nullptr;
   const bool mirror = SYM && (ti != tj);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TI; ++j)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int m = m0 + wm * 32 + i * 16 + Mfma<T>::row(v, lane);
-        const int n = n0 + wn * 32 + j * 16 + (lane & 15);
+        const int m = m0 + wm * WT + i * 16 + Mfma<T>::row(v, lane);
+        const int n = n0 + wn * WT + j * 16 + (lane & 15);
         if (m < d.M && n < d.N) {
           T o = (T)d.alpha * acc[i][j][v];
           if (gridDim.y > 1) {  // split-K: partial sums meet in a zeroed C
@@ -148,16 +215,49 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
       }
 }
 
+template <typename R>
+__global__ void fill_f64_kernel(R* p, long long n, R v) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+template <typename T, int BTt>
+long long blocks_of(const RealGemmDesc<T>& d) {
+  const long long tiles_m = (d.M + BTt - 1) / BTt, tiles_n = (d.N + BTt - 1) / BTt;
+  return ((d.symmetric || d.lower_only) ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n) * d.batch;
+}
+
+template <typename T, bool A_KS, bool B_KS, bool SYM, int BTt>
+int launch_bt(const RealGemmDesc<T>& d, int split, hipStream_t s) {
+  const long long blocks = blocks_of<T, BTt>(d);
+  if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL((gemm_f64_kernel<T, A_KS, B_KS, SYM, BTt>), dim3((unsigned)blocks, split), dim3(256), 0, s, d);
+  return da_launch_status();
+}
+
 template <typename T, bool A_KS, bool B_KS, bool SYM>
 int launch(const RealGemmDesc<T>& d, hipStream_t s) {
-  const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
-  const long long per_batch = (SYM || d.lower_only) ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
-  const long long blocks = per_batch * d.batch;
-  if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
-  int split = d.split_k > 1 ? d.split_k : 1;
-  if (d.E) split = 1;
-  hipLaunchKernelGGL((gemm_f64_kernel<T, A_KS, B_KS, SYM>), dim3((unsigned)blocks, split), dim3(256), 0, s, d);
-  return da_launch_status();
+  // Only the 64-wide tile is instantiated: the 128-wide one (half the operand bytes per flop, but 198 VGPRs
+  // and 64 KB of LDS in fp64, i.e. two workgroups per CU instead of five) measured 10-20 % slower on the
+  // orthonormaliser's products.
+  constexpr int BTt = 64;
+  const long long blocks = blocks_of<T, BTt>(d);
+  const bool auto_split = d.split_k < 0 && !d.E && d.c_store == DA_STORE_NATIVE;
+  int split = d.split_k > 1 && !d.E ? d.split_k : 1;
+  if (auto_split) {
+    // few output tiles, long K: slice K until ~512 workgroups exist
+    const int max_split = d.K / 256 > 0 ? d.K / 256 : 1;
+    const long long sp = (512 + blocks - 1) / blocks;
+    split = (int)(sp > max_split ? max_split : sp);
+    if (split > 1) {
+      // the slices add into C: clear it (the batches of C are contiguous here)
+      const long long n = (long long)d.sC * (d.batch - 1) + (long long)(d.M - 1) * d.ldc + d.N;
+      hipLaunchKernelGGL(fill_f64_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d.C, n, T(0));
+      const int rc = da_launch_status();
+      if (rc) return rc;
+    }
+  }
+  return launch_bt<T, A_KS, B_KS, SYM, BTt>(d, split, s);
 }
 
 template <typename T, typename R>
@@ -180,12 +280,6 @@ __global__ __launch_bounds__(256) void cvt_f64_to_f32_kernel(const double* __res
     dst[i] = (float)src[i];
 }
 
-template <typename R>
-__global__ void fill_f64_kernel(R* p, long long n, R v) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = v;
-}
-
 inline unsigned cvt_blocks(long long n) {
   long long b = (n + 255) / 256;
   return (unsigned)(b > 8192 ? 8192 : (b < 1 ? 1 : b));
@@ -195,6 +289,11 @@ template <typename T>
 int gemm_real(const RealGemmDesc<T>& d, hipStream_t s) {
   if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K < 0 || d.batch <= 0) return DA_ERR_ARG;
   if (d.lower_only && (d.M != d.N || d.symmetric)) return DA_ERR_ARG;
+  for (int st : {d.a_store, d.b_store})
+    if (st != DA_STORE_NATIVE && st != DA_STORE_BF16 && st != DA_STORE_F32 && st != DA_STORE_F64) return DA_ERR_DTYPE;
+  if (d.c_store != DA_STORE_NATIVE && d.c_store != DA_STORE_BF16 && d.c_store != DA_STORE_F32) return DA_ERR_DTYPE;
+  if (d.c_store != DA_STORE_NATIVE && (d.E || d.split_k > 1 || d.symmetric)) return DA_ERR_ARG;
+  if (d.k_tri && (d.symmetric || d.lower_only || d.split_k > 1)) return DA_ERR_ARG;
   if (d.symmetric) {
     if (d.M != d.N || !d.a_kstrided || !d.b_kstrided) return DA_ERR_ARG;  // only the Gram form A^T A
     return launch<T, true, true, true>(d, s);
@@ -234,21 +333,8 @@ int cvt_from(const R* src, void* dst, int dst_dtype, long long n, hipStream_t s)
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) { return gemm_real<double>(d, s); }
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s) { return gemm_real<float>(d, s); }
 
-int da_fill_f64(double* p, long long n, double v, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(fill_f64_kernel<double>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
-  return da_launch_status();
-}
-int da_fill_f32(float* p, long long n, float v, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(fill_f64_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n, v);
-  return da_launch_status();
-}
-
 int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) { return cvt_to<double>(src, src_dtype, dst, n, s); }
 int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<double>(src, dst, dst_dtype, n, s); }
-int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long n, hipStream_t s) { return cvt_to<float>(src, src_dtype, dst, n, s); }
-int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<float>(src, dst, dst_dtype, n, s); }
 int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
   hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, n);

@@ -7,7 +7,7 @@ arguments, defaults, validation errors, param-group keys and `self.state` layout
 
 Per `step()` the matrices of every "dion" group are bucketed by (shape, dtype) and each bucket
 goes, as arrays of device pointers, to `dion_amd_dion_step`: B = M + G, the tall-skinny MFMA
-GEMMs P = B Q and R = B^T P, an fp64 CholeskyQR2 orthonormalisation of P on the device, the
+GEMMs P = B Q and R = B^T P, a CholeskyQR2 orthonormalisation of P on the device (fp64 pass, fp32 polish), the
 error-feedback and weight updates fused into GEMM epilogues, and the column normalisation
 that yields the next Q.
 """

@@ -144,8 +144,9 @@ def gemm(A: Tensor, B: Tensor, *, a_kstrided=False, b_kstrided=False, E: Tensor 
 
 
 def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False):
-    """Thin-QR Q factor of P (rows x r) or a batch of them on the device (CholeskyQR `passes` times in fp64);
-    counterpart of `orthogonalize` (reference dion/dion.py:1267-1308), equal up to column signs."""
+    """Thin-QR Q factor of P (rows x r) or a batch of them on the device (one CholeskyQR pass in fp64, then
+    `passes - 1` fp32 polishing passes); counterpart of `orthogonalize` (reference dion/dion.py:1267-1308),
+    equal up to column signs."""
     lib = _lib.load()
     _lib.require_gpu(P, "orthonormalize")
     P3 = (P if P.ndim == 3 else P.unsqueeze(0)).contiguous()

@@ -187,9 +187,11 @@ size_t dion_amd_orthonormalize_workspace_bytes(int batch, int rows, int r);
 /* Replaces orthogonalize (reference dion/dion.py:1267-1308; per-matrix variants
  * dion/dion_reference.py:733-789): thin-QR Q factor of each of `batch` contiguous matrices
  * P_b (rows x r, rows >= r, dtype bf16 or f32), written to out_b (same layout; may alias P).
- * Method: CholeskyQR repeated `passes` times (2 = CholeskyQR2) with the Gram matrix, the
- * blocked Cholesky factorisation and the triangular solve all in fp64 on the device; no
- * host synchronisation.  The factor equals the reference's Householder / randomised
+ * Method: CholeskyQR2.  The first pass (Gram matrix, blocked Cholesky factorisation,
+ * triangular solve) runs in fp64 on the device; each further pass (`passes` - 1 of them) is
+ * the first-order form of a CholeskyQR pass on an almost orthonormal matrix,
+ * P <- P (I - up(P^T P - I)) in fp32, which squares the remaining defect ||P^T P - I||.
+ * No host synchronisation.  The factor equals the reference's Householder / randomised
  * Cholesky QR result up to column signs (Cholesky's diagonal is positive).
  * info (device, `batch` ints, may be NULL): 0, or 1 + the first column whose pivot was not
  * positive -- the analogue of torch.linalg.cholesky_ex's info; such columns come out as 0. */

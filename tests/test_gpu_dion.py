@@ -41,6 +41,29 @@ def test_orthonormalize(dev, rows, r, dtype):
     assert (torch.diagonal(Rm) > 0).all()
 
 
+@pytest.mark.parametrize("log_cond,passes,tol", [(4, 1, 5e-6), (6, 2, 5e-5), (7, 2, 2e-4), (7.5, 3, 5e-5)])
+def test_orthonormalize_conditioning(dev, log_cond, passes, tol):
+    """Genuinely ill-conditioned factors (singular values graded over `log_cond` decades between random
+    orthonormal bases, not a column scaling that a Cholesky factorisation does not feel).  The fp64 pass
+    leaves ||Q^T Q - I|| ~ eps64 * cond^2 and every fp32 polishing pass squares what is left, down to fp32
+    round-off; the optimizer runs two passes, so it holds the 1e-3 bar up to cond ~ 3e7."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(5)
+    rows, r = 1536, 320
+    U, _ = torch.linalg.qr(torch.randn(rows, r, dtype=torch.float64))
+    V, _ = torch.linalg.qr(torch.randn(r, r, dtype=torch.float64))
+    P = ((U * torch.logspace(0, -log_cond, r, dtype=torch.float64)) @ V.T).float()
+    Q, info = orthonormalize(P.to(dev), passes=passes, return_info=True)
+    assert int(info.item()) == 0
+    Qd = Q.double().cpu()
+    orth = (Qd.T @ Qd - torch.eye(r, dtype=torch.float64)).norm().item()
+    Qh, _ = torch.linalg.qr(P.double())
+    diff = rel_fro(_sign_align(Qd, Qh), Qh)
+    print(f"cond 1e{log_cond}, {passes} passes: ||QtQ-I|| = {orth:.2e}, vs Householder {diff:.2e}")
+    assert orth <= tol and diff <= tol
+
+
 def test_orthonormalize_batch_and_rank_deficient(dev):
     from dion_amd.newton_schulz import orthonormalize
 
