@@ -156,6 +156,23 @@ def summarize(name, wl, res):
                    ns_frac_mfma_peak=round(f_sym / (ns_ms * 1e-3) / PEAK_BF16_FLOPS, 4),
                    ns_dense_convention_tflops=round(ns_flops(shapes, False) / (ns_ms * 1e-3) / 1e12, 1))
     out["kernels"] = res["kernels"]
+    if wl["kind"] == "dion":
+        # Dion's products sit near the machine balance (arithmetic intensity ~ r flop/byte): report them against
+        # the HBM roofline as well.  Algorithmic bytes per step over all matrices, bf16 momentum / weights,
+        # factors in the momentum dtype: P = BQ and R = B^T P read B once; the error-feedback and weight-update
+        # products read and write an m x n matrix; each also moves its m' x r and n' x r factors.
+        import math
+
+        rd = upd = 0.0
+        for m, n in shapes:
+            r = min(math.ceil(wl["rank_fraction"] * min(m, n)), m, n)   # reference dion/dion.py:672-676
+            rd += 2.0 * (m * n + (m + n) * r)
+            upd += 2.0 * (2 * m * n + (m + n) * r)
+        for name, nbytes in (("dion_bq", rd), ("dion_btp", rd), ("dion_ef", upd), ("dion_upd", upd)):
+            k = out["kernels"].get(name)
+            if k and k["ms_per_step"] > 0:
+                rate = nbytes / (k["ms_per_step"] * 1e-3)
+                k.update(gbps=round(rate / 1e9, 1), frac_hbm=round(rate / PEAK_HBM_BPS, 4))
     return out
 
 
