@@ -264,7 +264,8 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 size_t da_orth_workspace_bytes(int batch, int rows, int r) {
   size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place (first pass)
                + 3 * (size_t)r * r * 8    // G, L, W (fp64; the polishing passes keep their fp32 G and V there)
-               + (size_t)rows * r * 4;    // fp32 iterate between polishing passes (three or more passes)
+               + (size_t)rows * r * 4     // the fp64 pass's result in fp32 (input of the polishing pass)
+               + (size_t)rows * r * 2;    // ... and in bf16 (operand of its correction product)
   return per * batch + 256;
 }
 
@@ -337,6 +338,52 @@ __global__ __launch_bounds__(256) void polish_factor_kernel(const float* __restr
   }
 }
 
+// U = up(G - I) in bf16 (see polish_factor_kernel): the factor of the correction product P U, which only has
+// to be known to the relative accuracy of bf16 because it is itself of the size of the defect.
+__global__ __launch_bounds__(256) void polish_correction_kernel(const float* __restrict__ G, bf16_t* __restrict__ U,
+                                                                long long rr, int r) {
+  const long long b = blockIdx.y;
+  const int i = blockIdx.x;
+  const float* g = G + b * rr + (long long)i * r;
+  bf16_t* u = U + b * rr + (long long)i * r;
+  for (int j = threadIdx.x; j < r; j += 256) {
+    const float x = g[j];
+    u[j] = f2bf(i < j ? x : (i == j ? 0.5f * (x - 1.f) : 0.f));
+  }
+}
+
+// The last polishing pass of an iterate that exists in fp32 and in bf16:  out <- in - in_bf16 U(in^T in).
+// The Gram product is fp32 as in polish_pass; the correction product runs on the bf16 matrix cores (its
+// relative error 2^-8 times the defect E of `in` adds 4e-3 E to the result, next to the pass's own O(E^2)).
+int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_dtype, float* G, bf16_t* U, int batch,
+                     int rows, int r, hipStream_t s) {
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  Gemm32Desc g{};
+  g.batch = batch;
+  g.A = in; g.B = in; g.C = G;
+  g.sA = pr; g.sB = pr; g.sC = rr;
+  g.lda = r; g.ldb = r; g.ldc = r;
+  g.M = r; g.N = r; g.K = rows;
+  g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
+  g.split_k = -1;
+  int rc = da_gemm_f32s(g, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(polish_correction_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, U, rr, r);
+  rc = da_launch_status();
+  if (rc) return rc;
+  GemmDesc c{};
+  c.batch = batch;
+  c.A = in_low; c.sA = pr; c.lda = r; c.a_kstrided = 0;
+  c.B = U; c.sB = rr; c.ldb = r; c.b_kstrided = 1;
+  c.C = out; c.sC = pr; c.ldc = r; c.c_dtype = out_dtype;
+  // the addend has C's dtype: the fp32 iterate for an fp32 result, its bf16 copy for a bf16 one
+  c.E = out_dtype == DA_F32 ? static_cast<const void*>(in) : static_cast<const void*>(in_low);
+  c.sE = pr; c.lde = r;
+  c.M = rows; c.N = r; c.K = r;
+  c.epilogue = DA_EPI_AXPBY; c.s0 = 1.f; c.s1 = -1.f; c.faithful = 0;
+  return da_gemm_bf16(c, s);
+}
+
 // One polishing pass in fp32:  out <- in V(in^T in).  `in` (fp64 or fp32) and `out` (fp32, or the caller's
 // dtype for the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one
 // product with the triangular V -- no serial chain.
@@ -383,14 +430,20 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   double* L = G + rr * batch;
   double* W = L + rr * batch;
   float* P0f = reinterpret_cast<float*>(W + rr * batch);
+  bf16_t* P0h = reinterpret_cast<bf16_t*>(P0f + pr * batch);
   int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
   if (rc) return rc;
   rc = cholqr_pass(P0, G, L, W, batch, rows, r, info, s);
   if (rc) return rc;
   if (passes == 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
   // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products
-  rc = da_cvt_f64_to_f32(P0, P0f, pr * batch, s);
+  // (the bf16 product moves 16-byte chunks: r a multiple of 8, else the all-fp32 form below)
+  const bool low = passes == 2 && (r & 7) == 0;
+  rc = da_cvt_f64_to_f32(P0, P0f, low ? P0h : nullptr, pr * batch, s);
   if (rc) return rc;
+  if (low)
+    return polish_pass_bf16(P0f, P0h, out, dtype, reinterpret_cast<float*>(G), reinterpret_cast<bf16_t*>(L), batch,
+                            rows, r, s);
   const float* cur = P0f;
   float* Gf = reinterpret_cast<float*>(G);
   float* Vf = reinterpret_cast<float*>(L);

@@ -37,7 +37,8 @@ typedef RealGemmDesc<float> Gemm32Desc;
 // The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the products of the polishing passes, whose input is
 // already orthonormal to 1e-4 or better, do not need fp64.
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s);
-int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s);
+// dst (f32) <- src (f64); `low`, if not null, receives the same values in bf16
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, hipStream_t s);
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
 
 // dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.

@@ -274,10 +274,14 @@ __global__ __launch_bounds__(256) void cvt_from_f64_kernel(const R* __restrict__
     st_from_float<T>(dst + i, (float)src[i]);
 }
 
+// fp64 -> fp32, and (if `low` is given) the same values rounded once more to bf16
 __global__ __launch_bounds__(256) void cvt_f64_to_f32_kernel(const double* __restrict__ src, float* __restrict__ dst,
-                                                              long long n) {
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
-    dst[i] = (float)src[i];
+                                                              bf16_t* __restrict__ low, long long n) {
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const float v = (float)src[i];
+    dst[i] = v;
+    if (low) low[i] = f2bf(v);
+  }
 }
 
 inline unsigned cvt_blocks(long long n) {
@@ -335,8 +339,8 @@ int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s) { return gemm_real<float>(d
 
 int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) { return cvt_to<double>(src, src_dtype, dst, n, s); }
 int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<double>(src, dst, dst_dtype, n, s); }
-int da_cvt_f64_to_f32(const double* src, float* dst, long long n, hipStream_t s) {
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, n);
+  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, low, n);
   return da_launch_status();
 }

@@ -46,7 +46,7 @@ def test_orthonormalize_conditioning(dev, log_cond, passes, tol):
     """Genuinely ill-conditioned factors (singular values graded over `log_cond` decades between random
     orthonormal bases, not a column scaling that a Cholesky factorisation does not feel).  The fp64 pass
     leaves ||Q^T Q - I|| ~ eps64 * cond^2 and every fp32 polishing pass squares what is left, down to fp32
-    round-off; the optimizer runs two passes, so it holds the 1e-3 bar up to cond ~ 3e7."""
+    round-off; the optimizer runs two passes, so it holds the 1e-3 bar up to cond ~ 2e7."""
     from dion_amd.newton_schulz import orthonormalize
 
     torch.manual_seed(5)
