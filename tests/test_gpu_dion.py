@@ -17,7 +17,7 @@ def _sign_align(a, ref):
     return a.double() * s
 
 
-@pytest.mark.parametrize("rows,r", [(768, 192), (3072, 768), (768, 768), (520, 72), (4096, 512)])
+@pytest.mark.parametrize("rows,r", [(768, 192), (3072, 768), (768, 768), (520, 72), (4096, 512), (100, 28)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_orthonormalize(dev, rows, r, dtype):
     from dion_amd.newton_schulz import orthonormalize
