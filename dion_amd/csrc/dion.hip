@@ -19,6 +19,17 @@ template <> struct V8<bf16_t> {
       v[2 * i + 1] = bf2f((bf16_t)(w[i] >> 16));
     }
   }
+  // read-once data (gradients): keep it out of the caches' way
+  static __device__ __forceinline__ void load_nt(const bf16_t* p, float (&v)[8]) {
+    typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+    const u32x4_t r = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned w = r[i];
+      v[2 * i] = bf2f((bf16_t)(w & 0xffffu));
+      v[2 * i + 1] = bf2f((bf16_t)(w >> 16));
+    }
+  }
   static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
     uint32_t w[4];
 #pragma unroll
@@ -33,6 +44,16 @@ template <> struct V8<float> {
     const float4 a = *reinterpret_cast<const float4*>(p);
     const float4 b = *reinterpret_cast<const float4*>(p + 4);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void load_nt(const float* p, float (&v)[8]) {
+    typedef float f32x4_nt_t __attribute__((ext_vector_type(4)));
+    const f32x4_nt_t a = __builtin_nontemporal_load(reinterpret_cast<const f32x4_nt_t*>(p));
+    const f32x4_nt_t b = __builtin_nontemporal_load(reinterpret_cast<const f32x4_nt_t*>(p + 4));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float x = a[i], y = b[i];
+      v[i] = x; v[4 + i] = y;
+    }
   }
   static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -61,7 +82,7 @@ __global__ __launch_bounds__(256) void add_grad_kernel(DaPtrTable mt, DaPtrTable
   for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
     float m[8], g[8];
     V8<TM>::load(M + i, m);
-    V8<TG>::load(G + i, g);
+    V8<TG>::load_nt(G + i, g);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       m[e] = V8<TM>::round(m[e] + g[e]);
