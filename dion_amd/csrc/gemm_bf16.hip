@@ -182,6 +182,35 @@ __device__ __forceinline__ float epi_value(float s0, float s1, float acc, float 
   return HAS_E ? s0 * e + s1 * acc : s1 * acc;
 }
 
+// Two neighbouring elements of a bf16 C at once.  Written with explicit pairs because the epilogue is bound by
+// its VALU instructions (a 256 x 256 tile has 128 elements per lane): converting element by element the
+// compiler issues one v_cvt_pk_bf16_f32 per value and 25 instructions per pair for the rounding-faithful
+// a X + B X form; with both halves of every conversion used, and the exact multiplication by s1 == 1 skipped,
+// it is 13 (and a single conversion for a plain rounded store).
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned cvt_pk_bf16(float a, float b) {
+  const f32x2_t f = {a, b};
+  const bf16x2_t h = __builtin_convertvector(f, bf16x2_t);
+  return __builtin_bit_cast(unsigned, h);
+}
+__device__ __forceinline__ float lo_f(unsigned w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float hi_f(unsigned w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// The value pair of epi_value<HAS_E, FAITHFUL, false>, rounded to bf16 and packed (`ew`: the two bf16 of E).
+template <bool HAS_E, bool FAITHFUL>
+__device__ __forceinline__ unsigned epi_pair(float s0, float s1, float a0, float a1, unsigned ew) {
+  if (FAITHFUL) {
+    unsigned p = cvt_pk_bf16(a0, a1);
+    if (s1 != 1.f) p = cvt_pk_bf16(s1 * lo_f(p), s1 * hi_f(p));
+    if (!HAS_E) return p;
+    const unsigned q = cvt_pk_bf16(s0 * lo_f(ew), s0 * hi_f(ew));
+    return cvt_pk_bf16(lo_f(q) + lo_f(p), hi_f(q) + hi_f(p));
+  }
+  if (HAS_E) return cvt_pk_bf16(s0 * lo_f(ew) + s1 * a0, s0 * hi_f(ew) + s1 * a1);
+  return cvt_pk_bf16(s1 * a0, s1 * a1);
+}
+
 typedef __attribute__((address_space(1))) u32x4_t global_u32x4_t;
 __device__ __forceinline__ u32x4_t ldg16(const char* p) { return *(const global_u32x4_t*)p; }
 __device__ __forceinline__ void stg16(char* p, u32x4_t v) { *(global_u32x4_t*)p = v; }
@@ -321,21 +350,15 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
           stg16(Cp, o0);
           stg16(Cp + 16, o1);
         } else {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const unsigned w = HAS_E ? ec[pass][0][q] : 0u;
-            e[2 * q] = __builtin_bit_cast(float, w << 16);
-            e[2 * q + 1] = __builtin_bit_cast(float, w & 0xffff0000u);
-          }
           u32x4_t pk;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const bf16_t lo = f2bf(epi_value<HAS_E, FAITHFUL, false>(s0, s1, v[2 * q], e[2 * q]));
-            const bf16_t hi = f2bf(epi_value<HAS_E, FAITHFUL, false>(s0, s1, v[2 * q + 1], e[2 * q + 1]));
-            pk[q] = (unsigned)lo | ((unsigned)hi << 16);
+            const unsigned w = HAS_E ? ec[pass][0][q] : 0u;   // (copied out: see the note on bit_cast above)
+            const unsigned o = epi_pair<HAS_E, FAITHFUL>(s0, s1, v[2 * q], v[2 * q + 1], w);
+            pk[q] = o;
             if (SYM) {
-              v[2 * q] = bf2f(lo);
-              v[2 * q + 1] = bf2f(hi);
+              v[2 * q] = lo_f(o);
+              v[2 * q + 1] = hi_f(o);
             }
           }
           stg16(Cp, pk);
@@ -369,7 +392,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
           } else {
             u32x4_t pk;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) pk[q] = (unsigned)f2bf(v[2 * q]) | ((unsigned)f2bf(v[2 * q + 1]) << 16);
+            for (int q = 0; q < 4; ++q) pk[q] = cvt_pk_bf16(v[2 * q], v[2 * q + 1]);
             stg16(Cp, pk);
           }
         }
