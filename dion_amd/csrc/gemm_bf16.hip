@@ -186,7 +186,7 @@ __device__ __forceinline__ float epi_value(float s0, float s1, float acc, float 
 // its VALU instructions (a 256 x 256 tile has 128 elements per lane): converting element by element the
 // compiler issues one v_cvt_pk_bf16_f32 per value and 25 instructions per pair for the rounding-faithful
 // a X + B X form; with both halves of every conversion used, and the exact multiplication by s1 == 1 skipped,
-// it is 13 (and a single conversion for a plain rounded store).
+// it is 13 (and a single conversion for a plain rounded store).  S1_ONE: s1 == 1 (a compile-time variant).
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned cvt_pk_bf16(float a, float b) {
@@ -198,11 +198,11 @@ __device__ __forceinline__ float lo_f(unsigned w) { return __builtin_bit_cast(fl
 __device__ __forceinline__ float hi_f(unsigned w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
 
 // The value pair of epi_value<HAS_E, FAITHFUL, false>, rounded to bf16 and packed (`ew`: the two bf16 of E).
-template <bool HAS_E, bool FAITHFUL>
+template <bool HAS_E, bool FAITHFUL, bool S1_ONE>
 __device__ __forceinline__ unsigned epi_pair(float s0, float s1, float a0, float a1, unsigned ew) {
   if (FAITHFUL) {
     unsigned p = cvt_pk_bf16(a0, a1);
-    if (s1 != 1.f) p = cvt_pk_bf16(s1 * lo_f(p), s1 * hi_f(p));
+    if (!S1_ONE) p = cvt_pk_bf16(s1 * lo_f(p), s1 * hi_f(p));
     if (!HAS_E) return p;
     const unsigned q = cvt_pk_bf16(s0 * lo_f(ew), s0 * hi_f(ew));
     return cvt_pk_bf16(lo_f(q) + lo_f(p), hi_f(q) + hi_f(p));
@@ -266,7 +266,7 @@ __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_wave_barrier();
 }
 
-template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL>
+template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL, bool S1_ONE>
 __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
                                               bool mirror, int m0, int n0, int wave, int lane, int wm, int wn) {
   constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
@@ -354,7 +354,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const unsigned w = HAS_E ? ec[pass][0][q] : 0u;   // (copied out: see the note on bit_cast above)
-            const unsigned o = epi_pair<HAS_E, FAITHFUL>(s0, s1, v[2 * q], v[2 * q + 1], w);
+            const unsigned o = epi_pair<HAS_E, FAITHFUL, S1_ONE>(s0, s1, v[2 * q], v[2 * q + 1], w);
             pk[q] = o;
             if (SYM) {
               v[2 * q] = lo_f(o);
@@ -407,13 +407,20 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
                                          int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
   const bool mirror = SYM && (ti != tj);
   const bool cf32 = d.c_dtype == DA_F32, has_e = d.epilogue == DA_EPI_AXPBY, fa = d.faithful != 0;
-#define DA_EPI(CF, HE, FA) epilogue_impl<C, SYM, FULL, CF, HE, FA>(acc, d, lds, b, mirror, m0, n0, wave, lane, wm, wn)
+  const bool one = d.s1 == 1.f;   // rounding-faithful bf16 output: the exact multiplication by 1 is left out
+#define DA_EPI(CF, HE, FA, S1) \
+  epilogue_impl<C, SYM, FULL, CF, HE, FA, S1>(acc, d, lds, b, mirror, m0, n0, wave, lane, wm, wn)
   if (!cf32) {
-    if (has_e) { if (fa) DA_EPI(false, true, true); else DA_EPI(false, true, false); }
-    else       { if (fa) DA_EPI(false, false, true); else DA_EPI(false, false, false); }
+    if (has_e) {
+      if (fa) { if (one) DA_EPI(false, true, true, true); else DA_EPI(false, true, true, false); }
+      else DA_EPI(false, true, false, false);
+    } else {
+      if (fa) { if (one) DA_EPI(false, false, true, true); else DA_EPI(false, false, true, false); }
+      else DA_EPI(false, false, false, false);
+    }
   } else {
-    if (has_e) { if (fa) DA_EPI(true, true, true); else DA_EPI(true, true, false); }
-    else       { if (fa) DA_EPI(true, false, true); else DA_EPI(true, false, false); }
+    if (has_e) { if (fa) DA_EPI(true, true, true, false); else DA_EPI(true, true, false, false); }
+    else       { if (fa) DA_EPI(true, false, true, false); else DA_EPI(true, false, false, false); }
   }
 #undef DA_EPI
 }
