@@ -26,13 +26,24 @@ FLAGS = [
 ]
 
 
+# MFMA accumulators of the fp64 / fp32 kernels stay in ordinary VGPRs: left to its heuristic the compiler
+# keeps them in AGPRs only inside the MFMA blocks and copies all of them over and back on every loop
+# iteration (32 v_accvgpr_write + 32 v_accvgpr_read per 16 MFMAs; 4-6 % of the orthonormaliser).  The bf16
+# kernel, whose K loop has no such copies, measured 2 % slower with the option and is built without it.
+PER_FILE_FLAGS = {
+    "gemm_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "cholesky.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
 def _compile(src):
     obj = os.path.join(OBJ, src[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *PER_FILE_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     return src, obj, res
 
