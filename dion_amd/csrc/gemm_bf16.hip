@@ -277,14 +277,18 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
   constexpr int CSZ = CF32 ? 4 : 2;
   constexpr int NV = CF32 ? 2 : 1;   // 16-byte vectors per 8 elements
   float* stg = reinterpret_cast<float*>(lds) + wave * (32 * PITCH);
+  // the descriptor lives in the kernel-argument segment: fields read inside the band loop would be fetched
+  // again after every store (scalar load + a full wait in the middle of the band), so they are copied first
   const float s0 = d.s0, s1 = d.s1;
+  const int dM = d.M, dN = d.N;
+  const long long ldc = d.ldc, lde = d.lde;
   const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
   char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * CSZ;
   const char* const Ebase = !HAS_E ? nullptr
                             : d.Etab ? static_cast<const char*>(d.Etab[b])
                                      : static_cast<const char*>(d.E) + (long long)b * d.sE * CSZ;
   const int lr = lane / CPR, c8 = (lane % CPR) * 8;
-  const bool col_ok = FULL || wn0 + c8 < d.N;
+  const bool col_ok = FULL || wn0 + c8 < dN;
   // E for one band is fetched up front (its latency overlaps the LDS staging of the accumulators)
   // and the next band's E is requested before the current band is finished.
   u32x4_t ev[NPASS][NV];
@@ -295,8 +299,8 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int h = 0; h < NV; ++h) ev[pass][h] = z;
-      if (col_ok && (FULL || m < d.M)) {
-        const char* Ep = Ebase + ((long long)m * d.lde + wn0 + c8) * CSZ;
+      if (col_ok && (FULL || m < dM)) {
+        const char* Ep = Ebase + ((long long)m * lde + wn0 + c8) * CSZ;
 #pragma unroll
         for (int h = 0; h < NV; ++h) ev[pass][h] = ldg16(Ep + 16 * h);
       }
@@ -328,13 +332,13 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
     for (int pass = 0; pass < NPASS; ++pass) {
       const int r = pass * RPP + lr;
       const int m = band_m + r;
-      if (col_ok && (FULL || m < d.M)) {
+      if (col_ok && (FULL || m < dM)) {
         float* sp = stg + r * PITCH + c8;
         const float4 a0 = *reinterpret_cast<const float4*>(sp);
         const float4 a1 = *reinterpret_cast<const float4*>(sp + 4);
         float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
         float e[8];
-        char* Cp = Cbase + ((long long)m * d.ldc + wn0 + c8) * CSZ;
+        char* Cp = Cbase + ((long long)m * ldc + wn0 + c8) * CSZ;
         if (CF32) {
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
@@ -377,11 +381,11 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
         const int nl = (pass >> 2) * 64 + lane;
         const int mg = (pass & 3) * 8;
         const int n = wn0 + nl, m = band_m + mg;
-        if (FULL || (n < d.N && m < d.M)) {  // M is a multiple of 8 for symmetric outputs
+        if (FULL || (n < dN && m < dM)) {  // M is a multiple of 8 for symmetric outputs
           float v[8];
 #pragma unroll
           for (int q = 0; q < 8; ++q) v[q] = stg[(mg + q) * PITCH + nl];
-          char* Cp = Cbase + ((long long)n * d.ldc + m) * CSZ;
+          char* Cp = Cbase + ((long long)n * ldc + m) * CSZ;
           if (CF32) {
             const u32x4_t o0 = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
                                 __builtin_bit_cast(unsigned, v[2]), __builtin_bit_cast(unsigned, v[3])};
