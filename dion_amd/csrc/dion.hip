@@ -405,16 +405,15 @@ int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_d
   return da_gemm_bf16(c, s);
 }
 
-// One polishing pass in fp32:  out <- in V(in^T in).  `in` (fp64 or fp32) and `out` (fp32, or the caller's
-// dtype for the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one
-// product with the triangular V -- no serial chain.
-int polish_pass(const void* in, int in_store, void* out, int out_store, float* G, float* V, int batch, int rows,
-                int r, hipStream_t s) {
+// One polishing pass in fp32:  out <- in V(in^T in).  `in` (fp32) and `out` (fp32, or the caller's dtype for
+// the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one product with
+// the triangular V -- no serial chain.
+int polish_pass(const float* in, void* out, int out_store, float* G, float* V, int batch, int rows, int r,
+                hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   Gemm32Desc g{};
   g.batch = batch;
-  g.A = static_cast<const float*>(in); g.B = g.A; g.C = G;
-  g.a_store = in_store; g.b_store = in_store;
+  g.A = in; g.B = in; g.C = G;
   g.sA = pr; g.sB = pr; g.sC = rr;
   g.lda = r; g.ldb = r; g.ldc = r;
   g.M = r; g.N = r; g.K = rows;
@@ -428,7 +427,7 @@ int polish_pass(const void* in, int in_store, void* out, int out_store, float* G
   // out = in V: V is upper triangular, so column tile j only sums k < 64 (j + 1)
   Gemm32Desc a{};
   a.batch = batch;
-  a.A = static_cast<const float*>(in); a.a_store = in_store; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+  a.A = in; a.sA = pr; a.lda = r; a.a_kstrided = 0;
   a.B = V; a.sB = rr; a.ldb = r; a.b_kstrided = 1;
   a.C = static_cast<float*>(out); a.c_store = out_store; a.sC = pr; a.ldc = r;
   a.M = rows; a.N = r; a.K = r; a.alpha = 1.0; a.beta = 0.0; a.k_tri = 1;
@@ -472,8 +471,8 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     const bool last = pass + 1 == passes;
     // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
     float* other = cur == P0f ? reinterpret_cast<float*>(P0) : P0f;
-    rc = polish_pass(cur, DA_STORE_NATIVE, last ? out : static_cast<void*>(other),
-                     last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf, Vf, batch, rows, r, s);
+    rc = polish_pass(cur, last ? out : static_cast<void*>(other), last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf, Vf,
+                     batch, rows, r, s);
     if (rc) return rc;
     cur = other;
   }

@@ -19,17 +19,15 @@ struct RealGemmDesc {
   int split_k;   // > 1: K is cut into that many slices whose partial products are added atomically into a
                  // zeroed C (no E term); the summation order, and so the last bits, vary run to run.
                  // < 0: the launcher picks the slice count for the tile it chooses and clears C itself
-  // Storage of A, B and C when it is not T (DA_STORE_*): the pointers then address elements of that dtype
-  // (cast to T* by the caller), leading dimensions and strides count its elements, operands are widened as
-  // they are fetched and the result is rounded once at the store.  A converted C excludes E, split_k and the
-  // symmetric form.
-  int a_store, b_store, c_store;
+  // Storage of C when it is not T (DA_STORE_*): the pointer then addresses elements of that dtype (cast to T*
+  // by the caller), ldc and sC count its elements and the result is rounded once at the store.  A converted C
+  // excludes E, split_k and the symmetric form.
+  int c_store;
   int k_tri;     // 1: B is block lower triangular -- output column tile j only sums k < 64 (j + 1)
 };
 #define DA_STORE_NATIVE 0
 #define DA_STORE_BF16 1
 #define DA_STORE_F32 2
-#define DA_STORE_F64 3   // operands only (an fp64 matrix read by the fp32 kernel)
 inline int da_store_of(int dtype) { return dtype == DA_BF16 ? DA_STORE_BF16 : DA_STORE_F32; }
 typedef RealGemmDesc<double> Gemm64Desc;
 typedef RealGemmDesc<float> Gemm32Desc;
