@@ -129,6 +129,32 @@ def ptr_array(tensors):
     return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
 
 
+def padded_dims(m, n):
+    """(m, n) rounded up to multiples of 8 (16-byte rows for the kernels) without changing which side is the
+    longer one: the orientation decides the transposes of both optimizers."""
+    m8, n8 = -(-m // 8) * 8, -(-n // 8) * 8
+    if m < n and m8 == n8:
+        n8 += 8
+    if m > n and m8 == n8:
+        m8 += 8
+    return m8, n8
+
+
+def zero_padded(mats, rows, cols):
+    """A (len(mats), rows, cols) tensor holding the 2-D tensors `mats` in its top-left corners, zero elsewhere.
+    Zero rows and columns go through Newton-Schulz and through a Dion step unchanged and change nothing else,
+    so a shape the kernels cannot take directly is stepped on such a copy and cropped back."""
+    out = mats[0].new_zeros((len(mats), rows, cols))
+    for o, t in zip(out, mats):
+        o[: t.size(0), : t.size(1)].copy_(t)
+    return out
+
+
+def crop_back(dst, padded):
+    for d, s in zip(dst, padded):
+        d.copy_(s[: d.size(0), : d.size(1)])
+
+
 class Workspace:
     """A grow-only byte buffer taken from PyTorch's caching allocator (stream-ordered lifetime)."""
 

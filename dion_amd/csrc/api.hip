@@ -438,14 +438,16 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
 namespace {
 
 struct DionLayout {
-  int mp, np, r;        // working orientation: B is mp x np with mp >= np; Q is np x r
+  // working orientation: B is mp x np with mp >= np; Q is np x r.  r is the rank rounded up to a multiple
+  // of 8 (16-byte rows for every working matrix); the extra columns are zero throughout the step.
+  int mp, np, r;
   size_t msz;           // bytes per element of the momentum dtype
   size_t qc, p, rb, qn, orth, small;  // per-matrix byte sizes
   size_t per_matrix;
   DionLayout(int m, int n, int rank, int m_dtype) {
     mp = m < n ? n : m;
     np = m < n ? m : n;
-    r = rank;
+    r = (rank + 7) & ~7;
     msz = m_dtype == DA_BF16 ? 2 : 4;
     qc = (size_t)np * r * msz;   // exact: the orthonormaliser and the GEMMs take these as
     p = (size_t)mp * r * msz;    // contiguous batches (multiples of 128 bytes by the alignment rule)
@@ -499,25 +501,26 @@ int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int 
   int rc = da_fill_int(inf, batch, 0, s);
   if (rc) return rc;
   DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-  return da_orthonormalize(P, out, dtype, batch, rows, r, passes, workspace, inf, s);
+  return da_orthonormalize(P, out, dtype, batch, rows, r, r, passes, workspace, inf, s);
 }
 
 int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
-                       int r, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
+                       int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
                        float scaled_lr, float eps, int faithful, int* info, void* workspace, size_t workspace_bytes,
                        void* stream) {
-  if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || r <= 0) return DA_ERR_ARG;
+  if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || rank <= 0) return DA_ERR_ARG;
   if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype) || !dtype_ok(m_dtype) || !dtype_ok(q_dtype)) return DA_ERR_DTYPE;
   if (m_dtype == DA_F32 && x_dtype != DA_F32) return DA_ERR_DTYPE;  // fp32 products update fp32 weights only
-  if ((m | n | r) & 7) return DA_ERR_ALIGN;
-  if (r > m || r > n) return DA_ERR_ARG;
+  if ((m | n) & 7) return DA_ERR_ALIGN;
+  if (rank > m || rank > n) return DA_ERR_ARG;
   if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
   for (int i = 0; i < batch; ++i) {
     if (!X[i] || !G[i] || !M[i] || !Q[i]) return DA_ERR_ARG;
     if (((uintptr_t)X[i] | (uintptr_t)G[i] | (uintptr_t)M[i] | (uintptr_t)Q[i]) & 15) return DA_ERR_ALIGN;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const DionLayout L(m, n, r, m_dtype);
+  const DionLayout L(m, n, rank, m_dtype);
+  const int r = L.r;   // padded rank: pitch and logical width of Qc, P, R, Qn
   const int chunk = L.chunk(batch, workspace_bytes);
   if (chunk < 1) return DA_ERR_WORKSPACE;
   const bool transposed = m < n;
@@ -559,7 +562,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
       rc = da_add_grad(tm, tg, m_dtype, g_dtype, mn, cb, nonzero, s);
       if (rc) return rc;
       // Q in the momentum dtype   (reference dion/dion.py:1216)
-      rc = da_cast_table(tq, q_dtype, Qc, m_dtype, (long long)np * r, cb, s);
+      rc = da_cast_table(tq, q_dtype, Qc, m_dtype, np, rank, r, cb, s);
       if (rc) return rc;
     }
     GemmDesc g{};
@@ -575,7 +578,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
     {
       DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-      rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, 2, orth_ws, linfo, s);
+      rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, orth_ws, linfo, s);
       if (rc) return rc;
       // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
       rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);
@@ -610,7 +613,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     {
       DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
       // the orthonormaliser is done with its fp64 scratch: reuse its head for the column sums
-      rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, eps, cb, reinterpret_cast<double*>(orth_ws), s);
+      rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, rank, eps, cb, reinterpret_cast<double*>(orth_ws), s);
       if (rc) return rc;
     }
     // ---- X <- (1 - lr wd) X - scaled_lr P Q_new^T  (or Q_new P^T)   (reference dion/dion.py:865-872)

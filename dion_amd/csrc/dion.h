@@ -7,17 +7,21 @@ int da_fill_int(int* p, int n, int v, hipStream_t s);
 int da_write_table(const DaPtrTable& t, void** dst, int n, hipStream_t s);
 int da_add_grad(const DaPtrTable& m, const DaPtrTable& g, int m_dtype, int g_dtype, long long n, int batch,
                 int* nonzero, hipStream_t s);
-int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, long long n, int batch, hipStream_t s);
+// dst[b] (rows x ld, contiguous batch) <- table[b] (rows x cols contiguous), columns beyond cols zeroed; ld % 8 == 0.
+int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, int rows, int cols, int ld, int batch,
+                  hipStream_t s);
 int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const int* nonzero, hipStream_t s);
-// `sums` is scratch for batch * r doubles.
-int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, float eps,
-               int batch, double* sums, hipStream_t s);
+// R, qn: rows x r (r % 8 == 0); the Q state receives the first q_cols columns as a contiguous rows x q_cols
+// matrix.  `sums` is scratch for batch * r doubles.
+int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, int q_cols,
+               float eps, int batch, double* sums, hipStream_t s);
 
 // CholeskyQR (passes = 1) / CholeskyQR2 (passes = 2) of `batch` contiguous matrices P[b]
 // (rows x r, dtype bf16 or f32): one pass with fp64 Gram, Cholesky and triangular solve, then
 // passes - 1 first-order polishing passes in fp32; result in `out` (same dtype and layout, may
 // alias P).  info[b] receives 1 + the first failed pivot
-// column (0 = success); failed columns come out as zeros.
+// column (0 = success); failed columns come out as zeros.  Columns r_live .. r-1 of P are zero
+// padding (r_live == r: none) and stay zero.
 size_t da_orth_workspace_bytes(int batch, int rows, int r);
-int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
-                      int* info, hipStream_t s);
+int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
+                      void* ws, int* info, hipStream_t s);

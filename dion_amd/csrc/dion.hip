@@ -1,7 +1,7 @@
 // Dion step building blocks that are not GEMMs: the momentum accumulation with its all-zero
 // guard, dtype casts, the NaN / all-zero fix-up of P and R, the column normalisation that
-// turns R into the next Q, and the host-side driver of the fp64 CholeskyQR2
-// orthonormalisation (Gram -> blocked Cholesky -> blocked triangular solve, twice).
+// turns R into the next Q, and the host-side driver of the orthonormalisation (one blocked
+// CholeskyQR pass in fp64: Gram -> Cholesky -> triangular solve, then closed-form polishing passes).
 #include "dion.h"
 #include "gemm_f64.h"
 #include "prof.h"
@@ -107,6 +107,21 @@ __global__ __launch_bounds__(256) void cast_table_kernel(DaPtrTable st, TD* dst,
   }
 }
 
+// dst[b] (rows x ld, contiguous, TD) <- src table[b] (rows x cols contiguous, TS); columns cols .. ld-1 are
+// zeroed.  For a column count that is not a multiple of 8: the working copy gets 16-byte rows.
+template <typename TS, typename TD>
+__global__ __launch_bounds__(256) void cast_table_pitched_kernel(DaPtrTable st, TD* dst, int rows, int cols, int ld) {
+  const int b = blockIdx.y;
+  const TS* S = static_cast<const TS*>(st.p[b]);
+  const long long n = (long long)rows * ld;
+  TD* D = dst + (long long)b * n;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const long long row = i / ld;
+    const int c = (int)(i - row * ld);
+    st_from_float<TD>(D + i, c < cols ? ld_as_float<TS>(S + row * cols + c) : 0.f);
+  }
+}
+
 // v <- nan_to_num(v) * nonzero + alt * (1 - nonzero)      (alt may be null: treated as 0)
 template <typename T>
 __global__ __launch_bounds__(256) void fix_kernel(T* V, const T* alt, long long n, const int* nonzero) {
@@ -132,7 +147,8 @@ __global__ __launch_bounds__(256) void fix_kernel(T* V, const T* alt, long long 
 
 // Column normalisation of R[b] (rows x r, TM): Qn = R / (sqrt(sum_rows R^2) + eps), computed in
 // fp32 (column sums accumulated in fp64), stored as TM into qn[b] and, cast to TQ, into the
-// optimizer's Q state.  Two launches: partial column sums over row slices (fp64 atomics into a
+// optimizer's Q state (its first q_cols columns: the working matrices may carry zero columns up to a
+// multiple of 8).  Two launches: partial column sums over row slices (fp64 atomics into a
 // zeroed buffer), then a fully parallel normalise pass.
 template <typename TM>
 __global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, double* __restrict__ sums, int rows, int r,
@@ -160,7 +176,8 @@ __global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, d
 
 template <typename TM, typename TQ>
 __global__ __launch_bounds__(256) void colscale_kernel(const TM* __restrict__ R, TM* __restrict__ qn, DaPtrTable qt,
-                                                       const double* __restrict__ sums, long long n, int r, float eps) {
+                                                       const double* __restrict__ sums, long long n, int r, int q_cols,
+                                                       float eps) {
   const int b = blockIdx.y;
   const TM* Rb = R + (long long)b * n;
   TM* Qn = qn + (long long)b * n;
@@ -177,7 +194,15 @@ __global__ __launch_bounds__(256) void colscale_kernel(const TM* __restrict__ R,
       q[e] = v[e];
     }
     V8<TM>::store(Qn + i, v);
-    V8<TQ>::store(Q + i, q);              // Q <- Q_new.to(Q.dtype) (reference dion/dion.py:1559-1561)
+    // Q <- Q_new.to(Q.dtype) (reference dion/dion.py:1559-1561); the state has q_cols <= r columns, contiguous
+    if (q_cols == r) {
+      V8<TQ>::store(Q + i, q);
+    } else {
+      const long long row = i / r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (c0 + e < q_cols) st_from_float<TQ>(Q + row * q_cols + c0 + e, q[e]);
+    }
   }
 }
 
@@ -221,19 +246,26 @@ int da_add_grad(const DaPtrTable& m, const DaPtrTable& g, int m_dtype, int g_dty
   return da_launch_status();
 }
 
-int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, long long n, int batch, hipStream_t s) {
-  if (n & 7) return DA_ERR_ALIGN;
-  dim3 grid(ew_blocks(n), batch);
-  if (s_dtype == DA_BF16 && d_dtype == DA_BF16)
-    hipLaunchKernelGGL((cast_table_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
-  else if (s_dtype == DA_F32 && d_dtype == DA_BF16)
-    hipLaunchKernelGGL((cast_table_kernel<float, bf16_t>), grid, dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
-  else if (s_dtype == DA_BF16 && d_dtype == DA_F32)
-    hipLaunchKernelGGL((cast_table_kernel<bf16_t, float>), grid, dim3(256), 0, s, src, static_cast<float*>(dst), n);
-  else if (s_dtype == DA_F32 && d_dtype == DA_F32)
-    hipLaunchKernelGGL((cast_table_kernel<float, float>), grid, dim3(256), 0, s, src, static_cast<float*>(dst), n);
-  else
-    return DA_ERR_DTYPE;
+int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, int rows, int cols, int ld, int batch,
+                  hipStream_t s) {
+  if (rows <= 0 || cols <= 0 || ld < cols || (ld & 7)) return DA_ERR_ALIGN;
+  const long long n = (long long)rows * ld;
+  const bool flat = cols == ld;
+  dim3 grid(flat ? ew_blocks(n) : ew_blocks(8 * n), batch);
+#define DA_CAST_CASE(TS, TD)                                                                                      \
+  do {                                                                                                            \
+    if (flat)                                                                                                     \
+      hipLaunchKernelGGL((cast_table_kernel<TS, TD>), grid, dim3(256), 0, s, src, static_cast<TD*>(dst), n);      \
+    else                                                                                                          \
+      hipLaunchKernelGGL((cast_table_pitched_kernel<TS, TD>), grid, dim3(256), 0, s, src, static_cast<TD*>(dst),  \
+                         rows, cols, ld);                                                                         \
+  } while (0)
+  if (s_dtype == DA_BF16 && d_dtype == DA_BF16) DA_CAST_CASE(bf16_t, bf16_t);
+  else if (s_dtype == DA_F32 && d_dtype == DA_BF16) DA_CAST_CASE(float, bf16_t);
+  else if (s_dtype == DA_BF16 && d_dtype == DA_F32) DA_CAST_CASE(bf16_t, float);
+  else if (s_dtype == DA_F32 && d_dtype == DA_F32) DA_CAST_CASE(float, float);
+  else return DA_ERR_DTYPE;
+#undef DA_CAST_CASE
   return da_launch_status();
 }
 
@@ -249,9 +281,9 @@ int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const in
   return da_launch_status();
 }
 
-int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, float eps,
-               int batch, double* sums, hipStream_t s) {
-  if (r & 7) return DA_ERR_ALIGN;
+int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, int q_cols,
+               float eps, int batch, double* sums, hipStream_t s) {
+  if ((r & 7) || q_cols < 1 || q_cols > r) return DA_ERR_ALIGN;
   const long long ns = (long long)batch * r;
   hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, sums, ns);
   int slices = (rows + 255) / 256;
@@ -267,13 +299,13 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
   const long long n = (long long)rows * r;
   dim3 g2(ew_blocks(n), batch);
   if (m_dtype == DA_BF16 && q_dtype == DA_BF16)
-    hipLaunchKernelGGL((colscale_kernel<bf16_t, bf16_t>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<bf16_t, bf16_t>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, q_cols, eps);
   else if (m_dtype == DA_BF16 && q_dtype == DA_F32)
-    hipLaunchKernelGGL((colscale_kernel<bf16_t, float>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<bf16_t, float>), g2, dim3(256), 0, s, static_cast<const bf16_t*>(R), static_cast<bf16_t*>(qn), q, sums, n, r, q_cols, eps);
   else if (m_dtype == DA_F32 && q_dtype == DA_BF16)
-    hipLaunchKernelGGL((colscale_kernel<float, bf16_t>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<float, bf16_t>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, q_cols, eps);
   else if (m_dtype == DA_F32 && q_dtype == DA_F32)
-    hipLaunchKernelGGL((colscale_kernel<float, float>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, eps);
+    hipLaunchKernelGGL((colscale_kernel<float, float>), g2, dim3(256), 0, s, static_cast<const float*>(R), static_cast<float*>(qn), q, sums, n, r, q_cols, eps);
   else
     return DA_ERR_DTYPE;
   return da_launch_status();
@@ -292,8 +324,16 @@ size_t da_orth_workspace_bytes(int batch, int rows, int r) {
 
 namespace {
 
+// G[b][i][i] = 1 for r_live <= i < r: the Gram matrix of a P whose last r - r_live columns are zero becomes
+// block diagonal with an identity block, and the factorisation leaves those columns of P zero.
+__global__ void pad_diag_kernel(double* G, long long rr, int r, int r_live) {
+  const int i = r_live + threadIdx.x;
+  if (i < r) G[blockIdx.x * rr + (long long)i * r + i] = 1.0;
+}
+
 // One blocked CholeskyQR pass in fp64, in place:  P <- P R^-1  with  P^T P = R^T R.
-int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int* info, hipStream_t s) {
+int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int r_live, int* info,
+                hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
@@ -308,6 +348,11 @@ int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows
   g.split_k = -1;   // few output tiles, long K: the launcher slices K until the GPU is full
   int rc = da_gemm_f64(g, s);
   if (rc) return rc;
+  if (r_live < r) {
+    hipLaunchKernelGGL(pad_diag_kernel, dim3((unsigned)batch), dim3(64), 0, s, G, rr, r, r_live);
+    rc = da_launch_status();
+    if (rc) return rc;
+  }
   // blocked lower Cholesky G = L L^T (right-looking), building W alongside
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
@@ -441,9 +486,11 @@ int polish_pass(const float* in, void* out, int out_store, float* G, float* V, i
 // such a matrix the second CholeskyQR pass has a closed form to O(E^2) <= 1e-8 -- below fp32 round-off,
 // which is all the output dtype (fp32 or bf16) can hold: R^-1 = I - up(P^T P - I).  So the later passes
 // are two fp32 products and no factorisation at all; the last one stores the output dtype.
-int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes, void* ws,
-                      int* info, hipStream_t s) {
-  if (passes < 1 || batch > 65535) return DA_ERR_ARG;
+// Columns r_live .. r-1 of P, if any, must be zero on entry and are zero on return (a caller pads the
+// rank to a multiple of 8 this way); the polishing passes multiply them by finite factors only.
+int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
+                      void* ws, int* info, hipStream_t s) {
+  if (passes < 1 || batch > 65535 || r_live < 1 || r_live > r || r - r_live > 63) return DA_ERR_ARG;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   double* P0 = static_cast<double*>(ws);
   double* G = P0 + pr * batch;
@@ -453,7 +500,7 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   bf16_t* P0h = reinterpret_cast<bf16_t*>(P0f + pr * batch);
   int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
   if (rc) return rc;
-  rc = cholqr_pass(P0, G, L, W, batch, rows, r, info, s);
+  rc = cholqr_pass(P0, G, L, W, batch, rows, r, r_live, info, s);
   if (rc) return rc;
   if (passes == 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
   // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products

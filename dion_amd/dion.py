@@ -266,17 +266,28 @@ class Dion(Optimizer):
             info = self._info[(shape, dtype, device)]
             with torch.cuda.device(device), torch.cuda.stream(stream):
                 # contiguous gradient copies and the workspace belong to this stream
+                Xs = plist
                 Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
+                crops = []
+                if m % 8 or n % 8:
+                    # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
+                    m, n = _lib.padded_dims(m, n)
+                    Xw, Gw, Mw = (_lib.zero_padded(t, m, n) for t in (plist, Gs, Ms))
+                    Qw = _lib.zero_padded(Qs, min(m, n), r)
+                    crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
+                    Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
                 ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
                 rc = lib.dion_amd_dion_step(
-                    _lib.ptr_array(plist), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
+                    _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
                     len(plist), m, n, r,
                     _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
                     ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1,
                     info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
                 )
                 _lib.check(rc, "dion_amd_dion_step")
-                del Gs
+                for dst, padded in crops:
+                    _lib.crop_back(dst, padded)
+                del Xs, Gs, Ms, Qs, crops
         for main, stream in forked.values():
             main.wait_stream(stream)
 

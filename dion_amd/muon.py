@@ -178,6 +178,7 @@ class Muon(Optimizer):
         # products are grouped launches, so small buckets share the GPU instead of queueing
         # (the reference overlaps them as async tasks, dion/muon.py:185-270).
         fused = defaultdict(list)
+        crops = []
         for (shape, dtype, gdtype, device), plist in buckets.items():
             states = [self._get_or_initialize_state(p, "muon") for p in plist]
             adjusted_lr = lr if adjust is None else _ADJUST[adjust](lr, shape)
@@ -186,6 +187,14 @@ class Muon(Optimizer):
                 continue
             _lib.require_gpu(plist[0], "Muon.step")
             X, G, M = self._matrix_views(plist, states, group["flatten"])
+            m, n = X[0].shape
+            if m % 8 or n % 8:
+                # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
+                m8, n8 = _lib.padded_dims(m, n)
+                Xw, Gw, Mw = (_lib.zero_padded(t, m8, n8) for t in (X, G, M))
+                crops.append((X, Xw))
+                crops.append((M, Mw))
+                X, G, M = list(Xw.unbind(0)), list(Gw.unbind(0)), list(Mw.unbind(0))
             fused[(dtype, gdtype, device)].append((X, G, M, float(adjusted_lr)))
 
         decay = 1 - lr * weight_decay
@@ -211,6 +220,8 @@ class Muon(Optimizer):
                 )
             _lib.check(rc, "dion_amd_muon_step_buckets")
             del keep
+        for dst, padded in crops:
+            _lib.crop_back(dst, padded)
 
     @staticmethod
     def _matrix_views(plist: List[Tensor], states: List[dict], flatten: bool):

@@ -49,6 +49,11 @@ def newton_schulz(
     G3 = G.reshape(-1, shape[-2], shape[-1]) if G.ndim == 2 else G
     if G3.stride(-1) != 1 or G3.stride(-2) != G3.size(-1) or (G3.size(0) > 1 and G3.stride(0) != G3.size(1) * G3.size(2)):
         G3 = G3.contiguous()
+    if G3.size(1) % 8 or G3.size(2) % 8:
+        # zero rows and columns stay zero through the iteration and change neither the norm nor the products
+        padded = _lib.zero_padded(list(G3.unbind(0)), *_lib.padded_dims(G3.size(1), G3.size(2)))
+        res = newton_schulz(padded, epsilon, coeffs, compute_dtype, faithful)
+        return res[:, : G3.size(1), : G3.size(2)].reshape(shape)
     batch, m, n = G3.shape
     out = torch.empty((batch, m, n), dtype=compute_dtype, device=G.device)
     cd = _lib.dtype_code(compute_dtype)

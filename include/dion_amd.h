@@ -213,7 +213,10 @@ size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype
  *   M <- B - (1-mu) P R^T  (transposed back when m < n);   Q <- R / (||R||_col + eps);
  *   X <- decay X - scaled_lr P Q^T.
  * ef_alpha = -(1 - mu), decay = 1 - lr*wd and scaled_lr = sqrt(m/n)*lr are passed as
- * already-evaluated fp32 values.  m_dtype f32 requires x_dtype f32.  info as above. */
+ * already-evaluated fp32 values.  m_dtype f32 requires x_dtype f32.  info as above.
+ * m and n must be multiples of 8 (the host side pads other shapes with zero rows / columns,
+ * which changes no result); the rank r is any value in 1 .. min(m, n): the working matrices
+ * carry zero columns up to the next multiple of 8 and Q keeps its r contiguous columns. */
 int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q,
                        int batch, int m, int n, int r,
                        int x_dtype, int g_dtype, int m_dtype, int q_dtype,

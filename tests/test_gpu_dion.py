@@ -17,7 +17,7 @@ def _sign_align(a, ref):
     return a.double() * s
 
 
-@pytest.mark.parametrize("rows,r", [(768, 192), (3072, 768), (768, 768), (520, 72), (4096, 512), (100, 28)])
+@pytest.mark.parametrize("rows,r", [(768, 192), (3072, 768), (768, 768), (520, 72), (4096, 512), (100, 28), (100, 27)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_orthonormalize(dev, rows, r, dtype):
     from dion_amd.newton_schulz import orthonormalize
@@ -139,6 +139,40 @@ def test_dion_fp32_matches_oracle_10_steps(dev, shapes, rank_fraction):
         assert int(info.abs().sum().item()) == 0
 
     _run_dion(dev, shapes, rank_fraction, 10, torch.float32, torch.float32, torch.float32, check=check)
+
+
+@pytest.mark.parametrize("shapes,rank_fraction", [
+    ([(768, 768), (1536, 768), (768, 1536)], 0.3),      # r = 231: aligned matrices, rank off the 8-grid
+    ([(100, 60), (60, 100), (50, 50), (101, 100)], 0.45),  # r = 27 / 27 / 23 / 45: nothing on the grid
+])
+def test_dion_shapes_and_ranks_off_the_alignment_grid(dev, shapes, rank_fraction):
+    """Ranks that are not multiples of 8 run with zero columns up to the next multiple inside the library, other
+    matrix dimensions on zero-padded copies made by the host side: same 1e-4 bar as any other shape."""
+    def check(step, params, opt, Xo, Mo, Qo):
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            assert st["Q"].shape == Qo[i].shape and st["momentum"].shape == p.shape
+            eM = rel_fro(st["momentum"], Mo[i])
+            eX = rel_fro(p.detach(), Xo[i])
+            eQ = rel_fro(_sign_align(st["Q"].cpu(), Qo[i]), Qo[i])
+            assert eM <= FP32_TOL and eX <= FP32_TOL and eQ <= FP32_TOL, (step, i, eM, eX, eQ)
+        info = torch.cat([v for v in opt.cholesky_info().values()])
+        assert int(info.abs().sum().item()) == 0
+
+    _run_dion(dev, shapes, rank_fraction, 5, torch.float32, torch.float32, torch.float32, check=check)
+
+
+def test_dion_bf16_off_the_alignment_grid(dev):
+    """The bf16 configuration (bf16 weights and momentum, fp32 Q) at a rank and at dimensions off the 8-grid."""
+    def check(step, params, opt, Xo, Mo, Qo):
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            eM, eX = rel_fro(st["momentum"], Mo[i]), rel_fro(p.detach(), Xo[i])
+            assert eM <= 1e-2 and eX <= 1e-2, (step, i, eM, eX)
+            assert (st["Q"].double().norm(dim=0) - 1).abs().max().item() < 1e-2
+
+    _run_dion(dev, [(768, 768), (300, 100), (100, 300)], 0.3, 5, torch.bfloat16, torch.bfloat16, torch.float32,
+              check=check)
 
 
 def test_dion_fp32_full_rank(dev):

@@ -60,6 +60,38 @@ def test_muon_step_matches_oracle(dev, dtype, nesterov):
     assert all(g["step"] == 3 for g in opt.param_groups)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_muon_shapes_off_the_alignment_grid(dev, dtype):
+    """Dimensions that are not multiples of 8 (a flattened 3x3 convolution over 3 channels, odd square and tall
+    matrices) are stepped on zero-padded copies: momentum bit exact, update within the NS bar, as for any shape."""
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    shapes = [(64, 27), (27, 64), (77, 77), (301, 100), (100, 301), (301, 100)]
+    X0, gen = _make(shapes, dtype, seed=5)
+    Xo = [x.clone() for x in X0]
+    Mo = [torch.zeros_like(x) for x in X0]
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    lr, mu, wd = 0.02, 0.95, 0.01
+    opt = Muon(params, lr=lr, mu=mu, weight_decay=wd, nesterov=True)
+    for step in range(2):
+        G = _grads(shapes, gen, dtype)
+        for p, g in zip(params, G):
+            p.grad = g.to(dev)
+        prev = [x.clone() for x in Xo]
+        O.muon_step(Xo, G, Mo, lr=lr, mu=mu, weight_decay=wd, epsilon=1e-8, nesterov=True)
+        opt.step()
+        for i, p in enumerate(params):
+            assert torch.equal(opt.state[p]["momentum"].cpu(), Mo[i]), (i, step)
+            decay = (1 - torch.tensor(lr) * torch.tensor(wd)).item()
+            upd_ref = prev[i].double() * decay - Xo[i].double()
+            if dtype == torch.float32:
+                assert rel_fro(prev[i].double() * decay - p.detach().cpu().double(), upd_ref) <= 2e-2, (i, step)
+            bound = 2e-2 * (upd_ref.norm() / Xo[i].double().norm()).item()
+            assert rel_fro(p.detach(), Xo[i]) <= bound + (4e-3 if dtype == torch.bfloat16 else 1e-6), (i, step)
+            p.data.copy_(Xo[i])
+
+
 def test_muon_bf16_single_step_bits(dev):
     """With bf16 weights the update is a few ulps per element; on one step from identical state at
     least 85% of the weights must be bit-identical to the oracle's (the ~1e-2 NS noise flips some roundings)

@@ -18,7 +18,8 @@ def _orth_err(X):
     return s.min().item(), s.max().item()
 
 
-@pytest.mark.parametrize("m,n", [(768, 3072), (3072, 768), (768, 768), (256, 1024), (256, 256), (1024, 4096), (136, 200)])
+@pytest.mark.parametrize("m,n", [(768, 3072), (3072, 768), (768, 768), (256, 1024), (256, 256), (1024, 4096), (136, 200),
+                                 (100, 301), (301, 100), (77, 77), (64, 27)])
 def test_ns_bf16_schedule_vs_oracle(dev, m, n):
     from dion_amd import zeropower_via_newtonschulz5
     from oracle import newton_schulz as O
