@@ -9,9 +9,9 @@
 // 32 x 32 as 2 x 2 accumulators of 16 x 16.  LDS tiles are k-major [16][64] doubles for
 // either operand layout, so the one-double-per-lane MFMA operands are conflict-free reads.
 // Double buffered: the global loads of the next stage are in flight during the MFMAs.
-// Operands may be stored narrower (bf16, fp32) or wider (fp64 into the fp32 instance) than the
-// compute type and the result may be stored as fp32 or bf16; a block-triangular B operand
-// shortens the sum per column tile.
+// The same template is instantiated for fp32 (v_mfma_f32_16x16x4_f32; the polishing passes); the
+// result may be stored as fp32 or bf16, and a block-triangular B operand shortens the sum per
+// column tile.
 #include "gemm_f64.h"
 
 namespace {
@@ -60,8 +60,7 @@ __device__ __forceinline__ void put(T* lds, const T (&v)[4], int tid) {
   }
 }
 
-// BTt x BTt output tile (64 or 128), 256 threads as 2 x 2 wavefronts of (BTt / 2) x (BTt / 2) each.  The larger
-// tile halves the operand bytes per flop: the 64-wide one is bound by the L2 -> LDS path on large products.
+// BTt x BTt output tile, 256 threads as 2 x 2 wavefronts of (BTt / 2) x (BTt / 2) each.
 template <typename T, bool A_KS, bool B_KS, bool SYM, int BTt>
 __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
   typedef typename Mfma<T>::acc_t acc_t;
