@@ -442,7 +442,7 @@ struct DionLayout {
   // of 8 (16-byte rows for every working matrix); the extra columns are zero throughout the step.
   int mp, np, r;
   size_t msz;           // bytes per element of the momentum dtype
-  size_t qc, p, rb, qn, orth, small;  // per-matrix byte sizes
+  size_t qc, p, rb, qn, orth, part, small;  // per-matrix byte sizes
   size_t per_matrix;
   DionLayout(int m, int n, int rank, int m_dtype) {
     mp = m < n ? n : m;
@@ -454,8 +454,10 @@ struct DionLayout {
     rb = qc;
     qn = qc;
     orth = align_up(da_orth_workspace_bytes(1, mp, r), 256);
+    // fp32 partial sums of R = B^T P when its inner dimension is cut into DA_MAX_GROUPS slices (bf16 only)
+    part = m_dtype == DA_BF16 ? (size_t)DA_MAX_GROUPS * np * r * sizeof(float) : 0;
     small = 256;  // flags, info, pointer-table slots
-    per_matrix = qc + p + rb + qn + orth + small + 256;
+    per_matrix = qc + p + rb + qn + orth + part + small + 256;
   }
   size_t fixed() const { return 4 * DA_MAX_PTRS * sizeof(void*) + 2 * DA_MAX_PTRS * sizeof(int) + 1024; }
   int chunk(int batch, size_t ws_bytes) const {
@@ -536,13 +538,16 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     void** tabX = reinterpret_cast<void**>(w); w += DA_MAX_PTRS * sizeof(void*);
     w += 2 * DA_MAX_PTRS * sizeof(void*);
     int* nonzero = reinterpret_cast<int*>(w); w += DA_MAX_PTRS * sizeof(int);
-    int* linfo = reinterpret_cast<int*>(w); w += DA_MAX_PTRS * sizeof(int);
+    // the orthonormaliser's status words go straight to the caller's array when there is one
+    int* linfo = info ? info + b0 : reinterpret_cast<int*>(w);
+    w += DA_MAX_PTRS * sizeof(int);
     w = static_cast<char*>(workspace) + L.fixed();
     char* Qc = w; w += L.qc * cb;
     char* P = w; w += L.p * cb;
     char* R = w; w += L.rb * cb;
     char* Qn = w; w += L.qn * cb;
     char* orth_ws = reinterpret_cast<char*>(align_up(reinterpret_cast<uintptr_t>(w), 256));
+    float* parts = reinterpret_cast<float*>(orth_ws + L.orth * cb);
     const long long sQ = (long long)(L.qc / L.msz), sP = (long long)(L.p / L.msz);
 
     DaPtrTable tx{}, tg{}, tm{}, tq{};
@@ -552,11 +557,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     int rc;
     {
       DaProfScope prof(DA_PROF_DION_ELEM, (double)mn * (2 * msz + gsz) * cb, s);
-      rc = da_fill_int(nonzero, 2 * DA_MAX_PTRS, 0, s);  // nonzero[] and linfo[] are adjacent
-      if (rc) return rc;
-      rc = da_write_table(tm, tabM, cb, s);
-      if (rc) return rc;
-      rc = da_write_table(tx, tabX, cb, s);
+      rc = da_dion_setup(tm, tabM, tx, tabX, cb, nonzero, linfo, s);
       if (rc) return rc;
       // B = M + G, kept in M   (reference dion/dion.py:794)
       rc = da_add_grad(tm, tg, m_dtype, g_dtype, mn, cb, nonzero, s);
@@ -592,9 +593,34 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     g.C = R; g.sC = sQ; g.ldc = r; g.c_dtype = m_dtype;
     g.M = np; g.N = r; g.K = mp;
     g.epilogue = DA_EPI_STORE; g.s1 = 1.f;
-    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BTP);
-    if (rc) return rc;
-    {
+    // A few output tiles with a long inner dimension (tall matrices at a low rank) leave most of the GPU idle:
+    // cut the inner dimension into slices that run side by side as the groups of one launch and leave fp32
+    // partial sums, which the fix-up pass that follows adds and rounds.
+    int slices = 1;
+    if (m_dtype == DA_BF16) {
+      const long long tiles = (long long)((np + 127) / 128) * ((r + 127) / 128) * cb;
+      while (slices < DA_MAX_GROUPS && tiles * slices < 384 && mp / (slices * 2) >= 512 && mp % (slices * 2 * 64) == 0)
+        slices *= 2;
+    }
+    if (slices > 1) {
+      GemmDesc gs[DA_MAX_GROUPS];
+      const int kslice = mp / slices;
+      const long long pstride = (long long)cb * sQ;
+      for (int k = 0; k < slices; ++k) {
+        gs[k] = g;
+        gs[k].K = kslice;
+        gs[k].a_off = (long long)k * kslice * (g.a_kstrided ? n : 1);
+        gs[k].B = P + (size_t)k * kslice * r * L.msz;
+        gs[k].C = parts + k * pstride; gs[k].c_dtype = DA_F32; gs[k].faithful = 0;
+      }
+      rc = gemm_group(gs, slices, m_dtype, s, DA_PROF_DION_BTP);
+      if (rc) return rc;
+      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+      rc = da_fix_sum(parts, slices, pstride, R, Qc, m_dtype, sQ, cb, nonzero, s);
+      if (rc) return rc;
+    } else {
+      rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BTP);
+      if (rc) return rc;
       DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
       rc = da_fix(R, Qc, m_dtype, sQ, cb, nonzero, s);
       if (rc) return rc;
@@ -627,10 +653,6 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     rc = gemm_any(g, m_dtype, s, DA_PROF_DION_UPD);
     if (rc) return rc;
     (void)xsz;
-    if (info) {
-      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
-      DA_HIP_CHECK(hipMemcpyAsync(info + b0, linfo, cb * sizeof(int), hipMemcpyDeviceToDevice, s));
-    }
   }
   return DA_OK;
 }

@@ -73,6 +73,7 @@ struct GemmDesc {
   const void* const* Btab;
   void* const* Ctab;
   const void* const* Etab;
+  long long a_off;    // elements added to Atab[b]: a K-slice of operands that are addressed through the table (bf16 kernel)
   long long sA, sB, sC, sE;  // batch strides
   int lda, ldb, ldc, lde;
   int M, N, K;

@@ -4,13 +4,19 @@
 #include "elementwise.h"
 
 int da_fill_int(int* p, int n, int v, hipStream_t s);
-int da_write_table(const DaPtrTable& t, void** dst, int n, hipStream_t s);
+// dst_a[i] = ta.p[i], dst_b[i] = tb.p[i], nonzero[i] = info[i] = 0 for i < n <= DA_MAX_PTRS, in one launch.
+int da_dion_setup(const DaPtrTable& ta, void** dst_a, const DaPtrTable& tb, void** dst_b, int n, int* nonzero,
+                  int* info, hipStream_t s);
 int da_add_grad(const DaPtrTable& m, const DaPtrTable& g, int m_dtype, int g_dtype, long long n, int batch,
                 int* nonzero, hipStream_t s);
 // dst[b] (rows x ld, contiguous batch) <- table[b] (rows x cols contiguous), columns beyond cols zeroed; ld % 8 == 0.
 int da_cast_table(const DaPtrTable& src, int s_dtype, void* dst, int d_dtype, int rows, int cols, int ld, int batch,
                   hipStream_t s);
 int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const int* nonzero, hipStream_t s);
+// v[b] <- fix(round(part[0][b] + ... + part[parts-1][b])): the partial sums (fp32, n elements per matrix, slice k
+// at part + k * pstride) of a product whose inner dimension was cut into slices.
+int da_fix_sum(const float* part, int parts, long long pstride, void* v, const void* alt, int dtype, long long n,
+               int batch, const int* nonzero, hipStream_t s);
 // R, qn: rows x r (r % 8 == 0); the Q state receives the first q_cols columns as a contiguous rows x q_cols
 // matrix.  `sums` is scratch for batch * r doubles.
 int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, int q_cols,

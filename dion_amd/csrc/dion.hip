@@ -68,8 +68,16 @@ __global__ void fill_int_kernel(int* p, int n, int v) {
   if (i < n) p[i] = v;
 }
 
-__global__ void write_table_kernel(DaPtrTable t, void** dst, int n) {
-  if ((int)threadIdx.x < n) dst[threadIdx.x] = t.p[threadIdx.x];
+// Start of a bucket chunk in one launch: the two device pointer tables and the cleared per-matrix words.
+__global__ void dion_setup_kernel(DaPtrTable ta, void** dst_a, DaPtrTable tb, void** dst_b, int n, int* nonzero,
+                                  int* info) {
+  const int i = threadIdx.x;
+  if (i < n) {
+    dst_a[i] = ta.p[i];
+    dst_b[i] = tb.p[i];
+    nonzero[i] = 0;
+    info[i] = 0;
+  }
 }
 
 // M <- M + G (rounded to M's dtype); nonzero[b] |= any(M != 0).
@@ -136,6 +144,38 @@ __global__ __launch_bounds__(256) void fix_kernel(T* V, const T* alt, long long 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float x = v[e];
+      if (x != x) x = 0.f;
+      else if (x > V8<T>::maxval()) x = V8<T>::maxval();
+      else if (x < -V8<T>::maxval()) x = -V8<T>::maxval();
+      v[e] = nz ? x : (a ? q[e] : 0.f);
+    }
+    V8<T>::store(p + i, v);
+  }
+}
+
+// The same fix-up for a product that was computed as `parts` partial sums over slices of its inner dimension
+// (fp32, `pstride` elements apart): v <- round(sum of the parts), then as fix_kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void fix_sum_kernel(const float* __restrict__ part, int parts, long long pstride,
+                                                      T* V, const T* alt, long long n, const int* nonzero) {
+  const int b = blockIdx.y;
+  const bool nz = nonzero[b] != 0;
+  T* p = V + (long long)b * n;
+  const float* s0 = part + (long long)b * n;
+  const T* a = alt ? alt + (long long)b * n : nullptr;
+  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < n; i += (long long)gridDim.x * 256 * 8) {
+    float v[8], q[8];
+    V8<float>::load(s0 + i, v);
+    for (int k = 1; k < parts; ++k) {
+      float t[8];
+      V8<float>::load(s0 + k * pstride + i, t);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] += t[e];
+    }
+    if (a && !nz) V8<T>::load(a + i, q);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float x = V8<T>::round(v[e]);
       if (x != x) x = 0.f;
       else if (x > V8<T>::maxval()) x = V8<T>::maxval();
       else if (x < -V8<T>::maxval()) x = -V8<T>::maxval();
@@ -223,9 +263,10 @@ int da_fill_int(int* p, int n, int v, hipStream_t s) {
   return da_launch_status();
 }
 
-int da_write_table(const DaPtrTable& t, void** dst, int n, hipStream_t s) {
-  if (n > DA_MAX_PTRS) return DA_ERR_LIMIT;
-  hipLaunchKernelGGL(write_table_kernel, dim3(1), dim3(64), 0, s, t, dst, n);
+int da_dion_setup(const DaPtrTable& ta, void** dst_a, const DaPtrTable& tb, void** dst_b, int n, int* nonzero,
+                  int* info, hipStream_t s) {
+  if (n < 1 || n > DA_MAX_PTRS) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL(dion_setup_kernel, dim3(1), dim3(64), 0, s, ta, dst_a, tb, dst_b, n, nonzero, info);
   return da_launch_status();
 }
 
@@ -281,13 +322,27 @@ int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const in
   return da_launch_status();
 }
 
+int da_fix_sum(const float* part, int parts, long long pstride, void* v, const void* alt, int dtype, long long n,
+               int batch, const int* nonzero, hipStream_t s) {
+  if ((n & 7) || (pstride & 7) || parts < 1) return DA_ERR_ALIGN;
+  dim3 grid(ew_blocks(n), batch);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL(fix_sum_kernel<bf16_t>, grid, dim3(256), 0, s, part, parts, pstride, static_cast<bf16_t*>(v), static_cast<const bf16_t*>(alt), n, nonzero);
+  else if (dtype == DA_F32)
+    hipLaunchKernelGGL(fix_sum_kernel<float>, grid, dim3(256), 0, s, part, parts, pstride, static_cast<float*>(v), static_cast<const float*>(alt), n, nonzero);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+
 int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, int q_cols,
                float eps, int batch, double* sums, hipStream_t s) {
   if ((r & 7) || q_cols < 1 || q_cols > r) return DA_ERR_ALIGN;
   const long long ns = (long long)batch * r;
   hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, sums, ns);
-  int slices = (rows + 255) / 256;
-  if (slices > 64) slices = 64;
+  // 64 rows per workgroup (16 per row group): enough workgroups to pull R at the memory system's rate
+  int slices = (rows + 63) / 64;
+  if (slices > 1024) slices = 1024;
   const int rps = (rows + slices - 1) / slices;
   dim3 g1((r + 63) / 64, slices, batch);
   if (m_dtype == DA_BF16)

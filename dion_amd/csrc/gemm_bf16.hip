@@ -459,7 +459,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0);
   const int b = tile.b, ti = tile.ti, tj = tile.tj;
   const int m0 = ti * BT, n0 = tj * BT;
-  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
+  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) + d.a_off : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
   const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
 
   f32x16_t acc[TMI][TNJ];
@@ -660,7 +660,8 @@ int check_desc(const GemmDesc& d) {
   if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
   if (d.c_dtype != DA_BF16 && d.c_dtype != DA_F32) return DA_ERR_DTYPE;
   if ((d.K | d.N | d.lda | d.ldb | d.ldc) & 7) return DA_ERR_ALIGN;
-  if ((d.sA | d.sB | d.sC) & 7) return DA_ERR_ALIGN;
+  if ((d.sA | d.sB | d.sC | d.a_off) & 7) return DA_ERR_ALIGN;
+  if (d.a_off && !d.Atab) return DA_ERR_ARG;
   if ((d.E || d.Etab) && ((d.lde & 7) || (d.sE & 7))) return DA_ERR_ALIGN;
   if (d.a_kstrided && (d.M & 7)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;

@@ -260,9 +260,9 @@ int launch_bt(const RealGemmDesc<T>& d, int split, hipStream_t s) {
 
 template <typename T, bool A_KS, bool B_KS, bool SYM>
 int launch(const RealGemmDesc<T>& d, hipStream_t s) {
-  // Only the 64-wide tile is instantiated: the 128-wide one (half the operand bytes per flop, but 198 VGPRs
-  // and 64 KB of LDS in fp64, i.e. two workgroups per CU instead of five) measured 10-20 % slower on the
-  // orthonormaliser's products.
+  // Only the 64-wide tile is instantiated: the 128-wide one (half the operand bytes per flop, but 200 VGPRs
+  // and 64 KB of LDS in fp64, i.e. two workgroups per CU instead of five) measured 10 % slower on the
+  // orthonormaliser's large products and equal on the small ones.
   constexpr int BTt = 64;
   const long long blocks = blocks_of<T, BTt>(d);
   const bool auto_split = d.split_k < 0 && !d.E && d.c_store == DA_STORE_NATIVE;
