@@ -528,7 +528,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
   const bool transposed = m < n;
   const int mp = L.mp, np = L.np;
   const long long mn = (long long)m * n;
-  const double msz = (double)L.msz, xsz = x_dtype == DA_BF16 ? 2 : 4, gsz = g_dtype == DA_BF16 ? 2 : 4;
+  const double msz = (double)L.msz, gsz = g_dtype == DA_BF16 ? 2 : 4;
 
   for (int b0 = 0; b0 < batch; b0 += chunk) {
     const int cb = batch - b0 < chunk ? batch - b0 : chunk;
@@ -652,7 +652,6 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
     g.epilogue = DA_EPI_AXPBY; g.s0 = decay; g.s1 = -scaled_lr;
     rc = gemm_any(g, m_dtype, s, DA_PROF_DION_UPD);
     if (rc) return rc;
-    (void)xsz;
   }
   return DA_OK;
 }
