@@ -508,9 +508,10 @@ int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int 
 
 int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
                        int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
-                       float scaled_lr, float eps, int faithful, int* info, void* workspace, size_t workspace_bytes,
-                       void* stream) {
+                       float scaled_lr, float eps, int faithful, int power_iters, int* info, void* workspace,
+                       size_t workspace_bytes, void* stream) {
   if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || rank <= 0) return DA_ERR_ARG;
+  if (power_iters < 1 || power_iters > 64) return DA_ERR_ARG;
   if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype) || !dtype_ok(m_dtype) || !dtype_ok(q_dtype)) return DA_ERR_DTYPE;
   if (m_dtype == DA_F32 && x_dtype != DA_F32) return DA_ERR_DTYPE;  // fp32 products update fp32 weights only
   if ((m | n) & 7) return DA_ERR_ALIGN;
@@ -567,64 +568,70 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
       if (rc) return rc;
     }
     GemmDesc g{};
-    g.batch = cb; g.faithful = faithful;
-    // ---- P = B Q   (reference dion/dion.py:801); B is M (mp x np) or M^T when m < n
-    g.Atab = const_cast<const void* const*>(tabM); g.A = nullptr; g.lda = n; g.a_kstrided = transposed ? 1 : 0;
-    g.B = Qc; g.sB = sQ; g.ldb = r; g.b_kstrided = 1;
-    g.C = P; g.sC = sP; g.ldc = r; g.c_dtype = m_dtype;
-    g.M = mp; g.N = r; g.K = np;
-    g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
-    rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
-    if (rc) return rc;
-    // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
-    {
-      DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-      rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, orth_ws, linfo, s);
+    // One power iteration is the reference's batched step (dion/dion.py:801-839); more of them repeat
+    // P = orth(B Q), Q = B^T P with the unnormalised R as the next Q (dion/dion_reference.py:712-730).  The
+    // all-zero / NaN guard runs in every round: between rounds it only matters for an all-zero or non-finite B.
+    for (int it = 0; it < power_iters; ++it) {
+      g = GemmDesc{};
+      g.batch = cb; g.faithful = faithful;
+      // ---- P = B Q   (reference dion/dion.py:801); B is M (mp x np) or M^T when m < n
+      g.Atab = const_cast<const void* const*>(tabM); g.A = nullptr; g.lda = n; g.a_kstrided = transposed ? 1 : 0;
+      g.B = it == 0 ? Qc : R; g.sB = sQ; g.ldb = r; g.b_kstrided = 1;
+      g.C = P; g.sC = sP; g.ldc = r; g.c_dtype = m_dtype;
+      g.M = mp; g.N = r; g.K = np;
+      g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
+      rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
       if (rc) return rc;
-      // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
-      rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);
-      if (rc) return rc;
-    }
-    // ---- R = B^T P   (reference dion/dion.py:839)
-    g = GemmDesc{};
-    g.batch = cb; g.faithful = faithful;
-    g.Atab = const_cast<const void* const*>(tabM); g.lda = n; g.a_kstrided = transposed ? 0 : 1;
-    g.B = P; g.sB = sP; g.ldb = r; g.b_kstrided = 1;
-    g.C = R; g.sC = sQ; g.ldc = r; g.c_dtype = m_dtype;
-    g.M = np; g.N = r; g.K = mp;
-    g.epilogue = DA_EPI_STORE; g.s1 = 1.f;
-    // A few output tiles with a long inner dimension (tall matrices at a low rank) leave most of the GPU idle:
-    // cut the inner dimension into slices that run side by side as the groups of one launch and leave fp32
-    // partial sums, which the fix-up pass that follows adds and rounds.
-    int slices = 1;
-    if (m_dtype == DA_BF16) {
-      const long long tiles = (long long)((np + 127) / 128) * ((r + 127) / 128) * cb;
-      while (slices < DA_MAX_GROUPS && tiles * slices < 384 && mp / (slices * 2) >= 512 && mp % (slices * 2 * 64) == 0)
-        slices *= 2;
-    }
-    if (slices > 1) {
-      GemmDesc gs[DA_MAX_GROUPS];
-      const int kslice = mp / slices;
-      const long long pstride = (long long)cb * sQ;
-      for (int k = 0; k < slices; ++k) {
-        gs[k] = g;
-        gs[k].K = kslice;
-        gs[k].a_off = (long long)k * kslice * (g.a_kstrided ? n : 1);
-        gs[k].B = P + (size_t)k * kslice * r * L.msz;
-        gs[k].C = parts + k * pstride; gs[k].c_dtype = DA_F32; gs[k].faithful = 0;
+      // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
+      {
+        DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
+        rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, orth_ws, linfo, s);
+        if (rc) return rc;
+        // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
+        rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);
+        if (rc) return rc;
       }
-      rc = gemm_group(gs, slices, m_dtype, s, DA_PROF_DION_BTP);
-      if (rc) return rc;
-      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
-      rc = da_fix_sum(parts, slices, pstride, R, Qc, m_dtype, sQ, cb, nonzero, s);
-      if (rc) return rc;
-    } else {
-      rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BTP);
-      if (rc) return rc;
-      DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
-      rc = da_fix(R, Qc, m_dtype, sQ, cb, nonzero, s);
-      if (rc) return rc;
-    }
+      // ---- R = B^T P   (reference dion/dion.py:839)
+      g = GemmDesc{};
+      g.batch = cb; g.faithful = faithful;
+      g.Atab = const_cast<const void* const*>(tabM); g.lda = n; g.a_kstrided = transposed ? 0 : 1;
+      g.B = P; g.sB = sP; g.ldb = r; g.b_kstrided = 1;
+      g.C = R; g.sC = sQ; g.ldc = r; g.c_dtype = m_dtype;
+      g.M = np; g.N = r; g.K = mp;
+      g.epilogue = DA_EPI_STORE; g.s1 = 1.f;
+      // A few output tiles with a long inner dimension (tall matrices at a low rank) leave most of the GPU idle:
+      // cut the inner dimension into slices that run side by side as the groups of one launch and leave fp32
+      // partial sums, which the fix-up pass that follows adds and rounds.
+      int slices = 1;
+      if (m_dtype == DA_BF16) {
+        const long long tiles = (long long)((np + 127) / 128) * ((r + 127) / 128) * cb;
+        while (slices < DA_MAX_GROUPS && tiles * slices < 384 && mp / (slices * 2) >= 512 && mp % (slices * 2 * 64) == 0)
+          slices *= 2;
+      }
+      if (slices > 1) {
+        GemmDesc gs[DA_MAX_GROUPS];
+        const int kslice = mp / slices;
+        const long long pstride = (long long)cb * sQ;
+        for (int k = 0; k < slices; ++k) {
+          gs[k] = g;
+          gs[k].K = kslice;
+          gs[k].a_off = (long long)k * kslice * (g.a_kstrided ? n : 1);
+          gs[k].B = P + (size_t)k * kslice * r * L.msz;
+          gs[k].C = parts + k * pstride; gs[k].c_dtype = DA_F32; gs[k].faithful = 0;
+        }
+        rc = gemm_group(gs, slices, m_dtype, s, DA_PROF_DION_BTP);
+        if (rc) return rc;
+        DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+        rc = da_fix_sum(parts, slices, pstride, R, Qc, m_dtype, sQ, cb, nonzero, s);
+        if (rc) return rc;
+      } else {
+        rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BTP);
+        if (rc) return rc;
+        DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+        rc = da_fix(R, Qc, m_dtype, sQ, cb, nonzero, s);
+        if (rc) return rc;
+      }
+    }  // power iterations
     // ---- error feedback  M <- M - (1 - mu) P R^T  (or R P^T)   (reference dion/dion.py:851-853)
     g = GemmDesc{};
     g.batch = cb; g.faithful = faithful;

@@ -34,6 +34,7 @@ class DionMixedPrecisionConfig:
 
 
 class Dion(Optimizer):
+    _REFERENCE_OPTIONS = False   # True in DionReference: power_iters >= 1 and all three qr_method names
     """
     Dion (https://arxiv.org/abs/2504.05295) for a single MI355X.
 
@@ -81,10 +82,17 @@ class Dion(Optimizer):
             raise ValueError(f"Invalid rank fraction: {rank_fraction}")
         if rank_multiple_of <= 0:
             raise ValueError(f"Invalid rank multiple of: {rank_multiple_of}")
-        if power_iters != 1:
-            raise ValueError("Async Dion only supports power_iters=1")
-        if qr_method != "rcqr":
-            raise ValueError("Async Dion only supports qr_method='rcqr'")
+        if self._REFERENCE_OPTIONS:
+            # the per-matrix reference class (dion/dion_reference.py:131-134)
+            if power_iters <= 0:
+                raise ValueError(f"Invalid power iterations: {power_iters}")
+            if qr_method not in ("qr", "cqr", "rcqr"):
+                raise ValueError(f"Unknown QR method: {qr_method}")
+        else:
+            if power_iters != 1:
+                raise ValueError("Async Dion only supports power_iters=1")
+            if qr_method != "rcqr":
+                raise ValueError("Async Dion only supports qr_method='rcqr'")
         for name, mesh in (("replicate_mesh", replicate_mesh), ("outer_shard_mesh", outer_shard_mesh),
                            ("inner_shard_mesh", inner_shard_mesh)):
             if mesh is not None:
@@ -99,6 +107,9 @@ class Dion(Optimizer):
         )
         super().__init__(params, defaults)
 
+        self._power_iters = power_iters
+        self._qr_method = qr_method
+        self._cqr_warmup_steps = cqr_warmup_steps
         self._replicate_mesh = None
         self._outer_shard_mesh = None
         self._inner_shard_mesh = None
@@ -281,7 +292,7 @@ class Dion(Optimizer):
                     _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
                     len(plist), m, n, r,
                     _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
-                    ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1,
+                    ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
                     info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
                 )
                 _lib.check(rc, "dion_amd_dion_step")
@@ -314,3 +325,19 @@ class Dion(Optimizer):
             weight_decay=torch.tensor(group["weight_decay"]), step=torch.tensor(group["step"]),
             epsilon=torch.tensor(group["epsilon"]),
         )
+
+
+class DionReference(Dion):
+    """Counterpart of the reference's per-matrix class (`dion.DionReference`, dion/dion_reference.py:64-365) on one
+    GPU: the same constructor, which also takes `power_iters` >= 1 and `qr_method` in {"qr", "cqr", "rcqr"}
+    (dion/dion_reference.py:131-134), and the same update (`dion_update`, dion/dion_reference.py:613-687; its
+    `power_iteration`, 690-730, repeats P = orth(B Q), Q = B^T P with the unnormalised Q).
+
+    All three `qr_method` names run the device orthonormaliser: Householder QR, Cholesky QR and randomised
+    Cholesky QR (dion/dion_reference.py:733-789) are three ways to the same thin-QR factor, which they return with
+    different column signs; M and X do not see those signs and Q carries them consistently.  So `cqr_warmup_steps`
+    and the fall-back from a failed Cholesky factorisation to the randomised method (752-758, 296-299) have nothing
+    left to switch between: the factorisation here is in fp64 and its status is in `cholesky_info()`.
+    `state["Q"]` is updated in place rather than replaced by a new tensor."""
+
+    _REFERENCE_OPTIONS = True

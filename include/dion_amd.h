@@ -214,6 +214,8 @@ size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype
  *   X <- decay X - scaled_lr P Q^T.
  * ef_alpha = -(1 - mu), decay = 1 - lr*wd and scaled_lr = sqrt(m/n)*lr are passed as
  * already-evaluated fp32 values.  m_dtype f32 requires x_dtype f32.  info as above.
+ * power_iters >= 1 repeats P = orth(B' Q), Q = B'^T P before the updates, the unnormalised R serving as the
+ * next Q (reference dion/dion_reference.py:690-730; the batched reference class only allows 1).
  * m and n must be multiples of 8 (the host side pads other shapes with zero rows / columns,
  * which changes no result); the rank r is any value in 1 .. min(m, n): the working matrices
  * carry zero columns up to the next multiple of 8 and Q keeps its r contiguous columns. */
@@ -221,6 +223,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
                        int batch, int m, int n, int r,
                        int x_dtype, int g_dtype, int m_dtype, int q_dtype,
                        float ef_alpha, float decay, float scaled_lr, float eps, int faithful,
+                       int power_iters,
                        int* info, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------

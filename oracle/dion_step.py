@@ -6,7 +6,11 @@ Follows reference dion/dion.py `dion_update_ddp` with `replicate_mesh=None` (742
 `R = M_batch.mT @ P` (839), `fix_all_zero_or_nan` (1416-1444), `foreach_baddbmm_` (1494-1530),
 `column_normalize` (1460-1491), `update_Q_matrix_` (1533-1561); state initialisation
 `_init_opt_state_dion` (649-721).  `orthogonalize_variant` adds the per-matrix variants of
-reference dion/dion_reference.py:733-789 ("qr", "cqr", "rcqr").
+reference dion/dion_reference.py:733-789 ("qr", "cqr", "rcqr"), and `dion_update_reference` the per-matrix
+update of the same file (613-687) with its `power_iteration` (690-730): any number of power iterations,
+any of the three methods.  Pinned in tests/test_oracle_math.py: with one iteration it equals `dion_update`,
+with more its M and X equal the closed form B - (1 - mu) Pk Pk^T B, Pk = thin-QR factor of B (B^T B)^(k-1) Q,
+evaluated in fp64.
 
 Everything is eager PyTorch on the CPU, one matrix per batch as on one GPU; dtypes follow
 the tensors exactly as in the reference (bf16 momentum => bf16 P, R, Q_new and products).
@@ -125,3 +129,37 @@ def dion_step(X, G, M, Q, lr, mu, weight_decay, epsilon=1e-8, oversample=1.25, g
     """One step for every matrix of the lists (in place)."""
     for x, g, m, q in zip(X, G, M, Q):
         dion_update(x, g, m, q, lr, mu, weight_decay, epsilon, oversample, generator, orth)
+
+
+def dion_update_reference(X, G, M, Q, lr, mu, weight_decay, epsilon=1e-8, power_iters=1, qr_method="rcqr",
+                          oversample=1.25, generator=None):
+    """reference dion/dion_reference.py:613-687 with power_iteration (690-730), one matrix, no meshes.
+    X and M are modified in place; returns the new Q (the reference class stores it in state["Q"], 319-325)."""
+    lr = torch.tensor(lr) if not isinstance(lr, torch.Tensor) else lr
+    mu = torch.tensor(mu) if not isinstance(mu, torch.Tensor) else mu
+    weight_decay = torch.tensor(weight_decay) if not isinstance(weight_decay, torch.Tensor) else weight_decay
+    transpose = X.size(0) < X.size(1)                         # dion_reference.py:396-420 (is_transposed)
+    Q_init_dtype = Q.dtype
+    Q = Q.to(M.dtype)                                         # 636-637
+    M.add_(G)                                                 # 640
+    B = M.T if transpose else M                               # 645
+    Qi = Q
+    for _ in range(power_iters):                              # 712-728
+        P = B @ Qi
+        P = orthogonalize_variant(P, qr_method, oversample, generator)
+        Qi = B.T @ P
+    R = Qi
+    P, R = fix_all_zero_or_nan(P, R, Q, M)                    # 656
+    if not transpose:                                         # 660-663
+        M.add_(P @ R.T, alpha=-(1 - mu))
+    else:
+        M.add_(R @ P.T, alpha=-(1 - mu))
+    R = R.to(dtype=torch.float32)                             # 668-670
+    Qn = (R / (R.norm(dim=0, keepdim=True) + epsilon)).to(P.dtype)
+    X.mul_(1 - lr * weight_decay)                             # 673
+    scaled_lr = ((X.size(0) / X.size(1)) ** 0.5) * lr         # 676-678
+    if not transpose:                                         # 682-685
+        X.add_(P @ Qn.T, alpha=-scaled_lr)
+    else:
+        X.add_(Qn @ P.T, alpha=-scaled_lr)
+    return Qn.to(Q_init_dtype)                                # 687

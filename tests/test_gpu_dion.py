@@ -243,3 +243,46 @@ def test_dion_groups_and_validation(dev):
     t3.grad = torch.randn_like(t3)
     with pytest.raises(NotImplementedError):
         Dion([t3]).step()
+
+
+@pytest.mark.parametrize("qr_method,power_iters", [("cqr", 1), ("qr", 2), ("rcqr", 3)])
+def test_dion_reference_class(dev, qr_method, power_iters):
+    """`DionReference` (reference dion/dion_reference.py:64-365): every `qr_method` name and several power
+    iterations against the oracle's per-matrix update, all-fp32 state, 1e-4 on M, X and sign-aligned Q."""
+    from dion_amd import DionMixedPrecisionConfig, DionReference
+    from oracle import dion_step as O
+
+    shapes = [(512, 256), (256, 512), (200, 120)]
+    rank_fraction = 0.25
+    g = torch.Generator().manual_seed(31)
+    X0 = [torch.randn(s, generator=g) * 0.02 for s in shapes]
+    Q0 = []
+    for (m, n) in shapes:
+        q = torch.randn((m if m < n else n, O.rank_of(m, n, rank_fraction)), generator=g)
+        Q0.append(q / q.norm(dim=0, keepdim=True))
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    cfg = DionMixedPrecisionConfig(momentum_dtype=torch.float32, Q_dtype=torch.float32)
+    opt = DionReference(params, rank_fraction=rank_fraction, lr=0.01, mu=0.95, weight_decay=0.01, qr_method=qr_method,
+                        power_iters=power_iters, cqr_warmup_steps=1, mixed_precision_config=cfg)
+    Xo, Mo, Qo = [x.clone() for x in X0], [torch.zeros_like(x) for x in X0], [q.clone() for q in Q0]
+    sk = torch.Generator().manual_seed(0)
+    for step in range(4):
+        G = [torch.randn(s, generator=g) * 1e-3 for s in shapes]
+        for p, gr in zip(params, G):
+            p.grad = gr.to(dev)
+        if step == 0:
+            for p, q in zip(params, Q0):
+                opt._get_or_initialize_state(p, opt.param_groups[0])["Q"].copy_(q.to(dev))
+        for i in range(len(shapes)):
+            Qo[i] = O.dion_update_reference(Xo[i], G[i], Mo[i], Qo[i], 0.01, 0.95, 0.01, 1e-8, power_iters=power_iters,
+                                            qr_method=qr_method, generator=sk)
+        opt.step()
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            eM, eX = rel_fro(st["momentum"], Mo[i]), rel_fro(p.detach(), Xo[i])
+            eQ = rel_fro(_sign_align(st["Q"].cpu(), Qo[i]), Qo[i])
+            assert eM <= FP32_TOL and eX <= FP32_TOL and eQ <= FP32_TOL, (step, i, eM, eX, eQ)
+    with pytest.raises(ValueError):
+        DionReference(params, power_iters=0)
+    with pytest.raises(ValueError):
+        DionReference(params, qr_method="svd")

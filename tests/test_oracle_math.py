@@ -155,6 +155,50 @@ def test_dion_full_rank_and_zero_cases():
     assert O.rank_of(768, 3072, 0.25) == 192 and O.rank_of(100, 60, 0.3, 8) == 24 and O.rank_of(10, 10, 1.0, 16) == 10
 
 
+@pytest.mark.parametrize("shape", [(96, 64), (64, 96)])
+@pytest.mark.parametrize("qr_method", ["qr", "cqr", "rcqr"])
+def test_dion_reference_update_power_iterations(shape, qr_method):
+    """`dion_update_reference`: one iteration equals `dion_update`; k iterations give the projector onto
+    col(B (B^T B)^(k-1) Q) in the error feedback and the update -- the closed form, evaluated here with
+    a Householder QR in fp64 (a dropped or repeated iteration, or a missing transpose, changes the subspace)."""
+    from oracle import dion_step as O
+
+    torch.manual_seed(8)
+    r = 12
+    X0 = torch.randn(shape, dtype=torch.float64) * 0.02
+    G = torch.randn(shape, dtype=torch.float64) * 1e-3
+    M0 = torch.randn(shape, dtype=torch.float64) * 1e-3
+    Q0 = torch.randn(min(shape), r, dtype=torch.float64)
+    lr, mu, wd, eps = 0.01, 0.95, 0.1, 1e-8
+    Xa, Ma, Qa = X0.clone(), M0.clone(), Q0.clone()
+    O.dion_update(Xa, G, Ma, Qa, lr, mu, wd, eps)
+    Xb, Mb = X0.clone(), M0.clone()
+    Qb = O.dion_update_reference(Xb, G, Mb, Q0.clone(), lr, mu, wd, eps, power_iters=1, qr_method=qr_method,
+                                 generator=torch.Generator().manual_seed(1))
+    sgn = torch.sign((Qa * Qb).sum(dim=0))
+    assert rel_fro(Mb, Ma) < 1e-6 and rel_fro(Xb, Xa) < 1e-6 and rel_fro(Qb * sgn, Qa) < 1e-5
+    B = M0 + G
+    Bv = B.T if shape[0] < shape[1] else B
+    for k in (2, 3):
+        X, M = X0.clone(), M0.clone()
+        Qn = O.dion_update_reference(X, G, M, Q0.clone(), lr, mu, wd, eps, power_iters=k, qr_method=qr_method,
+                                     generator=torch.Generator().manual_seed(1))
+        K = Bv @ Q0
+        for _ in range(k - 1):
+            K = Bv @ (Bv.T @ torch.linalg.qr(K)[0])   # re-orthonormalised: the powers of B^T B are ill-conditioned
+        Pk = torch.linalg.qr(K)[0]
+        low = Pk @ (Pk.T @ Bv)
+        low = low.T if shape[0] < shape[1] else low
+        assert rel_fro(M, B - (1 - mu) * low) < 1e-6, (k, qr_method)
+        Rk = Bv.T @ Pk
+        Qk = Rk / (Rk.norm(dim=0, keepdim=True) + eps)
+        upd = Pk @ Qk.T
+        upd = upd.T if shape[0] < shape[1] else upd
+        assert rel_fro(X, (1 - lr * wd) * X0 - (shape[0] / shape[1]) ** 0.5 * lr * upd) < 1e-6, (k, qr_method)
+        s2 = torch.sign((Qn * Qk).sum(dim=0))
+        assert rel_fro(Qn * s2, Qk) < 1e-5
+
+
 def test_orthogonalize_variants_agree():
     from oracle import dion_step as O
 
