@@ -253,6 +253,21 @@ def cpu_baseline(wl, budget_s=20.0):
                 sample=f"{reps} full steps of the same {len(shapes)}-matrix workload after 1 warm-up ({what})")
 
 
+def device_info(dev):
+    """What the rooflines are priced against, as the runtime reports it for the GPU the numbers come from."""
+    import torch
+
+    p = torch.cuda.get_device_properties(dev)
+    info = dict(name=p.name, compute_units=p.multi_processor_count, hbm_gib=round(p.total_memory / 2**30, 1))
+    clock_khz = getattr(p, "clock_rate", None)
+    if clock_khz:
+        info["max_shader_clock_mhz"] = round(clock_khz / 1e3)
+        # dense bf16 MFMA: 4096 flops per clock per CU (a 32x32x16 MFMA, 32768 flops, per SIMD every 32 clocks)
+        info["bf16_dense_peak_at_that_clock_tflops"] = round(p.multi_processor_count * 4096 * clock_khz * 1e3 / 1e12, 1)
+    info["arch"] = getattr(p, "gcnArchName", "")
+    return info
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -304,6 +319,7 @@ def main():
         "event_ms_per_step": round(res["event_ms"], 4),
         "wall_ms_per_step": round(res["wall_ms"], 4),
         "roofline": roofline_of(res, wl["kind"], args.workload),
+        "device": device_info(dev),
     }
     out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
     if not args.no_extra:
