@@ -175,6 +175,21 @@ def test_dion_bf16_off_the_alignment_grid(dev):
               check=check)
 
 
+def test_dion_bucket_larger_than_one_chunk(dev):
+    """70 same-shape matrices: more than the 64 a launch's pointer tables hold, so the bucket goes through the
+    library in two chunks (status words and pointer tables at an offset)."""
+    def check(step, params, opt, Xo, Mo, Qo):
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            eM, eX = rel_fro(st["momentum"], Mo[i]), rel_fro(p.detach(), Xo[i])
+            eQ = rel_fro(_sign_align(st["Q"].cpu(), Qo[i]), Qo[i])
+            assert eM <= FP32_TOL and eX <= FP32_TOL and eQ <= FP32_TOL, (step, i, eM, eX, eQ)
+        info = torch.cat([v for v in opt.cholesky_info().values()])
+        assert info.numel() == 70 and int(info.abs().sum().item()) == 0
+
+    _run_dion(dev, [(64, 48)] * 70, 0.5, 2, torch.float32, torch.float32, torch.float32, check=check)
+
+
 def test_dion_fp32_full_rank(dev):
     """rank_fraction 1.0: square matrices are conditioning-limited (cond(BQ) ~ 1e5-1e6): the reference's own
     fp32-vs-fp64 spread in Q is ~7e-4 there, while M and X stay tight.  At full rank M_new = mu * B exactly."""
