@@ -272,9 +272,11 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
   const int below = (rest + NB - 1) / NB;
   const int smem = 2 * NB * LP * (int)sizeof(T);
-  // workgroups per matrix: enough for ~384 in flight over the batch, never more than there are roles
+  // workgroups per matrix: as many as fit one per CU over the batch (the factorisation every workgroup repeats is
+  // bound by fp64 instruction issue, which two workgroups on a CU would share: 384 instead of 256 in flight cost
+  // 3 % of the orthonormaliser on a 48-matrix bucket), never more than there are roles
   const int nroles = 1 + below + o / NB;
-  int per = 384 / batch;
+  int per = 256 / batch;
   if (per < 1) per = 1;
   if (per > nroles) per = nroles;
   static bool configured = false;  // benign race: the attribute call is idempotent
