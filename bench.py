@@ -15,6 +15,8 @@ Workloads (numbered as the benchmark's configurations):
   dion_gpt_small_r1     rank fraction 1.0; bf16 weights / momentum, fp32 Q, G seed 3.
   muon_llama8b_layer    (configs[3], one of the 32 layers) Muon on 7 bf16 matrices incl. 4096x14336.
   dion_llama70b_layer   (configs[4], one of the 8 layers) Dion r=512 on 2 x 28672x8192 + 8192x28672.
+  muon_llama8b          (configs[3], all 32 layers) 224 bf16 matrices, 6.98e9 elements, drawn on the GPU.
+  dion_llama70b_mlp     (configs[4], all 8 layers) 24 bf16 matrices, 5.64e9 elements, drawn on the GPU.
   scalar_gpt_small      the non-matrix groups of GPT-small: Lion / AdamW on embedding, lm_head, norms.
 """
 import argparse
@@ -44,20 +46,26 @@ WORKLOADS = {
                                desc="Muon step, one Llama-3-8B layer: 7 bf16 matrices incl. 4096x14336"),
     "dion_llama70b_layer": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER, seed=5, rank_fraction=1.0 / 16,
                                 desc="Dion step, one Llama-3-70B MLP layer (28672x8192 x2, 8192x28672), r=512"),
+    "muon_llama8b": dict(kind="muon", shapes=LLAMA8B_LAYER * 32, seed=4, on_device=True,
+                         desc="Full Muon step, Llama-3-8B-shaped stack: 32 layers x 7 bf16 matrices (6.98e9 elements)"),
+    "dion_llama70b_mlp": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER * 8, seed=5, rank_fraction=1.0 / 16, on_device=True,
+                              desc="Full Dion step, Llama-3-70B-shaped MLP matrices: 8 layers x 3 (5.64e9 elements), r=512"),
     "scalar_gpt_small": dict(kind="scalar", shapes=[(50304, 768)] * 2 + [(768,)] * 25, seed=6,
                              desc="Lion on the GPT-small embedding and norms, AdamW on lm_head (50304x768 each), bf16"),
 }
 GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd")
 
 
-def make_problem(shapes, seed, dtype):
+def make_problem(shapes, seed, dtype, device="cpu"):
+    """Weights N(0, 0.02^2) and gradients N(0, 1e-6) from a seeded generator; the multi-gigabyte workloads draw
+    them on the GPU (the values differ from the CPU generator's, the distribution does not)."""
     import torch
 
-    gen = torch.Generator(device="cpu").manual_seed(seed)
+    gen = torch.Generator(device=device).manual_seed(seed)
     params, grads = [], []
     for s in shapes:
-        params.append((torch.randn(s, generator=gen) * 0.02).to(dtype))
-        grads.append((torch.randn(s, generator=gen) * 1e-3).to(dtype))
+        params.append((torch.randn(s, generator=gen, device=device) * 0.02).to(dtype))
+        grads.append((torch.randn(s, generator=gen, device=device) * 1e-3).to(dtype))
     return params, grads
 
 
@@ -73,7 +81,7 @@ def build_optimizer(wl, dev):
     import torch
     from dion_amd import Dion, DionMixedPrecisionConfig, Muon
 
-    X, G = make_problem(wl["shapes"], wl["seed"], torch.bfloat16)
+    X, G = make_problem(wl["shapes"], wl["seed"], torch.bfloat16, dev if wl.get("on_device") else "cpu")
     params = [torch.nn.Parameter(x.to(dev)) for x in X]
     for p, g in zip(params, G):
         p.grad = g.to(dev)
@@ -325,7 +333,7 @@ def main():
     if not args.no_extra:
         extra = {}
         for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "dion_llama70b_layer",
-                     "scalar_gpt_small"):
+                     "muon_llama8b", "dion_llama70b_mlp", "scalar_gpt_small"):
             if name == args.workload:
                 continue
             w = WORKLOADS[name]
