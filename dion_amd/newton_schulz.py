@@ -6,8 +6,6 @@ Mirrors the reference operator interface:
   * `zeropower_via_newtonschulz5_keller(G, steps=5, eps=1e-7)` -- reference dion/muon_reference.py:10-27
   * `ns_line_1(A)`, `ns_line_2(A, alpha, beta)`               -- reference dion/newton_schulz_triton.py:134-170, 261-302
 """
-import ctypes
-
 import torch
 from torch import Tensor
 
