@@ -187,7 +187,12 @@ def summarize(name, wl, res):
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.000 and
 # WRITE_SIZE x 1.000, in KiB, the factors being what the same counters read for a plain 512 MiB copy);
 # the runs used the default workload with three 512 MiB copies first (--calibrate-copy).  Keyed by (workload, kernel).
-MEASURED_TRAFFIC_BYTES = {("muon_gpt_small", "ns_axpy"): 683634 * 1024}
+MEASURED_TRAFFIC_BYTES = {
+    ("muon_gpt_small", "ns_axpy"): 683634 * 1024,
+    # error feedback / weight update of the Llama-3-70B layer: mean over the 2-matrix and the 1-matrix bucket
+    ("dion_llama70b_layer", "dion_ef"): 1896506 * 1024,
+    ("dion_llama70b_layer", "dion_upd"): 1896506 * 1024,
+}
 
 
 def roofline_of(res, kind, workload=None):
