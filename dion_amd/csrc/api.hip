@@ -177,6 +177,27 @@ int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype,
 
 bool dtype_ok(int d) { return d == DA_BF16 || d == DA_F32; }
 
+// Number of slices (1, 2 or 4) of the inner dimension `mp` for the product R = B^T P (np x r per matrix, `cb`
+// matrices), by the bf16 launcher's own estimate: workgroup rounds x 64-deep stages per tile, a 256 x 256 tile
+// costing 4 per stage on a whole CU and a 128 x 128 tile 3 on half a CU; a sliced product also pays for writing
+// and adding its fp32 partial sums.
+int btp_slices(int np, int r, int mp, int cb) {
+  int best = 1;
+  double best_cost = 0.0;
+  for (int s = 1; s <= DA_MAX_GROUPS; s *= 2) {
+    if (s > 1 && (mp / s < 512 || mp % (s * 64) != 0)) break;
+    const long long t256 = (long long)((np + 255) / 256) * ((r + 255) / 256) * cb * s;
+    const long long t128 = (long long)((np + 127) / 128) * ((r + 127) / 128) * cb * s;
+    const double stages = (double)(mp / s) / 64.0;
+    const double big = np >= 256 && r >= 256 ? (double)((t256 + 255) / 256) * stages * 4.0 : 1e30;
+    const double small = (double)((t128 + 511) / 512) * stages * 3.0;
+    double cost = big < small ? big : small;
+    if (s > 1) cost += 32.0 + 8.0 * s;
+    if (s == 1 || cost < best_cost) { best = s; best_cost = cost; }
+  }
+  return best;
+}
+
 }  // namespace
 
 extern "C" {
@@ -602,12 +623,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
       // A few output tiles with a long inner dimension (tall matrices at a low rank) leave most of the GPU idle:
       // cut the inner dimension into slices that run side by side as the groups of one launch and leave fp32
       // partial sums, which the fix-up pass that follows adds and rounds.
-      int slices = 1;
-      if (m_dtype == DA_BF16) {
-        const long long tiles = (long long)((np + 127) / 128) * ((r + 127) / 128) * cb;
-        while (slices < DA_MAX_GROUPS && tiles * slices < 384 && mp / (slices * 2) >= 512 && mp % (slices * 2 * 64) == 0)
-          slices *= 2;
-      }
+      const int slices = m_dtype == DA_BF16 ? btp_slices(np, r, mp, cb) : 1;
       if (slices > 1) {
         GemmDesc gs[DA_MAX_GROUPS];
         const int kslice = mp / slices;
