@@ -387,8 +387,8 @@ __global__ void pad_diag_kernel(double* G, long long rr, int r, int r_live) {
 }
 
 // One blocked CholeskyQR pass in fp64, in place:  P <- P R^-1  with  P^T P = R^T R.
-int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int r_live, int* info,
-                hipStream_t s) {
+int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int r_live, bool g_cleared,
+                int* info, hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
@@ -401,6 +401,7 @@ int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows
   g.M = r; g.N = r; g.K = rows;
   g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
   g.split_k = -1;   // few output tiles, long K: the launcher slices K until the GPU is full
+  g.c_is_zero = g_cleared ? 1 : 0;
   int rc = da_gemm_f64(g, s);
   if (rc) return rc;
   if (r_live < r) {
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256) void polish_correction_kernel(const float* __r
 // The Gram product is fp32 as in polish_pass; the correction product runs on the bf16 matrix cores (its
 // relative error 2^-8 times the defect E of `in` adds 4e-3 E to the result, next to the pass's own O(E^2)).
 int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_dtype, float* G, bf16_t* U, int batch,
-                     int rows, int r, hipStream_t s) {
+                     int rows, int r, bool g_cleared, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   Gemm32Desc g{};
   g.batch = batch;
@@ -487,6 +488,7 @@ int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_d
   g.M = r; g.N = r; g.K = rows;
   g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
   g.split_k = -1;
+  g.c_is_zero = g_cleared ? 1 : 0;
   int rc = da_gemm_f32s(g, s);
   if (rc) return rc;
   hipLaunchKernelGGL(polish_correction_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, U, rr, r);
@@ -509,7 +511,7 @@ int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_d
 // the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one product with
 // the triangular V -- no serial chain.
 int polish_pass(const float* in, void* out, int out_store, float* G, float* V, int batch, int rows, int r,
-                hipStream_t s) {
+                bool g_cleared, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   Gemm32Desc g{};
   g.batch = batch;
@@ -519,6 +521,7 @@ int polish_pass(const float* in, void* out, int out_store, float* G, float* V, i
   g.M = r; g.N = r; g.K = rows;
   g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
   g.split_k = -1;
+  g.c_is_zero = g_cleared ? 1 : 0;
   int rc = da_gemm_f32s(g, s);
   if (rc) return rc;
   hipLaunchKernelGGL(polish_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, V, rr, r);
@@ -553,19 +556,24 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   double* W = L + rr * batch;
   float* P0f = reinterpret_cast<float*>(W + rr * batch);
   bf16_t* P0h = reinterpret_cast<bf16_t*>(P0f + pr * batch);
-  int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, s);
+  // the Gram products are split over K when they have few tiles: their output is cleared by the conversion
+  // launch that precedes them rather than by one of its own
+  const bool split = da_auto_split(da_gram_blocks(r, batch), rows) > 1;
+  int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, split ? G : nullptr, rr * batch, s);
   if (rc) return rc;
-  rc = cholqr_pass(P0, G, L, W, batch, rows, r, r_live, info, s);
+  rc = cholqr_pass(P0, G, L, W, batch, rows, r, r_live, split, info, s);
   if (rc) return rc;
   if (passes == 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
   // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products
   // (the bf16 product moves 16-byte chunks: r a multiple of 8, else the all-fp32 form below)
   const bool low = passes == 2 && (r & 7) == 0;
-  rc = da_cvt_f64_to_f32(P0, P0f, low ? P0h : nullptr, pr * batch, s);
+  // the fp32 Gram matrix of the first polishing pass goes where G was: cleared here for its split-K product
+  rc = da_cvt_f64_to_f32(P0, P0f, low ? P0h : nullptr, pr * batch, split ? reinterpret_cast<float*>(G) : nullptr,
+                         rr * batch, s);
   if (rc) return rc;
   if (low)
     return polish_pass_bf16(P0f, P0h, out, dtype, reinterpret_cast<float*>(G), reinterpret_cast<bf16_t*>(L), batch,
-                            rows, r, s);
+                            rows, r, split, s);
   const float* cur = P0f;
   float* Gf = reinterpret_cast<float*>(G);
   float* Vf = reinterpret_cast<float*>(L);
@@ -574,7 +582,7 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
     float* other = cur == P0f ? reinterpret_cast<float*>(P0) : P0f;
     rc = polish_pass(cur, last ? out : static_cast<void*>(other), last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf, Vf,
-                     batch, rows, r, s);
+                     batch, rows, r, split && pass == 1, s);
     if (rc) return rc;
     cur = other;
   }

@@ -24,23 +24,37 @@ struct RealGemmDesc {
   // excludes E, split_k and the symmetric form.
   int c_store;
   int k_tri;     // 1: B is block lower triangular -- output column tile j only sums k < 64 (j + 1)
+  int c_is_zero; // 1: the caller has cleared C (batch * sC elements): an auto-split product need not do it
 };
 #define DA_STORE_NATIVE 0
 #define DA_STORE_BF16 1
 #define DA_STORE_F32 2
 inline int da_store_of(int dtype) { return dtype == DA_BF16 ? DA_STORE_BF16 : DA_STORE_F32; }
+// Slices of K an auto-split product (split_k < 0) of `blocks` output tiles uses: few tiles with a long K are
+// sliced until ~512 workgroups exist.  > 1 means the product adds into a cleared C.
+inline int da_auto_split(long long blocks, int K) {
+  const int max_split = K / 256 > 0 ? K / 256 : 1;
+  const long long sp = (512 + blocks - 1) / blocks;
+  return (int)(sp > max_split ? max_split : sp);
+}
+// Output tiles of the symmetric (Gram) form for `batch` r x r matrices.
+inline long long da_gram_blocks(int r, int batch) {
+  const long long t = (r + 63) / 64;
+  return t * (t + 1) / 2 * batch;
+}
 typedef RealGemmDesc<double> Gemm64Desc;
 typedef RealGemmDesc<float> Gemm32Desc;
 
 // The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the products of the polishing passes, whose input is
 // already orthonormal to 1e-4 or better, do not need fp64.
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s);
-// dst (f32) <- src (f64); `low`, if not null, receives the same values in bf16
-int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, hipStream_t s);
+// dst (f32) <- src (f64); `low`, if not null, receives the same values in bf16; `zero`, if not null, nz floats
+// cleared in the same launch
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, float* zero, long long nz, hipStream_t s);
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
 
 // dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.
-int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s);
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, double* zero, long long nz, hipStream_t s);
 int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s);
 
 // Block-column step j = o / 64 of the blocked lower Cholesky G = L L^T of each r x r matrix

@@ -268,11 +268,8 @@ int launch(const RealGemmDesc<T>& d, hipStream_t s) {
   const bool auto_split = d.split_k < 0 && !d.E && d.c_store == DA_STORE_NATIVE;
   int split = d.split_k > 1 && !d.E ? d.split_k : 1;
   if (auto_split) {
-    // few output tiles, long K: slice K until ~512 workgroups exist
-    const int max_split = d.K / 256 > 0 ? d.K / 256 : 1;
-    const long long sp = (512 + blocks - 1) / blocks;
-    split = (int)(sp > max_split ? max_split : sp);
-    if (split > 1) {
+    split = da_auto_split(blocks, d.K);
+    if (split > 1 && !d.c_is_zero) {
       // the slices add into C: clear it (the batches of C are contiguous here)
       const long long n = (long long)d.sC * (d.batch - 1) + (long long)(d.M - 1) * d.ldc + d.N;
       hipLaunchKernelGGL(fill_f64_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d.C, n, T(0));
@@ -283,11 +280,14 @@ int launch(const RealGemmDesc<T>& d, hipStream_t s) {
   return launch_bt<T, A_KS, B_KS, SYM, BTt>(d, split, s);
 }
 
+// (`zero`, if not null: nz elements cleared in the same launch -- the output of the split-K product that follows)
 template <typename T, typename R>
 __global__ __launch_bounds__(256) void cvt_to_f64_kernel(const T* __restrict__ src, R* __restrict__ dst,
-                                                         long long n) {
+                                                         long long n, R* __restrict__ zero, long long nz) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
     dst[i] = (R)ld_as_float<T>(src + i);
+  if (zero)
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nz; i += (long long)gridDim.x * 256) zero[i] = R(0);
 }
 
 template <typename T, typename R>
@@ -299,12 +299,15 @@ __global__ __launch_bounds__(256) void cvt_from_f64_kernel(const R* __restrict__
 
 // fp64 -> fp32, and (if `low` is given) the same values rounded once more to bf16
 __global__ __launch_bounds__(256) void cvt_f64_to_f32_kernel(const double* __restrict__ src, float* __restrict__ dst,
-                                                              bf16_t* __restrict__ low, long long n) {
+                                                              bf16_t* __restrict__ low, long long n,
+                                                              float* __restrict__ zero, long long nz) {
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
     const float v = (float)src[i];
     dst[i] = v;
     if (low) low[i] = f2bf(v);
   }
+  if (zero)
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nz; i += (long long)gridDim.x * 256) zero[i] = 0.f;
 }
 
 inline unsigned cvt_blocks(long long n) {
@@ -330,12 +333,12 @@ int gemm_real(const RealGemmDesc<T>& d, hipStream_t s) {
 }
 
 template <typename R>
-int cvt_to(const void* src, int src_dtype, R* dst, long long n, hipStream_t s) {
+int cvt_to(const void* src, int src_dtype, R* dst, long long n, R* zero, long long nz, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
   if (src_dtype == DA_BF16)
-    hipLaunchKernelGGL((cvt_to_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n);
+    hipLaunchKernelGGL((cvt_to_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n, zero, nz);
   else if (src_dtype == DA_F32)
-    hipLaunchKernelGGL((cvt_to_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n);
+    hipLaunchKernelGGL((cvt_to_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n, zero, nz);
   else
     return DA_ERR_DTYPE;
   return da_launch_status();
@@ -358,10 +361,12 @@ int cvt_from(const R* src, void* dst, int dst_dtype, long long n, hipStream_t s)
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) { return gemm_real<double>(d, s); }
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s) { return gemm_real<float>(d, s); }
 
-int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, hipStream_t s) { return cvt_to<double>(src, src_dtype, dst, n, s); }
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, double* zero, long long nz, hipStream_t s) {
+  return cvt_to<double>(src, src_dtype, dst, n, zero, nz, s);
+}
 int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<double>(src, dst, dst_dtype, n, s); }
-int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, hipStream_t s) {
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, float* zero, long long nz, hipStream_t s) {
   if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, low, n);
+  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, low, n, zero, nz);
   return da_launch_status();
 }
