@@ -89,17 +89,18 @@ def test_muon_step_vs_reference_vectors(dev, gold):
 
 
 def test_ns_properties_at_llama8b_shape(dev):
-    """4096 x 14336 (and its tall twin): transpose equivariance and near-orthonormal rows, checked with
-    plain fp32 torch matmuls on the GPU."""
+    """4096 x 14336 (and its tall twin): transpose equivariance and near-orthonormal rows (Gram matrix of the
+    first 1024 rows, a plain fp32 matmul on the CPU)."""
     from dion_amd import zeropower_via_newtonschulz5
 
     g = torch.Generator(device=dev).manual_seed(4)
     G = (torch.randn(4096, 14336, device=dev, generator=g) * 1e-3).bfloat16()
     X = zeropower_via_newtonschulz5(G)
     assert torch.equal(zeropower_via_newtonschulz5(G.mT.contiguous()), X.mT)
-    gram = X.float() @ X.float().T
-    dev_from_i = (gram - torch.eye(4096, device=dev)).norm().item() / 64.0   # / sqrt(4096)
-    print(f"||X X^T - I||_F / sqrt(m) = {dev_from_i:.3f}")
+    Xs = X[:1024].float().cpu()
+    gram = Xs @ Xs.T
+    dev_from_i = (gram - torch.eye(1024)).norm().item() / 32.0   # / sqrt(rows)
+    print(f"||X X^T - I||_F / sqrt(rows) = {dev_from_i:.3f}")
     assert dev_from_i < 0.1
     assert torch.isfinite(X.float()).all()
 
@@ -128,5 +129,5 @@ def test_dion_properties_at_llama70b_shape(dev):
     assert (p.detach().float() - x0.float()).abs().max().item() > 0
     assert int(torch.cat(list(opt.cholesky_info().values())).abs().sum().item()) == 0
     P = torch.randn(28672, 512, device=dev, generator=g)
-    Qf = orthonormalize(P)
-    assert ((Qf.T @ Qf) - torch.eye(512, device=dev)).norm().item() <= 1e-3
+    Qf = orthonormalize(P).cpu()
+    assert ((Qf.T @ Qf) - torch.eye(512)).norm().item() <= 1e-3
