@@ -153,3 +153,42 @@ def test_reference_import_paths_exist():
     assert list(inspect.signature(nst.newton_schulz_triton).parameters) == ["G", "epsilon"]
     assert list(inspect.signature(muon_reference.zeropower_via_newtonschulz5).parameters) == ["G", "steps", "eps"]
     assert callable(nst.ns_line_1) and callable(nst.ns_line_2)
+
+
+def test_dion_reference_constructor_contract():
+    """The per-matrix reference class's extra options (reference dion/dion_reference.py:131-134)."""
+    from dion_amd import Dion, DionReference
+
+    p = [torch.nn.Parameter(torch.randn(8, 8))]
+    for method in ("qr", "cqr", "rcqr"):
+        opt = DionReference(p, qr_method=method, power_iters=3, cqr_warmup_steps=7)
+        assert isinstance(opt, Dion) and opt._power_iters == 3 and opt._qr_method == method
+        assert opt._cqr_warmup_steps == 7 and opt.defaults == Dion(p).defaults
+    with pytest.raises(ValueError, match="Invalid power iterations"):
+        DionReference(p, power_iters=0)
+    with pytest.raises(ValueError, match="Unknown QR method"):
+        DionReference(p, qr_method="svd")
+    with pytest.raises(NotImplementedError):
+        DionReference(p, replicate_mesh=object())
+
+
+def test_zero_padding_helpers():
+    """Shapes off the 8-element grid are stepped on zero-padded copies: the padded dimensions keep which side is
+    the longer one (it decides the transposes), and the copies round-trip."""
+    from dion_amd import _lib
+
+    assert _lib.padded_dims(768, 3072) == (768, 3072)
+    assert _lib.padded_dims(100, 60) == (104, 64)
+    assert _lib.padded_dims(60, 100) == (64, 104)
+    assert _lib.padded_dims(77, 77) == (80, 80)
+    assert _lib.padded_dims(100, 101) == (104, 112)      # m < n must stay m < n
+    assert _lib.padded_dims(101, 100) == (112, 104)      # m > n must stay m > n
+    assert _lib.padded_dims(1, 7) == (8, 16)
+    mats = [torch.arange(6.0).reshape(2, 3), -torch.arange(6.0).reshape(2, 3)]
+    big = _lib.zero_padded(mats, 8, 8)
+    assert big.shape == (2, 8, 8) and torch.equal(big[1, :2, :3], mats[1]) and big[:, 2:].abs().sum() == 0
+    assert big[:, :, 3:].abs().sum() == 0
+    big[0, :2, :3] += 1
+    out = [torch.zeros(2, 3), torch.zeros(2, 3)]
+    _lib.crop_back(out, big)
+    assert torch.equal(out[0], mats[0] + 1) and torch.equal(out[1], mats[1])
