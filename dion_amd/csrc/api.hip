@@ -216,7 +216,9 @@ int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int l
   if (!dtype_ok(g_dtype) || !dtype_ok(compute_dtype)) return DA_ERR_DTYPE;
   if ((m | n | ldg | ldo) & 7) return DA_ERR_ALIGN;
   if ((g_stride | out_stride) & 7) return DA_ERR_ALIGN;
-  if (((uintptr_t)G | (uintptr_t)out | (uintptr_t)workspace) & 255) return DA_ERR_ALIGN;
+  // matrices move as 16-byte chunks; only the workspace, which the library carves up itself, needs 256
+  if (((uintptr_t)G | (uintptr_t)out) & 15) return DA_ERR_ALIGN;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const NsLayout L(m, n, compute_dtype);
   const int chunk = L.chunk(batch, workspace_bytes);
@@ -356,6 +358,73 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
     if (rc) return rc;
   }
   return DA_OK;
+}
+
+int dion_amd_muon_pre(const void* const* G, void* const* M, void* const* U, int batch, int m, int n, int g_dtype,
+                      int m_dtype, float mu, int nesterov, void* stream) {
+  if (!G || !M || !U || batch <= 0 || m <= 0 || n <= 0) return DA_ERR_ARG;
+  if (!dtype_ok(g_dtype) || !dtype_ok(m_dtype)) return DA_ERR_DTYPE;
+  if (n & 7) return DA_ERR_ALIGN;
+  for (int i = 0; i < batch; ++i) {
+    if (!G[i] || !M[i] || !U[i]) return DA_ERR_ARG;
+    if (((uintptr_t)G[i] | (uintptr_t)M[i] | (uintptr_t)U[i]) & 15) return DA_ERR_ALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const double gsz = g_dtype == DA_BF16 ? 2 : 4, msz = m_dtype == DA_BF16 ? 2 : 4;
+  for (int b0 = 0; b0 < batch; b0 += DA_MAX_PTRS) {
+    const int cb = batch - b0 < DA_MAX_PTRS ? batch - b0 : DA_MAX_PTRS;
+    DaStage st{};
+    for (int i = 0; i < cb; ++i) {
+      st.g.p[i] = const_cast<void*>(G[b0 + i]);
+      st.mom.p[i] = M[b0 + i];
+      st.wtab.p[i] = U[b0 + i];
+    }
+    st.use_wtab = 1; st.wide = nullptr; st.partials = nullptr;
+    st.batch = cb; st.rows = m; st.cols = n; st.ld = n; st.ldw = n;
+    st.g_dtype = g_dtype; st.m_dtype = m_dtype; st.w_dtype = DA_BF16;
+    st.mu = mu; st.nesterov = nesterov; st.muon = 1;
+    DaProfScope prof(DA_PROF_STAGE, (double)m * n * (gsz + 2 * msz + 2) * cb, s);
+    const int rc = da_stage_wide(st, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+int dion_amd_muon_post(void* const* X, const void* const* O, int batch, int m, int n, int x_dtype, float decay,
+                       float adjusted_lr, void* stream) {
+  if (!X || !O || batch <= 0 || m <= 0 || n <= 0) return DA_ERR_ARG;
+  if (!dtype_ok(x_dtype)) return DA_ERR_DTYPE;
+  if (n & 7) return DA_ERR_ALIGN;
+  for (int i = 0; i < batch; ++i) {
+    if (!X[i] || !O[i]) return DA_ERR_ARG;
+    if (((uintptr_t)X[i] | (uintptr_t)O[i]) & 15) return DA_ERR_ALIGN;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const double xsz = x_dtype == DA_BF16 ? 2 : 4;
+  for (int b0 = 0; b0 < batch; b0 += DA_MAX_PTRS) {
+    const int cb = batch - b0 < DA_MAX_PTRS ? batch - b0 : DA_MAX_PTRS;
+    DaUnstage us{};
+    for (int i = 0; i < cb; ++i) {
+      us.x.p[i] = X[b0 + i];
+      us.wtab.p[i] = const_cast<void*>(O[b0 + i]);
+    }
+    us.use_wtab = 1; us.wide = nullptr;
+    us.batch = cb; us.rows = m; us.cols = n; us.ld = n; us.ldw = n;
+    us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
+    us.decay = decay; us.step = adjusted_lr; us.muon = 1;
+    DaProfScope prof(DA_PROF_UNSTAGE, (double)m * n * (2 * xsz + 2) * cb, s);
+    const int rc = da_unstage(us, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
+}
+
+int dion_amd_gemm_plan(int M, int N, int K, int lda, int a_kstrided, int ldb, int b_kstrided) {
+  if (M <= 0 || N <= 0 || K <= 0 || lda <= 0 || ldb <= 0) return DA_ERR_ARG;
+  GemmDesc g{};
+  g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.batch = 1;
+  g.a_kstrided = a_kstrided != 0; g.b_kstrided = b_kstrided != 0;
+  return da_gemm_bf16_plan(g);
 }
 
 size_t dion_amd_muon_buckets_workspace_bytes(const dion_amd_muon_bucket* buckets, int nbuckets) {
@@ -534,7 +603,6 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
   if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || rank <= 0) return DA_ERR_ARG;
   if (power_iters < 1 || power_iters > 64) return DA_ERR_ARG;
   if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype) || !dtype_ok(m_dtype) || !dtype_ok(q_dtype)) return DA_ERR_DTYPE;
-  if (m_dtype == DA_F32 && x_dtype != DA_F32) return DA_ERR_DTYPE;  // fp32 products update fp32 weights only
   if ((m | n) & 7) return DA_ERR_ALIGN;
   if (rank > m || rank > n) return DA_ERR_ARG;
   if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;

@@ -102,3 +102,5 @@ int da_gemm_bf16(const GemmDesc& d, hipStream_t stream);
 constexpr int DA_MAX_GROUPS = 4;
 int da_gemm_bf16_grouped(const GemmDesc* d, int n, hipStream_t stream);
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream);
+// Tile edge (128 / 256) the bf16 launcher picks for one product, + 1 if its K loop is the direct-to-LDS one.
+int da_gemm_bf16_plan(const GemmDesc& d);

@@ -18,7 +18,7 @@ int da_fix(void* v, const void* alt, int dtype, long long n, int batch, const in
 int da_fix_sum(const float* part, int parts, long long pstride, void* v, const void* alt, int dtype, long long n,
                int batch, const int* nonzero, hipStream_t s);
 // R, qn: rows x r (r % 8 == 0); the Q state receives the first q_cols columns as a contiguous rows x q_cols
-// matrix.  `sums` is scratch for batch * r doubles.
+// matrix.  `sums` is scratch for (1 + min(ceil(rows / 64), 1024)) * batch * r doubles.
 int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_dtype, int rows, int r, int q_cols,
                float eps, int batch, double* sums, hipStream_t s);
 

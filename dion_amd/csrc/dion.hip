@@ -188,12 +188,12 @@ __global__ __launch_bounds__(256) void fix_sum_kernel(const float* __restrict__ 
 // Column normalisation of R[b] (rows x r, TM): Qn = R / (sqrt(sum_rows R^2) + eps), computed in
 // fp32 (column sums accumulated in fp64), stored as TM into qn[b] and, cast to TQ, into the
 // optimizer's Q state (its first q_cols columns: the working matrices may carry zero columns up to a
-// multiple of 8).  Two launches: partial column sums over row slices (fp64 atomics into a
-// zeroed buffer), then a fully parallel normalise pass.
+// multiple of 8).  Three launches: partial column sums over row slices, their sum in slice order (so the
+// result does not depend on which workgroup finishes first), then a fully parallel normalise pass.
 template <typename TM>
-__global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, double* __restrict__ sums, int rows, int r,
+__global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, double* __restrict__ part, int rows, int r,
                                                      int rows_per_slice) {
-  __shared__ double part[4][64];
+  __shared__ double red[4][64];
   const int b = blockIdx.z;
   const int c = blockIdx.x * 64 + (threadIdx.x & 63);
   const int g = threadIdx.x >> 6;
@@ -206,12 +206,22 @@ __global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, d
       const float v = ld_as_float<TM>(Rb + (long long)i * r + c);
       s += (double)v * (double)v;
     }
-  part[g][threadIdx.x & 63] = s;
+  red[g][threadIdx.x & 63] = s;
   __syncthreads();
   if (g == 0 && c < r) {
-    const double t = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-    atomicAdd(sums + (long long)b * r + c, t);
+    const double t = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    part[((long long)blockIdx.y * gridDim.z + b) * r + c] = t;
   }
+}
+
+// sums[b][c] = part[0][b][c] + part[1][b][c] + ... in that order
+__global__ __launch_bounds__(256) void colsum_finish_kernel(const double* __restrict__ part, double* __restrict__ sums,
+                                                            int slices, long long per_slice) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= per_slice) return;
+  double s = 0.0;
+  for (int k = 0; k < slices; ++k) s += part[k * per_slice + i];
+  sums[i] = s;
 }
 
 template <typename TM, typename TQ>
@@ -244,11 +254,6 @@ __global__ __launch_bounds__(256) void colscale_kernel(const TM* __restrict__ R,
         if (c0 + e < q_cols) st_from_float<TQ>(Q + row * q_cols + c0 + e, q[e]);
     }
   }
-}
-
-__global__ void fill_f64_kernel(double* p, long long n) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0.0;
 }
 
 inline unsigned ew_blocks(long long n) {
@@ -339,18 +344,19 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
                float eps, int batch, double* sums, hipStream_t s) {
   if ((r & 7) || q_cols < 1 || q_cols > r) return DA_ERR_ALIGN;
   const long long ns = (long long)batch * r;
-  hipLaunchKernelGGL(fill_f64_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, sums, ns);
   // 64 rows per workgroup (16 per row group): enough workgroups to pull R at the memory system's rate
   int slices = (rows + 63) / 64;
   if (slices > 1024) slices = 1024;
   const int rps = (rows + slices - 1) / slices;
+  double* part = sums + ns;   // [slices][batch][r]
   dim3 g1((r + 63) / 64, slices, batch);
   if (m_dtype == DA_BF16)
-    hipLaunchKernelGGL(colsum_kernel<bf16_t>, g1, dim3(256), 0, s, static_cast<const bf16_t*>(R), sums, rows, r, rps);
+    hipLaunchKernelGGL(colsum_kernel<bf16_t>, g1, dim3(256), 0, s, static_cast<const bf16_t*>(R), part, rows, r, rps);
   else if (m_dtype == DA_F32)
-    hipLaunchKernelGGL(colsum_kernel<float>, g1, dim3(256), 0, s, static_cast<const float*>(R), sums, rows, r, rps);
+    hipLaunchKernelGGL(colsum_kernel<float>, g1, dim3(256), 0, s, static_cast<const float*>(R), part, rows, r, rps);
   else
     return DA_ERR_DTYPE;
+  hipLaunchKernelGGL(colsum_finish_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, part, sums, slices, ns);
   const long long n = (long long)rows * r;
   dim3 g2(ew_blocks(n), batch);
   if (m_dtype == DA_BF16 && q_dtype == DA_BF16)

@@ -19,6 +19,10 @@ struct DaStage {
   float mu;
   int nesterov;
   int muon;
+  // Stand-alone momentum pass (no Newton-Schulz behind it): each result keeps the source orientation and goes
+  // to its own matrix wtab.p[b] (rows x cols, contiguous) instead of the batch `wide`; no partial sums.
+  int use_wtab;
+  DaPtrTable wtab;
 };
 
 struct DaUnstage {
@@ -29,6 +33,10 @@ struct DaUnstage {
   int x_dtype, w_dtype;
   float decay, step;
   int muon;
+  // Stand-alone weight update: the orthogonalised matrices are wtab.p[b] (rows x cols, contiguous, source
+  // orientation) instead of the batch `wide`.
+  int use_wtab;
+  DaPtrTable wtab;
 };
 
 int da_stage_tiles(int rows, int cols);

@@ -114,6 +114,8 @@ struct StageArgs {
   float mu;
   int nesterov;
   int muon;           // 1: momentum update, 0: plain cast
+  int use_wtab;       // 1: result b goes to wtab.p[b] (rows x cols contiguous); never with TALL
+  DaPtrTable wtab;
 };
 
 template <typename TG, typename TM, typename TW, bool TALL>
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
   const TG* G = static_cast<const TG*>(a.g.p[b]);
   TM* M = a.muon ? static_cast<TM*>(a.mom.p[b]) : nullptr;
   const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
-  TW* W = a.wide + (long long)b * mw * a.ldw;
+  TW* W = a.use_wtab ? static_cast<TW*>(a.wtab.p[b]) : a.wide + (long long)b * mw * a.ldw;
 
   float ss = 0.f;
 #pragma unroll
@@ -187,6 +189,7 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
       }
     }
   }
+  if (!a.partials) return;   // (uniform over the grid)
   const float s = block_sum(ss, red);
   if (tid == 0) a.partials[(long long)b * gridDim.x + blockIdx.x] = s;
 }
@@ -242,6 +245,8 @@ struct UnstageArgs {
   float decay;        // 1 - lr * weight_decay
   float step;         // adjusted learning rate
   int muon;           // 1: X <- X*decay - wide*step ; 0: X <- wide
+  int use_wtab;       // 1: source b is wtab.p[b] (rows x cols contiguous); never with TALL
+  DaPtrTable wtab;
 };
 
 template <typename TX, typename TW, bool TALL>
@@ -253,7 +258,7 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
   const int tid = threadIdx.x;
   TX* X = static_cast<TX*>(a.x.p[b]);
   const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
-  const TW* W = a.wide + (long long)b * mw * a.ldw;
+  const TW* W = a.use_wtab ? static_cast<const TW*>(a.wtab.p[b]) : a.wide + (long long)b * mw * a.ldw;
 
   if (TALL) {
 #pragma unroll
@@ -314,19 +319,19 @@ int stage_launch(const StageArgs<TG, TM, TW>& a, int batch, bool tall, hipStream
 template <typename TG, typename TM>
 int stage_dispatch_w(const DaStage& d, hipStream_t s) {
   if (d.w_dtype == DA_BF16) {
-    StageArgs<TG, TM, bf16_t> a{d.g, d.mom, static_cast<bf16_t*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon};
-    return stage_launch(a, d.batch, d.rows > d.cols, s);
+    StageArgs<TG, TM, bf16_t> a{d.g, d.mom, static_cast<bf16_t*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon, d.use_wtab, d.wtab};
+    return stage_launch(a, d.batch, d.rows > d.cols && !d.use_wtab, s);
   }
-  StageArgs<TG, TM, float> a{d.g, d.mom, static_cast<float*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon};
-  return stage_launch(a, d.batch, d.rows > d.cols, s);
+  StageArgs<TG, TM, float> a{d.g, d.mom, static_cast<float*>(d.wide), d.partials, d.rows, d.cols, d.ld, d.ldw, d.mu, d.nesterov, d.muon, d.use_wtab, d.wtab};
+  return stage_launch(a, d.batch, d.rows > d.cols && !d.use_wtab, s);
 }
 
 template <typename TX, typename TW>
 int unstage_launch(const DaUnstage& d, hipStream_t s) {
-  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon};
+  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon, d.use_wtab, d.wtab};
   const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
   dim3 grid(tiles, d.batch);
-  if (d.rows > d.cols) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
+  if (d.rows > d.cols && !d.use_wtab) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((unstage_kernel<TX, TW, false>), grid, dim3(256), 0, s, a);
   return da_launch_status();
 }

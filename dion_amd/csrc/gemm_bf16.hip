@@ -514,7 +514,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
     koff_a += (unsigned)(sa.tstep * 2);                                                            \
     koff_b += (unsigned)(sb.tstep * 2);                                                            \
   } while (0)
-    unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB)
+    unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB: checked by the launcher)
     DA_DMA(lds);
     dma_wait();
     __syncthreads();
@@ -606,6 +606,23 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   epilogue<C, SYM, FULL>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
 }
 
+// Bytes from the first to the last element a workgroup reads of one operand (BT rows, all of K).
+long long da_tile_span_bytes(bool kstrided, int bt, long long ld, long long K) {
+  return 2 * (kstrided ? (K - 1) * ld + bt : (bt - 1) * ld + K);
+}
+
+// Whether every tile of every group is interior for tile edge `bt` (the direct-to-LDS K loop).  That path
+// addresses a tile's operands with 32-bit byte offsets from the tile's first element: an operand whose tile
+// spans 4 GiB or more takes the register-staged path, which walks 64-bit pointers.
+bool all_interior(const GemmDesc* d, int n, int bt) {
+  for (int g = 0; g < n; ++g) {
+    if (d[g].M % bt || d[g].N % bt || d[g].K % BK) return false;
+    if (da_tile_span_bytes(d[g].a_kstrided != 0, bt, d[g].lda, d[g].K) >= (1LL << 32)) return false;
+    if (da_tile_span_bytes(d[g].b_kstrided != 0, bt, d[g].ldb, d[g].K) >= (1LL << 32)) return false;
+  }
+  return true;
+}
+
 template <typename C>
 long long tiles_of(const GemmDesc& d) {
   const long long tm = (d.M + C::BT - 1) / C::BT, tn = (d.N + C::BT - 1) / C::BT;
@@ -628,12 +645,11 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   }
   GemmArgs args{};
   args.n = n;
-  bool full = true;
+  const bool full = all_interior(d, n, BT);
   long long blocks = 0;
   for (int g = 0; g < n; ++g) {
     args.d[g] = d[g];
     args.start[g] = (int)blocks;
-    full = full && (d[g].M % BT == 0) && (d[g].N % BT == 0) && (d[g].K % BK == 0);
     const long long t = tiles_of<C>(d[g]);
     if (t <= 0) return DA_ERR_LIMIT;
     blocks += t;
@@ -693,6 +709,24 @@ double launch_cost(const GemmDesc* d, int n, int slots, double unit) {
   return unit * (level > longest ? level : longest);
 }
 
+typedef Cfg<256, 2, 4> Big;
+typedef Cfg<128, 2, 2> Small;
+
+// Tile choice by cost model: 256 x 256 tiles run one per CU, 128 x 128 tiles two per CU; a small
+// tile does a quarter of the work on half a CU at about 2/3 of the large tile's MFMA efficiency
+// (measured on grouped Newton-Schulz products of 768-wide matrices).
+// Interior-only (direct-to-LDS) eligibility wins over either.
+int choose_tile(const GemmDesc* d, int n) {
+  static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
+  if (forced == 128 || forced == 256) return forced;
+  bool fits_big = true;
+  for (int g = 0; g < n; ++g) fits_big = fits_big && d[g].M >= 256 && d[g].N >= 256;
+  const bool full_big = all_interior(d, n, 256), full_small = all_interior(d, n, 128);
+  const double cost_big = launch_cost<Big>(d, n, 256, 4.0);
+  const double cost_small = launch_cost<Small>(d, n, 512, 3.0);
+  return fits_big && (full_big || !full_small) && cost_big <= cost_small ? 256 : 128;
+}
+
 }  // namespace
 
 // Alignment contract: K, N, every leading dimension and every batch stride are multiples
@@ -712,25 +746,15 @@ int da_gemm_bf16_grouped(const GemmDesc* din, int n, hipStream_t stream) {
     while (pos > 0 && d[pos - 1].K < a.K) { d[pos] = d[pos - 1]; --pos; }
     d[pos] = a;
   }
-  typedef Cfg<256, 2, 4> Big;
-  typedef Cfg<128, 2, 2> Small;
-  static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
-  if (forced == 128) return dispatch_layout<Small>(d, n, stream);
-  if (forced == 256) return dispatch_layout<Big>(d, n, stream);
-  // Tile choice by cost model: 256 x 256 tiles run one per CU, 128 x 128 tiles two per CU; a small
-  // tile does a quarter of the work on half a CU at about 2/3 of the large tile's MFMA efficiency
-  // (measured on grouped Newton-Schulz products of 768-wide matrices).
-  // Interior-only (direct-to-LDS) eligibility wins over either.
-  bool full_big = true, full_small = true, fits_big = true;
-  for (int g = 0; g < n; ++g) {
-    full_big = full_big && d[g].M % 256 == 0 && d[g].N % 256 == 0 && d[g].K % BK == 0;
-    full_small = full_small && d[g].M % 128 == 0 && d[g].N % 128 == 0 && d[g].K % BK == 0;
-    fits_big = fits_big && d[g].M >= 256 && d[g].N >= 256;
-  }
-  const double cost_big = launch_cost<Big>(d, n, 256, 4.0);
-  const double cost_small = launch_cost<Small>(d, n, 512, 3.0);
-  if (fits_big && (full_big || !full_small) && cost_big <= cost_small) return dispatch_layout<Big>(d, n, stream);
+  if (choose_tile(d, n) == 256) return dispatch_layout<Big>(d, n, stream);
   return dispatch_layout<Small>(d, n, stream);
+}
+
+// What the launcher would do with one product of these dimensions, without launching anything:
+// tile edge (128 or 256), plus 1 if the K loop is the direct-to-LDS one.
+int da_gemm_bf16_plan(const GemmDesc& d) {
+  const int bt = choose_tile(&d, 1);
+  return bt + (all_interior(&d, 1, bt) ? 1 : 0);
 }
 
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) { return da_gemm_bf16_grouped(&d, 1, stream); }

@@ -9,6 +9,7 @@
 // plain indexed LDS read: k-contiguous tiles are kept [128][16+1], k-strided tiles
 // [16][128+4], both conflict-free for the 32-rows-per-half-wave fragment read.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -57,7 +58,10 @@ __device__ __forceinline__ float read_frag(const float* lds, int r0, int ks, int
   return KS ? lds[k * KS_LD + row] : lds[row * KC_LD + k];
 }
 
-template <bool A_KS, bool B_KS, bool SYM>
+// CBF: C and E are bf16 (fp32 factors updating bf16 weights): the addend is scaled and rounded in C's dtype
+// first, as an in-place  X.mul_(s0); X.add_(fp32 update)  on a bf16 tensor does, and the sum is rounded once
+// at the store.
+template <bool A_KS, bool B_KS, bool SYM, bool CBF>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
   constexpr int A_FL = A_KS ? KS_FLOATS : KC_FLOATS;
   constexpr int B_FL = B_KS ? KS_FLOATS : KC_FLOATS;
@@ -130,10 +134,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
 
   const bool mirror = SYM && (ti != tj);
   const bool has_e = d.epilogue == DA_EPI_AXPBY;
-  float* const Cbase = d.Ctab ? static_cast<float*>(d.Ctab[b]) : static_cast<float*>(d.C) + (long long)b * d.sC;
-  const float* const Ebase = !has_e ? nullptr
-                             : d.Etab ? static_cast<const float*>(d.Etab[b])
-                                      : static_cast<const float*>(d.E) + (long long)b * d.sE;
+  typedef typename std::conditional<CBF, bf16_t, float>::type TC;
+  TC* const Cbase = d.Ctab ? static_cast<TC*>(d.Ctab[b]) : static_cast<TC*>(d.C) + (long long)b * d.sC;
+  const TC* const Ebase = !has_e ? nullptr
+                          : d.Etab ? static_cast<const TC*>(d.Etab[b])
+                                   : static_cast<const TC*>(d.E) + (long long)b * d.sE;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int m = m0 + wm * 64 + i * 32 + (lane & 31);
@@ -143,20 +148,34 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
       for (int vq = 0; vq < 4; ++vq) {
         const int n = n0 + wn * 64 + j * 32 + vq * 8 + (lane >> 5) * 4;
         if (m >= d.M || n >= d.N) continue;
-        float* Cp = Cbase + (long long)m * d.ldc + n;
+        TC* Cp = Cbase + (long long)m * d.ldc + n;
         float o[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) o[q] = d.s1 * acc[i][j][vq * 4 + q];
-        if (has_e) {
-          const float4 ev = *reinterpret_cast<const float4*>(Ebase + (long long)m * d.lde + n);
-          o[0] = d.s0 * ev.x + o[0]; o[1] = d.s0 * ev.y + o[1];
-          o[2] = d.s0 * ev.z + o[2]; o[3] = d.s0 * ev.w + o[3];
-        }
-        *reinterpret_cast<float4*>(Cp) = make_float4(o[0], o[1], o[2], o[3]);
-        if (mirror) {
-          float* Ct = Cbase + (long long)n * d.ldc + m;
+        if constexpr (CBF) {
+          if (has_e) {
+            const uint2 ev = *reinterpret_cast<const uint2*>(Ebase + (long long)m * d.lde + n);
+            const float e[4] = {__builtin_bit_cast(float, ev.x << 16), __builtin_bit_cast(float, ev.x & 0xffff0000u),
+                                __builtin_bit_cast(float, ev.y << 16), __builtin_bit_cast(float, ev.y & 0xffff0000u)};
 #pragma unroll
-          for (int q = 0; q < 4; ++q) Ct[(long long)q * d.ldc] = o[q];
+            for (int q = 0; q < 4; ++q) o[q] = rbf(d.s0 * e[q]) + o[q];
+          }
+          uint2 w;
+          w.x = (uint32_t)f2bf(o[0]) | ((uint32_t)f2bf(o[1]) << 16);
+          w.y = (uint32_t)f2bf(o[2]) | ((uint32_t)f2bf(o[3]) << 16);
+          *reinterpret_cast<uint2*>(Cp) = w;
+        } else {
+          if (has_e) {
+            const float4 ev = *reinterpret_cast<const float4*>(Ebase + (long long)m * d.lde + n);
+            o[0] = d.s0 * ev.x + o[0]; o[1] = d.s0 * ev.y + o[1];
+            o[2] = d.s0 * ev.z + o[2]; o[3] = d.s0 * ev.w + o[3];
+          }
+          *reinterpret_cast<float4*>(Cp) = make_float4(o[0], o[1], o[2], o[3]);
+        }
+        if (mirror) {
+          TC* Ct = Cbase + (long long)n * d.ldc + m;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) st_from_float<TC>(Ct + (long long)q * d.ldc, o[q]);
         }
       }
     }
@@ -165,22 +184,24 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmDesc d) {
 
 template <bool A_KS, bool B_KS, bool SYM>
 int launch(const GemmDesc& d, hipStream_t stream) {
+  const bool cbf = d.c_dtype == DA_BF16;
   const int tiles_m = (d.M + BT - 1) / BT, tiles_n = (d.N + BT - 1) / BT;
   const long long per_batch = SYM ? (long long)tiles_m * (tiles_m + 1) / 2 : (long long)tiles_m * tiles_n;
   const long long blocks = per_batch * d.batch;
   if (blocks <= 0 || blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
-  hipLaunchKernelGGL((gemm_f32_kernel<A_KS, B_KS, SYM>), dim3((unsigned)blocks), dim3(256), 0, stream, d);
+  if (cbf) hipLaunchKernelGGL((gemm_f32_kernel<A_KS, B_KS, SYM, true>), dim3((unsigned)blocks), dim3(256), 0, stream, d);
+  else hipLaunchKernelGGL((gemm_f32_kernel<A_KS, B_KS, SYM, false>), dim3((unsigned)blocks), dim3(256), 0, stream, d);
   return da_launch_status();
 }
 
 }  // namespace
 
 // Alignment contract: K, N, leading dimensions and batch strides multiples of 4 elements,
-// M too when A is k-strided; pointers 16-byte aligned.  C and E are fp32.
+// M too when A is k-strided; pointers 16-byte aligned.  C and E are fp32, or bf16 (rounded at the store).
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream) {
   if ((!d.A && !d.Atab) || (!d.B && !d.Btab) || (!d.C && !d.Ctab) || d.M <= 0 || d.N <= 0 || d.K <= 0 || d.batch <= 0) return DA_ERR_ARG;
   if (d.epilogue == DA_EPI_AXPBY && !d.E && !d.Etab) return DA_ERR_ARG;
-  if (d.c_dtype != DA_F32) return DA_ERR_DTYPE;
+  if (d.c_dtype != DA_F32 && d.c_dtype != DA_BF16) return DA_ERR_DTYPE;
   if ((d.K | d.N | d.lda | d.ldb | d.ldc) & 3) return DA_ERR_ALIGN;
   if ((d.sA | d.sB | d.sC) & 3) return DA_ERR_ALIGN;
   if ((d.E || d.Etab) && ((d.lde & 3) || (d.sE & 3))) return DA_ERR_ALIGN;

@@ -161,7 +161,8 @@ class Dion(Optimizer):
         return
 
     def cholesky_info(self) -> Dict[Tuple, Tensor]:
-        """Device tensors with the orthonormaliser's per-matrix status of the last step, keyed by bucket:
+        """Device tensors with the orthonormaliser's per-matrix status of the last step, keyed by bucket
+        (shape, dtype, gradient dtype, device):
         0 = success, k > 0 = pivot k-1 was not positive (the analogue of `torch.linalg.cholesky_ex`'s info)."""
         return dict(self._info)
 
@@ -246,9 +247,10 @@ class Dion(Optimizer):
             _lib.require_gpu(plist[0], "Dion.step")
             for p in plist:
                 self._get_or_initialize_state(p, group)
-            info = self._info.get((shape, dtype, device))
+            key = (shape, dtype, gdtype, device)
+            info = self._info.get(key)
             if info is None or info.numel() != len(plist):
-                self._info[(shape, dtype, device)] = torch.zeros(len(plist), dtype=torch.int32, device=device)
+                self._info[key] = torch.zeros(len(plist), dtype=torch.int32, device=device)
         slots = min(len(buckets), self._max_concurrent_tasks)
         forked = {}
         for index, ((shape, dtype, gdtype, device), plist) in enumerate(buckets.items()):
@@ -274,7 +276,7 @@ class Dion(Optimizer):
                     raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
             scaled_lr = ((m / n) ** 0.5) * lr
             mcode = _lib.dtype_code(Ms[0].dtype)
-            info = self._info[(shape, dtype, device)]
+            info = self._info[(shape, dtype, gdtype, device)]
             with torch.cuda.device(device), torch.cuda.stream(stream):
                 # contiguous gradient copies and the workspace belong to this stream
                 Xs = plist

@@ -62,7 +62,7 @@ class Muon(Optimizer):
         lr, mu, betas, weight_decay, epsilon, nesterov, adjust_lr, flatten: as in the reference.
         use_triton: accepted and ignored; the HIP kernels are always used.
         newton_schulz_func: optional custom `func(input: Tensor, epsilon) -> Tensor`; when
-            given, the matrices take an unfused PyTorch pre/post pass around that function.
+            given, the momentum pass and the weight update run as separate kernels around that function.
     """
 
     def __init__(
@@ -244,23 +244,61 @@ class Muon(Optimizer):
         return X, G, M
 
     def _muon_bucket_unfused(self, plist, states, lr, adjusted_lr, mu, weight_decay, epsilon, group):
-        """Custom `newton_schulz_func`: PyTorch pre/post passes around the user function
-        (op sequence of reference dion/muon.py:536-552, 568-573, 585-593)."""
-        for p, st in zip(plist, states):
-            M = st["momentum"]
-            g = p.grad.to(dtype=M.dtype)
-            M.mul_(mu.to(M.device)).add_(g)
-            U = (M * mu.to(M.device)).add_(g) if group["nesterov"] else M
-            U = U.to(dtype=torch.bfloat16)
-            shape = U.shape
-            if group["flatten"] and U.ndim >= 3:
-                U = U.flatten(start_dim=1)
-            elif U.ndim >= 4:
-                U = U.flatten(end_dim=-3)
-            U = self._newton_schulz_func(U, epsilon=epsilon).reshape(shape)
-            p.mul_((1 - lr * weight_decay).to(p.device))
-            alr = adjusted_lr if isinstance(adjusted_lr, Tensor) else torch.tensor(adjusted_lr)
-            p.sub_(U * alr.to(p.device))
+        """Custom `newton_schulz_func` (the reference's plug-in hook, dion/muon.py:48-49, 122-131): the momentum pass
+        and the weight update run as the library's stand-alone stages (`dion_amd_muon_pre` / `dion_amd_muon_post`,
+        reference dion/muon.py:536-552 and 568-573) around the user's function, which is called per parameter with
+        the reference's flatten rules (585-593) and a 0-dim fp32 `epsilon` tensor."""
+        lib = _lib.load()
+        p0 = plist[0]
+        _lib.require_gpu(p0, "Muon.step")
+        device = p0.device
+        cols = p0.size(-1)
+        rows = p0.numel() // cols
+        Ms = [st["momentum"] for st in states]
+        for t in (*plist, *Ms):
+            if not t.is_contiguous():
+                raise _lib.DionAmdError("Muon.step: parameters and momentum buffers must be contiguous")
+        X = [p.view(rows, cols) for p in plist]
+        G = [(p.grad if p.grad.is_contiguous() else p.grad.contiguous()).view(rows, cols) for p in plist]
+        M = [m.view(rows, cols) for m in Ms]
+        crops = []
+        c8 = cols
+        if cols % 8:
+            # the stages move 16-byte row segments: step zero-padded copies and crop the results back
+            c8 = -(-cols // 8) * 8
+            Xw, Gw, Mw = (_lib.zero_padded(t, rows, c8) for t in (X, G, M))
+            crops = [(X, Xw), (M, Mw)]
+            X, G, M = list(Xw.unbind(0)), list(Gw.unbind(0)), list(Mw.unbind(0))
+        U = torch.empty((len(plist), rows, c8), dtype=torch.bfloat16, device=device)
+        Us = list(U.unbind(0))
+        with torch.cuda.device(device):
+            rc = lib.dion_amd_muon_pre(
+                _lib.ptr_array(G), _lib.ptr_array(M), _lib.ptr_array(Us), len(plist), rows, c8,
+                _lib.dtype_code(G[0].dtype), _lib.dtype_code(M[0].dtype), mu.item(), int(bool(group["nesterov"])),
+                _lib.stream_ptr(device))
+        _lib.check(rc, "dion_amd_muon_pre")
+        O = []
+        for p, u in zip(plist, Us):
+            u = u[:, :cols].reshape(p.shape) if c8 != cols else u.view(p.shape)
+            if group["flatten"] and u.ndim >= 3:
+                v = u.flatten(start_dim=1)
+            elif u.ndim >= 4:
+                v = u.flatten(end_dim=-3)
+            else:
+                v = u
+            o = self._newton_schulz_func(v, epsilon=epsilon).reshape(p.shape)
+            o = o.to(dtype=torch.bfloat16).reshape(rows, cols)
+            if c8 != cols:
+                o = torch.nn.functional.pad(o, (0, c8 - cols))
+            O.append(o.contiguous())
+        alr = adjusted_lr.item() if isinstance(adjusted_lr, Tensor) else float(torch.tensor(adjusted_lr).item())
+        with torch.cuda.device(device):
+            rc = lib.dion_amd_muon_post(
+                _lib.ptr_array(X), _lib.ptr_array(O), len(plist), rows, c8, _lib.dtype_code(X[0].dtype),
+                (1 - lr * weight_decay).item(), alr, _lib.stream_ptr(device))
+        _lib.check(rc, "dion_amd_muon_post")
+        for dst, padded in crops:
+            _lib.crop_back(dst, padded)
 
     # ------------------------------------------------------------------ element-wise groups
     def _lion_group_step(self, group: dict):

@@ -15,6 +15,7 @@
  *   - Return value: 0 ok; <0 argument error (DION_AMD_ERR_*); >0 a hipError_t.
  *   - Alignment: bf16 matrices need every dimension, pitch and batch stride to be a
  *     multiple of 8 elements and 16-byte aligned base pointers (fp32: multiples of 4).
+ *     A `workspace` pointer must be 256-byte aligned (the library carves it up itself).
  *     Violations return DION_AMD_ERR_ALIGN; nothing is launched.
  */
 #ifndef DION_AMD_H
@@ -88,7 +89,7 @@ int dion_amd_sym_poly(const void* A, long long a_stride, int lda,
  *   C_b (M x N) = s0 * E_b + s1 * sum_k Aop_b(i,k) Bop_b(j,k)      (epilogue AXPBY)
  *   C_b         = s1 * sum_k ...                                   (epilogue STORE)
  * a_kstrided = 0: A stored M x K (pitch lda); 1: stored K x M.  Same for B (N x K / K x N).
- * in_dtype bf16 or f32; c_dtype (for C and E) bf16 or f32 (f32 only when in_dtype is f32).
+ * in_dtype bf16 or f32; c_dtype (for C and E) bf16 or f32, in any combination.
  * E may alias C. */
 int dion_amd_gemm(const void* A, long long a_stride, int lda, int a_kstrided,
                   const void* B, long long b_stride, int ldb, int b_kstrided,
@@ -97,6 +98,13 @@ int dion_amd_gemm(const void* A, long long a_stride, int lda, int a_kstrided,
                   int batch, int M, int N, int K,
                   int in_dtype, int c_dtype, int epilogue, float s0, float s1,
                   int faithful, void* stream);
+
+/* What the bf16 launcher behind dion_amd_gemm would do with one product of these dimensions
+ * (host-side query, nothing is launched; no counterpart in the reference): the tile edge it
+ * picks (128 or 256), plus 1 if the product runs the interior-only K loop that stages operands
+ * with direct-to-LDS loads.  That loop addresses a tile's operands with 32-bit byte offsets:
+ * an operand whose tile spans 4 GiB or more takes the bounds-checked loop instead. */
+int dion_amd_gemm_plan(int M, int N, int K, int lda, int a_kstrided, int ldb, int b_kstrided);
 
 /* ---------------------------------------------------------------------------------------
  * Muon step for one bucket of same-shape matrices
@@ -119,6 +127,24 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
                        float mu, int nesterov, float decay, float adjusted_lr,
                        const float* coeffs, int steps, float eps, int faithful,
                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* The two element-wise stages of a Muon step on their own, for a caller that supplies its own
+ * orthogonalisation (the reference's plug-in hook `newton_schulz_func`, dion/muon.py:48-49,
+ * 122-131, called at 585-593).
+ *
+ * dion_amd_muon_pre replaces muon_update_pre_orthogonalize (reference dion/muon.py:525-552):
+ * per matrix  M <- mu M + G (G cast to M's dtype first);  U = bf16(nesterov ? mu M + G : M),
+ * with the reference's rounding after every tensor op.  G, M, U: HOST arrays of `batch` device
+ * pointers to contiguous m x n matrices (n a multiple of 8); U receives bf16.
+ *
+ * dion_amd_muon_post replaces muon_update_post_orthogonalize (reference dion/muon.py:556-573):
+ * X <- decay X;  X <- X - bf16(adjusted_lr O)  for bf16 O of the same shape. */
+int dion_amd_muon_pre(const void* const* G, void* const* M, void* const* U,
+                      int batch, int m, int n, int g_dtype, int m_dtype,
+                      float mu, int nesterov, void* stream);
+int dion_amd_muon_post(void* const* X, const void* const* O,
+                       int batch, int m, int n, int x_dtype,
+                       float decay, float adjusted_lr, void* stream);
 
 /* Several buckets (each of one shape) in one call.  Replaces the task generator and the task
  * runtime around muon_update_batch_async (reference dion/muon.py:185-270 _create_muon_tasks,
@@ -213,7 +239,7 @@ size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype
  *   M <- B - (1-mu) P R^T  (transposed back when m < n);   Q <- R / (||R||_col + eps);
  *   X <- decay X - scaled_lr P Q^T.
  * ef_alpha = -(1 - mu), decay = 1 - lr*wd and scaled_lr = sqrt(m/n)*lr are passed as
- * already-evaluated fp32 values.  m_dtype f32 requires x_dtype f32.  info as above.
+ * already-evaluated fp32 values.  Every combination of bf16 / f32 for x, g, m and q is accepted.  info as above.
  * power_iters >= 1 repeats P = orth(B' Q), Q = B'^T P before the updates, the unnormalised R serving as the
  * next Q (reference dion/dion_reference.py:690-730; the batched reference class only allows 1).
  * m and n must be multiples of 8 (the host side pads other shapes with zero rows / columns,

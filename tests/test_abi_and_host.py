@@ -51,6 +51,27 @@ def test_workspace_queries_and_argument_errors_without_gpu():
         _lib.dtype_code(torch.float16)
 
 
+def test_gemm_plan_keeps_huge_operands_off_the_32_bit_offset_path():
+    """The direct-to-LDS K loop addresses a tile's operand with 32-bit byte offsets: an operand whose tile spans
+    4 GiB or more (a k-strided bf16 matrix of 131136 rows x 16384 columns, as in R = B^T P of a vocabulary-sized layer) must
+    take the bounds-checked loop.  Host-side query, nothing is launched."""
+    from dion_amd import _lib
+
+    lib = _lib.load()
+    # interior tiles, small operands: 256-wide tile on the direct path
+    assert lib.dion_amd_gemm_plan(4096, 4096, 4096, 4096, 0, 4096, 0) == 257
+    # A k-strided with (K - 1) * ld * 2 bytes = 131135 * 16384 * 2 >= 2^32: checked loop
+    assert lib.dion_amd_gemm_plan(16384, 512, 131136, 16384, 1, 512, 1) % 2 == 0
+    # just below the limit stays on the direct path
+    assert lib.dion_amd_gemm_plan(16384, 512, 131008, 16384, 1, 512, 1) % 2 == 1
+    # a k-contiguous operand is addressed per tile row: (tile rows - 1) x pitch
+    assert lib.dion_amd_gemm_plan(4096, 4096, 4096, 1 << 25, 0, 4096, 0) % 2 == 0
+    assert lib.dion_amd_gemm_plan(4096, 4096, 4096, 1 << 20, 0, 4096, 0) % 2 == 1
+    # ragged sizes never take it
+    assert lib.dion_amd_gemm_plan(200, 136, 72, 72, 0, 72, 0) % 2 == 0
+    assert lib.dion_amd_gemm_plan(0, 8, 8, 8, 0, 8, 0) == -1
+
+
 def test_no_cpu_fallback():
     from dion_amd import Dion, Muon, _lib, zeropower_via_newtonschulz5
 

@@ -221,6 +221,24 @@ def test_dion_bf16_momentum(dev):
               check=check)
 
 
+def test_dion_fp32_momentum_with_bf16_weights(dev):
+    """`DionMixedPrecisionConfig(momentum_dtype=float32)` on bf16 parameters (the reference accepts it:
+    `foreach_baddbmm_` adds the fp32 update into the bf16 weights, dion/dion.py:1513-1530): fp32 factors, bf16 X."""
+    def check(step, params, opt, Xo, Mo, Qo):
+        for i, p in enumerate(params):
+            st = opt.state[p]
+            assert p.dtype == torch.bfloat16 and st["momentum"].dtype == torch.float32
+            eM, eX = rel_fro(st["momentum"], Mo[i]), rel_fro(p.detach(), Xo[i])
+            eQ = rel_fro(_sign_align(st["Q"].cpu(), Qo[i]), Qo[i])
+            assert eM <= FP32_TOL and eQ <= FP32_TOL, (step, i, eM, eQ)
+            # bf16 weights: the two runs may round an element differently once in a while
+            assert eX <= 2e-3, (step, i, eX)
+            assert (p.detach().cpu() == Xo[i]).float().mean().item() > 0.98
+
+    _run_dion(dev, [(256, 128), (128, 256), (192, 192)], 0.25, 4, torch.bfloat16, torch.float32, torch.float32,
+              check=check)
+
+
 def test_dion_all_zero_gradient(dev):
     """All-zero B: P = 0, Q_new = colnorm(Q), M = 0, X = (1 - lr wd) X (reference dion/dion.py:1416-1444)."""
     from dion_amd import Dion

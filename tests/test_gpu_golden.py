@@ -75,11 +75,29 @@ def test_dion_two_steps_vs_reference_vectors(dev, gold, dt, name):
 
 
 def test_muon_step_vs_reference_vectors(dev, gold):
-    """The reference's own momentum pass output U, orthogonalised on the GPU and applied, against the
-    reference's post pass applied to the reference's NS of the same U (all from the golden file)."""
+    """`Muon.step()` with the golden file's orthogonalised matrix plugged in through `newton_schulz_func`: momentum,
+    the matrix handed to the hook, and the updated weights are the reference's own, bit for bit (the momentum pass
+    and the weight update are element-wise with the reference's rounding points)."""
     from dion_amd import Muon
 
     for dt, dtype in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+        for nest in (True, False):
+            tag = f"muon_{dt}_{'nesterov' if nest else 'plain'}"
+            seen = []
+
+            def hook(U, epsilon):
+                seen.append(U.detach().float().cpu())
+                return gold[f"muon_{dt}_Uo"].bfloat16().to(dev)
+
+            p = torch.nn.Parameter(gold[f"muon_{dt}_X0"].to(dtype).to(dev))
+            p.grad = gold[f"muon_{dt}_G"].to(dtype).to(dev)
+            opt = Muon([p], lr=0.02, mu=0.95, weight_decay=0.01, nesterov=nest, newton_schulz_func=hook)
+            opt.state[p]["momentum"] = gold[f"muon_{dt}_M0"].to(dtype).to(dev)
+            opt.step()
+            assert torch.equal(opt.state[p]["momentum"].float().cpu(), gold[tag + "_M1"])
+            assert len(seen) == 1 and torch.equal(seen[0], gold[tag + "_U"])
+            assert torch.equal(p.detach().float().cpu(), gold[f"muon_{dt}_X1"])
+        # the fused path (library Newton-Schulz): same momentum
         p = torch.nn.Parameter(gold[f"muon_{dt}_X0"].to(dtype).to(dev))
         p.grad = gold[f"muon_{dt}_G"].to(dtype).to(dev)
         opt = Muon([p], lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True)

@@ -189,6 +189,69 @@ def test_muon_custom_newton_schulz_hook(dev):
     assert torch.allclose(p.detach(), torch.full_like(p, 1 - 0.1 * 0.5), atol=1e-3)  # U * lr rounds in bf16
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_muon_hook_path_matches_oracle(dev, dtype):
+    """The plug-in hook path (stand-alone momentum pass and weight update around a user function) against the
+    oracle's step with the same function: a deterministic element-wise stand-in for the orthogonalisation, so every
+    tensor must match bit for bit -- 2-D, a batch of matrices, a flattened conv weight and a column count off the
+    8-grid."""
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    def stand_in(X, epsilon):
+        assert X.dtype == torch.bfloat16 and X.ndim in (2, 3)
+        return (X.float() * 3.0).bfloat16() - (X.float() * X.float()).bfloat16()
+
+    shapes = [(64, 96), (64, 96), (3, 32, 40), (16, 4, 3, 3), (40, 27)]
+    gen = torch.Generator().manual_seed(21)
+    X0 = [(torch.randn(s, generator=gen) * 0.02).to(dtype) for s in shapes]
+    Xo, Mo = [x.clone() for x in X0], [torch.zeros_like(x) for x in X0]
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    groups = [dict(params=[params[0], params[1], params[2], params[4]]), dict(params=[params[3]], flatten=True)]
+    opt = Muon(groups, lr=0.02, mu=0.9, weight_decay=0.01, nesterov=True, newton_schulz_func=stand_in)
+    for step in range(3):
+        G = [(torch.randn(s, generator=gen) * 1e-1).to(dtype) for s in shapes]
+        for p, g in zip(params, G):
+            p.grad = g.to(dev)
+        for i in range(len(shapes)):
+            O.muon_step([Xo[i]], [G[i]], [Mo[i]], lr=0.02, mu=0.9, weight_decay=0.01, nesterov=True,
+                        flatten=(i == 3), ns_func=stand_in)
+        opt.step()
+        for i, p in enumerate(params):
+            assert torch.equal(opt.state[p]["momentum"].cpu(), Mo[i]), (step, i)
+            assert torch.equal(p.detach().cpu(), Xo[i]), (step, i)
+
+
+def test_newton_schulz_accepts_16_byte_aligned_views(dev):
+    """A contiguous view such as `grad[1]` of a 3 x 136 x 200 tensor starts 16-byte, not 256-byte, aligned: it goes
+    through the C entry point as it is and gives what a fresh copy of the same matrix gives."""
+    from dion_amd import _lib
+    from dion_amd.newton_schulz import NS_SCHEDULE_COEFFS, flat_coeffs
+
+    lib = _lib.load()
+    torch.manual_seed(3)
+    big = torch.randn(3, 136, 200, device=dev).bfloat16()
+    view = big[1]
+    assert view.data_ptr() % 256 != 0 and view.data_ptr() % 16 == 0
+    outs = []
+    for src in (view, view.clone()):
+        out_all = torch.empty(2, 136, 200, dtype=torch.bfloat16, device=dev)
+        out = out_all[1] if src is view else out_all[0]
+        ws = torch.empty(lib.dion_amd_ns_workspace_bytes(1, 136, 200, _lib.BF16), dtype=torch.uint8, device=dev)
+        rc = lib.dion_amd_newton_schulz(src.data_ptr(), _lib.BF16, 136 * 200, 200, out.data_ptr(), 136 * 200, 200,
+                                        1, 136, 200, flat_coeffs(NS_SCHEDULE_COEFFS), 5, 1e-7, _lib.BF16, 1,
+                                        ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+        assert rc == 0, rc
+        outs.append(out.clone())
+    assert torch.equal(outs[0], outs[1])
+    # 8 bytes off: refused, nothing launched
+    flat = torch.zeros(136 * 200 + 8, dtype=torch.bfloat16, device=dev)
+    rc = lib.dion_amd_newton_schulz(flat.data_ptr() + 8, _lib.BF16, 136 * 200, 200, out.data_ptr(), 136 * 200, 200,
+                                    1, 136, 200, flat_coeffs(NS_SCHEDULE_COEFFS), 5, 1e-7, _lib.BF16, 1,
+                                    ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev))
+    assert rc == -2
+
+
 def test_muon_step_buckets_equals_per_bucket_calls(dev):
     """The multi-bucket entry (grouped launches, more buckets than one grouped launch takes, a bucket
     of more matrices than one staging launch takes, shapes that are not multiples of the tile) gives
