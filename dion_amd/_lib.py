@@ -43,6 +43,8 @@ _SIGNATURES = {
     "dion_amd_version": (_c.c_char_p, []),
     "dion_amd_ns_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "dion_amd_newton_schulz": (_i, [_vp, _i, _ll, _i, _vp, _ll, _i, _i, _i, _i, _fp, _i, _f, _i, _i, _vp, _sz, _vp]),
+    "dion_amd_static_scratch_bytes": (_sz, []),
+    "dion_amd_newton_schulz_static": (_i, [_vp, _i, _ll, _i, _vp, _ll, _i, _i, _i, _i, _fp, _i, _f, _i, _i, _vp]),
     "dion_amd_syrk": (_i, [_vp, _ll, _i, _vp, _ll, _i, _i, _i, _i, _i, _vp]),
     "dion_amd_sym_poly": (_i, [_vp, _ll, _i, _vp, _ll, _i, _i, _i, _f, _f, _i, _i, _vp]),
     "dion_amd_gemm": (_i, [_vp, _ll, _i, _i, _vp, _ll, _i, _i, _vp, _ll, _i, _vp, _ll, _i,

@@ -3,6 +3,7 @@
 #include "../../include/dion_amd.h"
 #include "common.h"
 #include <cstdlib>
+#include <mutex>
 #include "elementwise.h"
 #include "prof.h"
 #include "dion.h"
@@ -209,9 +210,13 @@ size_t dion_amd_ns_workspace_bytes(int batch, int m, int n, int compute_dtype) {
   return NsLayout(m, n, compute_dtype).recommended(batch);
 }
 
-int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int ldg, void* out, long long out_stride,
-                           int ldo, int batch, int m, int n, const float* coeffs, int steps, float eps,
-                           int compute_dtype, int faithful, void* workspace, size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+namespace {
+
+int ns_run(const void* G, int g_dtype, long long g_stride, int ldg, void* out, long long out_stride, int ldo,
+           int batch, int m, int n, const float* coeffs, int steps, float eps, int compute_dtype, int faithful,
+           void* workspace, size_t workspace_bytes, void* stream) {
   if (!G || !out || !coeffs || !workspace || batch <= 0 || m <= 0 || n <= 0 || steps < 0) return DA_ERR_ARG;
   if (!dtype_ok(g_dtype) || !dtype_ok(compute_dtype)) return DA_ERR_DTYPE;
   if ((m | n | ldg | ldo) & 7) return DA_ERR_ALIGN;
@@ -257,6 +262,56 @@ int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int l
     if (rc) return rc;
   }
   return DA_OK;
+}
+
+// Working memory of dion_amd_newton_schulz_static: one array per GPU, part of the library's device image (it lives
+// as long as the process).  Host code never uses the array's name as an address: `static_scratch()` asks the
+// runtime for the device address on the current GPU, once per device, and hands that pointer on.
+static __device__ __align__(256) unsigned char scratch[DION_AMD_STATIC_SCRATCH_BYTES];
+constexpr int DA_MAX_DEVICES = 64;
+void* g_scratch_ptr[DA_MAX_DEVICES];
+std::mutex g_scratch_mutex;
+
+int static_scratch(void** ptr) {
+  int dev = -1;
+  DA_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= DA_MAX_DEVICES) return DA_ERR_LIMIT;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    DA_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return DA_ERR_ARG;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return DA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int ldg, void* out, long long out_stride,
+                           int ldo, int batch, int m, int n, const float* coeffs, int steps, float eps,
+                           int compute_dtype, int faithful, void* workspace, size_t workspace_bytes, void* stream) {
+  return ns_run(G, g_dtype, g_stride, ldg, out, out_stride, ldo, batch, m, n, coeffs, steps, eps, compute_dtype,
+                faithful, workspace, workspace_bytes, stream);
+}
+
+size_t dion_amd_static_scratch_bytes(void) { return DION_AMD_STATIC_SCRATCH_BYTES; }
+
+int dion_amd_newton_schulz_static(const void* G, int g_dtype, long long g_stride, int ldg, void* out,
+                                  long long out_stride, int ldo, int batch, int m, int n, const float* coeffs,
+                                  int steps, float eps, int compute_dtype, int faithful, void* stream) {
+  if (batch <= 0 || m <= 0 || n <= 0) return DA_ERR_ARG;
+  if (!dtype_ok(compute_dtype)) return DA_ERR_DTYPE;
+  // one matrix's working set must fit the array (a batch then goes through it in chunks)
+  if (NsLayout(m, n, compute_dtype).per_matrix > (size_t)DION_AMD_STATIC_SCRATCH_BYTES) return DA_ERR_LIMIT;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  return ns_run(G, g_dtype, g_stride, ldg, out, out_stride, ldo, batch, m, n, coeffs, steps, eps, compute_dtype,
+                faithful, ws, DION_AMD_STATIC_SCRATCH_BYTES, stream);
 }
 
 int dion_amd_syrk(const void* A, long long a_stride, int lda, void* C, long long c_stride, int ldc, int batch, int m,

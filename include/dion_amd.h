@@ -70,6 +70,24 @@ int dion_amd_newton_schulz(const void* G, int g_dtype, long long g_stride, int l
                            int compute_dtype, int faithful,
                            void* workspace, size_t workspace_bytes, void* stream);
 
+/* dion_amd_newton_schulz without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference: it is for callers that cannot allocate device memory -- code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The working
+ * matrices live in an array of DION_AMD_STATIC_SCRATCH_BYTES that is part of the library's
+ * device image (every GPU the library runs on holds one copy until the process ends).
+ * Same arguments and result as dion_amd_newton_schulz.  One matrix's working set
+ * (dion_amd_ns_workspace_bytes(1, m, n, compute_dtype)) must fit the array, else
+ * DION_AMD_ERR_LIMIT and nothing is launched; a batch goes through it in chunks.  Every call
+ * on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream are ordered and safe. */
+#define DION_AMD_STATIC_SCRATCH_BYTES (32u << 20)
+size_t dion_amd_static_scratch_bytes(void);
+int dion_amd_newton_schulz_static(const void* G, int g_dtype, long long g_stride, int ldg,
+                                  void* out, long long out_stride, int ldo,
+                                  int batch, int m, int n,
+                                  const float* coeffs, int steps, float eps,
+                                  int compute_dtype, int faithful, void* stream);
+
 /* Replaces ns_line_1 (reference dion/newton_schulz_triton.py:134-170):
  * C_b (m x m) = A_b A_b^T for A_b (m x k); upper tiles computed, mirrored store. */
 int dion_amd_syrk(const void* A, long long a_stride, int lda,
