@@ -174,7 +174,7 @@ class Workspace:
 
 
 PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
-              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt")
+              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt", "dion_ef_upd")
 
 
 def profile_read():

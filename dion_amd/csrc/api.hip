@@ -771,6 +771,21 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
         if (rc) return rc;
       }
     }  // power iterations
+    // ---- error feedback, column normalisation and weight update (reference dion/dion.py:851-872)
+    static const bool no_fused = getenv("DION_AMD_NO_FUSED") != nullptr;
+    if (faithful && !no_fused && da_dion_ef_update_applicable(mp, np, r, m_dtype)) {
+      // Q_new first (it only needs R), then both rank-r updates in one pass over M and X
+      {
+        DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);
+        rc = da_colnorm(R, Qn, m_dtype, tq, q_dtype, np, r, rank, eps, cb, reinterpret_cast<double*>(orth_ws), s);
+        if (rc) return rc;
+      }
+      DaProfScope prof(DA_PROF_DION_EFUPD, 4.0 * (double)mp * np * r * cb, s);
+      rc = da_dion_ef_update(P, R, Qn, tm, tx, cb, mp, np, r, n, transposed ? 1 : 0, x_dtype, ef_alpha, decay,
+                             scaled_lr, s);
+      if (rc) return rc;
+      continue;
+    }
     // ---- error feedback  M <- M - (1 - mu) P R^T  (or R P^T)   (reference dion/dion.py:851-853)
     g = GemmDesc{};
     g.batch = cb; g.faithful = faithful;

@@ -31,3 +31,13 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 size_t da_orth_workspace_bytes(int batch, int rows, int r);
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
                       void* ws, int* info, hipStream_t s);
+
+// Error feedback and weight update in one pass (dion_fused.hip), bf16 factors:
+//   M[b] <- M[b] + ef_alpha P[b] R[b]^T,  X[b] <- decay X[b] - scaled_lr P[b] Qn[b]^T   (R P^T, Qn P^T when `transposed`)
+// with every rounding of the reference's separate tensor ops.  P: batch x mp x r, R / Qn: batch x np x r (contiguous);
+// tabM / tabX: the matrices (row pitch ldo; momentum bf16, weights x_dtype), at most DA_MAX_PTRS of them.
+// Applicable when mp and np are multiples of 128 and r of 64.
+bool da_dion_ef_update_applicable(int mp, int np, int r, int m_dtype);
+int da_dion_ef_update(const void* P, const void* R, const void* Qn, const DaPtrTable& tabM, const DaPtrTable& tabX, int batch,
+                      int mp, int np, int r, int ldo, int transposed, int x_dtype, float ef_alpha, float decay,
+                      float scaled_lr, hipStream_t s);

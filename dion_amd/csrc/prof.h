@@ -18,7 +18,8 @@ enum DaProfKind {
   DA_PROF_DION_ORTH = 11, // orthonormalisation of P (all of its launches)
   DA_PROF_DION_ELEM = 12, // B = M + G, column norms, guards
   DA_PROF_SCALAR_OPT = 13,// fused Lion / AdamW pass over non-matrix parameters
-  DA_PROF_KINDS = 14
+  DA_PROF_DION_EFUPD = 14,// error feedback and weight update in one pass
+  DA_PROF_KINDS = 15
 };
 
 struct DaProfScope {

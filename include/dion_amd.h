@@ -291,7 +291,8 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
 #define DION_AMD_PROF_DION_ORTH 11
 #define DION_AMD_PROF_DION_ELEM 12
 #define DION_AMD_PROF_SCALAR_OPT 13
-#define DION_AMD_PROF_KINDS 14
+#define DION_AMD_PROF_DION_EFUPD 14
+#define DION_AMD_PROF_KINDS 15
 int dion_amd_profile_enable(int on);
 int dion_amd_profile_reset(void);
 /* Waits for the recorded events of `kind`; returns launch count, summed milliseconds and
