@@ -34,7 +34,8 @@ template <> __device__ __forceinline__ float rsqrt_seed<float>(float p) { return
 template <typename T>
 __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G, T* __restrict__ Lmat,
                                                         T* __restrict__ Wmat, long long sG, int r, int o, int nb,
-                                                        int below, int* __restrict__ info) {
+                                                        int below, int* __restrict__ info, const int* gate,
+                                                        int gate_want) {
   typedef typename Mfma<T>::acc_t acc_t;
   __shared__ T dinv4[4][4];            // inverse of the current diagonal 4 x 4 factor (lower)
   __shared__ T lcol[NB][4];            // rows > 4cb+3: L[i][4cb .. 4cb+3]
@@ -43,6 +44,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   extern __shared__ __attribute__((aligned(16))) unsigned char opnd_raw[];   // two k-major 64 x 64 operand tiles
   T* const opnd = reinterpret_cast<T*>(opnd_raw);
   const int b = blockIdx.y, tid = threadIdx.x;
+  if (gate && (gate[b] != 0) != (gate_want != 0)) return;
   const int bi = tid >> 4, bj = tid & 15;
   const T* g = G + (long long)b * sG + (long long)o * r + o;
   T a[4][4], y[4][4];
@@ -266,7 +268,8 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
 }
 
 template <typename T>
-int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, int* info, int batch, hipStream_t s) {
+int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, int* info, int batch, DaGate gate,
+              hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   const int rest = r - o - nb;
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
@@ -285,13 +288,18 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  hipLaunchKernelGGL(chol_step_kernel<T>, dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb, below, info);
+  hipLaunchKernelGGL(chol_step_kernel<T>, dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb, below, info,
+                     gate.flags, gate.want);
   return da_launch_status();
 }
 
 }  // namespace
 
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, hipStream_t s) {
-  return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, s);
+                 int batch, DaGate gate, hipStream_t s) {
+  return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, s);
+}
+int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
+                     int batch, DaGate gate, hipStream_t s) {
+  return chol_step<float>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, s);
 }

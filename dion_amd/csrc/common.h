@@ -58,6 +58,19 @@ static inline int da_launch_status() {
   return e == hipSuccess ? DA_OK : (int)e;
 }
 
+// Compute units of the current device (persistent kernels size their grids with it).
+static inline int da_cu_count() {
+  static int cache[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cache[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cache[dev] = n;
+  }
+  return cache[dev];
+}
+
 // ---- GEMM descriptor shared by the bf16 / f32 / f64 kernels -------------------------
 // C[b] (M x N) = epilogue( sum_k Aop[b](i,k) * Bop[b](j,k) ).
 // An operand is either "k-contiguous" (stored rows x K, ld = row pitch) or
@@ -84,6 +97,10 @@ struct GemmDesc {
   int faithful;       // 1: reproduce every bf16 rounding of the op-by-op reference
   float s0, s1;       // epilogue scalars
   int c_dtype;        // dtype of C / E for the f32 and f64 kernels' mixed outputs
+  // Optional per-matrix switch (bf16 kernel): with `gate` set, matrix b is computed only if
+  // (gate[b] != 0) == (gate_want != 0); the workgroups of the other matrices return at once.
+  const int* gate;
+  int gate_want;
 };
 
 // Epilogues.  With `faithful` set the rounding points of the reference's separate

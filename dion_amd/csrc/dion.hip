@@ -373,63 +373,197 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 }
 
 // ---------------------------------------------------------------------------------------
-// CholeskyQR2 in fp64
+// Orthonormalisation: CholeskyQR in fp32 with a measured defect, CholeskyQR in fp64 where that is not enough,
+// closed-form polishing pass
 // ---------------------------------------------------------------------------------------
-size_t da_orth_workspace_bytes(int batch, int rows, int r) {
-  size_t per = (size_t)rows * r * 8       // P in fp64, orthonormalised in place (first pass)
-               + 3 * (size_t)r * r * 8    // G, L, W (fp64; the polishing passes keep their fp32 G and V there)
-               + (size_t)rows * r * 4     // the fp64 pass's result in fp32 (input of the polishing pass)
-               + (size_t)rows * r * 2;    // ... and in bf16 (operand of its correction product)
-  return per * batch + 256;
-}
+namespace {
+
+// Slices of K of the Gram products of `batch` rows x r matrices (1: unsliced).
+int gram_slices(int batch, int rows, int r) { return da_auto_split(da_gram_blocks(r, batch), rows); }
+
+size_t orth_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Workspace of one call, carved in this order.
+struct OrthWs {
+  double* P0;      // rows x r per matrix, fp64: the fp64 pass works in place here
+  float* Pf;       // ... fp32: the fp32 pass works in place here; later the fp64 pass's result for its polishing pass
+  bf16_t* Ph;      // ... bf16 copy of Pf (operand of the correction product)
+  double* G;       // r x r per matrix (fp64, or fp32 in the same place): Gram matrix
+  double* L;       // Cholesky factor; later the correction factor of the polishing pass
+  double* W;       // inverse-factor blocks
+  double* part;    // K-slice outputs of a sliced Gram product
+  float* rowdef;   // r per matrix: squared defect of each row of the polishing pass's Gram matrix
+  int* need;       // per matrix: 1 = the fp32 pass was not enough, the fp64 pass runs
+  int* info32;     // per matrix: status of the fp32 factorisation
+  int* bad;        // r per matrix: 1 = the column is not usable (noise-level pivot), it is zeroed
+  size_t bytes;
+  OrthWs(void* ws, int batch, int rows, int r) {
+    const size_t pr = (size_t)rows * r * batch, rr = (size_t)r * r * batch;
+    const int sp = gram_slices(batch, rows, r);
+    char* p = static_cast<char*>(ws);
+    auto take = [&](size_t n) { char* q = p; p += orth_align(n); return q; };
+    P0 = reinterpret_cast<double*>(take(pr * 8));
+    Pf = reinterpret_cast<float*>(take(pr * 4));
+    Ph = reinterpret_cast<bf16_t*>(take(pr * 2));
+    G = reinterpret_cast<double*>(take(rr * 8));
+    L = reinterpret_cast<double*>(take(rr * 8));
+    W = reinterpret_cast<double*>(take(rr * 8));
+    // K-slice outputs: `sp` slices of the fp64 / fp32 Gram kernels, or up to four fp32 slabs of the bf16 one
+    part = reinterpret_cast<double*>(take(rr * 8 * (sp > 2 ? sp : 2)));
+    rowdef = reinterpret_cast<float*>(take((size_t)r * batch * 4));
+    need = reinterpret_cast<int*>(take((size_t)batch * 4));
+    info32 = reinterpret_cast<int*>(take((size_t)batch * 4));
+    bad = reinterpret_cast<int*>(take((size_t)r * batch * 4));
+    bytes = (size_t)(p - static_cast<char*>(ws));
+  }
+};
+
+}  // namespace
+
+size_t da_orth_workspace_bytes(int batch, int rows, int r) { return OrthWs(nullptr, batch, rows, r).bytes + 256; }
 
 namespace {
 
-// G[b][i][i] = 1 for r_live <= i < r: the Gram matrix of a P whose last r - r_live columns are zero becomes
-// block diagonal with an identity block, and the factorisation leaves those columns of P zero.
-__global__ void pad_diag_kernel(double* G, long long rr, int r, int r_live) {
-  const int i = r_live + threadIdx.x;
-  if (i < r) G[blockIdx.x * rr + (long long)i * r + i] = 1.0;
+__device__ __forceinline__ bool orth_gate_open(const int* flags, int want, int b) {
+  return !flags || (flags[b] != 0) == (want != 0);
 }
 
-// One blocked CholeskyQR pass in fp64, in place:  P <- P R^-1  with  P^T P = R^T R.
-int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows, int r, int r_live, bool g_cleared,
-                int* info, hipStream_t s) {
-  const int NB = DA_CHOL_NB;
-  const int nblk = (r + NB - 1) / NB;
+// Row i of G[b] = sum of the K slices in slice order (sp > 1; else G already holds the product); rows
+// r_live .. r-1 get a one on the diagonal: the Gram matrix of a P whose last r - r_live columns are zero becomes
+// block diagonal with an identity block, and the factorisation leaves those columns of P zero.
+// rowdef (if given): sum_j (G[i][j] - delta_ij)^2, the row's share of the squared defect ||G - I||_F^2.
+template <typename T>
+__global__ __launch_bounds__(256) void gram_finish_kernel(const T* __restrict__ part, int sp, long long slice_stride,
+                                                          T* __restrict__ G, long long rr, int r, int r_live,
+                                                          float* __restrict__ rowdef, const int* gate, int want) {
+  const int b = blockIdx.y, i = blockIdx.x;
+  if (!orth_gate_open(gate, want, b)) return;
+  T* g = G + b * rr + (long long)i * r;
+  float acc = 0.f;
+  for (int j = threadIdx.x; j < r; j += 256) {
+    T v;
+    if (sp > 1) {
+      v = T(0);
+      for (int q = 0; q < sp; ++q) v += part[q * slice_stride + b * rr + (long long)i * r + j];
+    } else {
+      v = g[j];
+    }
+    if (i >= r_live && j == i) v = T(1);
+    if (sp > 1 || (i >= r_live && j == i)) g[j] = v;
+    const float e = (float)v - (i == j ? 1.f : 0.f);
+    acc += e * e;
+  }
+  if (rowdef) {
+    __shared__ float red[256];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) rowdef[(long long)b * r + i] = red[0];
+  }
+}
+
+// After the fp32 pass: need[b] = the fp32 factorisation failed or left a defect ||P^T P - I||_F above `tol`
+// (then the closed-form polishing pass could not bring it to round-off, and the fp64 pass takes the matrix over).
+__global__ __launch_bounds__(64) void decide_fast_kernel(const float* __restrict__ rowdef, const int* __restrict__ info32,
+                                                         int* __restrict__ need, int r, float tol2) {
+  const int b = blockIdx.x;
+  if (threadIdx.x != 0) return;
+  float s = 0.f;
+  for (int i = 0; i < r; ++i) s += rowdef[(long long)b * r + i];   // fixed order
+  need[b] = (info32[b] != 0 || !(s <= tol2)) ? 1 : 0;
+}
+
+// After the fp64 pass: a column whose row of P^T P - I is not small (or not finite) came from a pivot at round-off
+// level -- a numerically rank-deficient P; it is dropped (zeroed) and reported like a failed pivot.
+__global__ __launch_bounds__(256) void decide_cols_kernel(const float* __restrict__ rowdef, int* __restrict__ bad,
+                                                          int* __restrict__ info, int r, const int* gate, int want) {
+  const int b = blockIdx.x;
+  if (!orth_gate_open(gate, want, b)) return;
+  __shared__ int first;
+  if (threadIdx.x == 0) first = 0x7fffffff;
+  __syncthreads();
+  for (int j = threadIdx.x; j < r; j += 256) {
+    const float d = rowdef[(long long)b * r + j];
+    const int is_bad = !(d <= 0.25f) ? 1 : 0;
+    bad[(long long)b * r + j] = is_bad;
+    if (is_bad) atomicMin(&first, j);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && first != 0x7fffffff && info[b] == 0) info[b] = first + 1;
+}
+
+// out[:, j] = 0 for the dropped columns.
+template <typename T>
+__global__ __launch_bounds__(256) void zero_cols_kernel(T* __restrict__ out, const int* __restrict__ bad, int rows, int r,
+                                                        const int* __restrict__ info, const int* gate, int want) {
+  const int b = blockIdx.y;
+  if (!orth_gate_open(gate, want, b) || info[b] == 0) return;
+  const int* bd = bad + (long long)b * r;
+  T* o = out + (long long)b * rows * r;
+  for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < (long long)rows * r; e += (long long)gridDim.x * 256)
+    if (bd[e % r]) st_from_float<T>(o + e, 0.f);
+}
+
+inline int gemm_real(const Gemm64Desc& d, hipStream_t s) { return da_gemm_f64(d, s); }
+inline int gemm_real(const Gemm32Desc& d, hipStream_t s) { return da_gemm_f32s(d, s); }
+inline int chol_step_real(const double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info, int batch,
+                          DaGate g, hipStream_t s) { return da_chol_step(G, L, W, sG, r, o, nb, info, batch, g, s); }
+inline int chol_step_real(const float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info, int batch,
+                          DaGate g, hipStream_t s) { return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, g, s); }
+
+// G = P^T P (K-sliced if that fills the GPU; the slices are added in a fixed order), padded diagonal, and
+// optionally the rows' squared defects.
+template <typename T>
+int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, float* rowdef, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
-  Gemm64Desc g{};
+  const int sp = gram_slices(batch, rows, r);
+  RealGemmDesc<T> g{};
   g.batch = batch;
-  // G = P0^T P0
-  g.A = P0; g.B = P0; g.C = G; g.E = nullptr;
+  g.A = P; g.B = P; g.C = sp > 1 ? part : G; g.E = nullptr;
   g.sA = pr; g.sB = pr; g.sC = rr;
   g.lda = r; g.ldb = r; g.ldc = r;
   g.M = r; g.N = r; g.K = rows;
   g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
-  g.split_k = -1;   // few output tiles, long K: the launcher slices K until the GPU is full
-  g.c_is_zero = g_cleared ? 1 : 0;
-  int rc = da_gemm_f64(g, s);
+  g.split_k = sp; g.split_stride = rr * batch;
+  g.gate = gate.flags; g.gate_want = gate.want;
+  int rc = gemm_real(g, s);
   if (rc) return rc;
-  if (r_live < r) {
-    hipLaunchKernelGGL(pad_diag_kernel, dim3((unsigned)batch), dim3(64), 0, s, G, rr, r, r_live);
+  if (sp > 1 || r_live < r || rowdef) {
+    hipLaunchKernelGGL(gram_finish_kernel<T>, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, part, sp, rr * batch,
+                       G, rr, r, r_live, rowdef, gate.flags, gate.want);
     rc = da_launch_status();
-    if (rc) return rc;
   }
+  return rc;
+}
+
+// One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
+template <typename T>
+int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, int r_live, int* info, DaGate gate,
+                hipStream_t s) {
+  const int NB = DA_CHOL_NB;
+  const int nblk = (r + NB - 1) / NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  int rc = gram<T>(P0, G, part, batch, rows, r, r_live, nullptr, gate, s);
+  if (rc) return rc;
   // blocked lower Cholesky G = L L^T (right-looking), building W alongside
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-    rc = da_chol_step(G, L, W, rr, r, o, nb, info, batch, s);
+    rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s);
     if (rc) return rc;
     if (rest <= 0) break;
     // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
-    Gemm64Desc u{};
+    RealGemmDesc<T> u{};
     u.batch = batch;
     u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
     u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
     u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
     u.E = u.C; u.sE = rr; u.lde = r;
     u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
-    rc = da_gemm_f64(u, s);
+    u.gate = gate.flags; u.gate_want = gate.want;
+    rc = gemm_real(u, s);
     if (rc) return rc;
   }
   // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
@@ -438,14 +572,15 @@ int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows
   // those rows before it stores)
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB;
-    Gemm64Desc a{};
+    RealGemmDesc<T> a{};
     a.batch = batch;
     a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
     a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
     a.C = P0 + o; a.sC = pr; a.ldc = r;
     a.E = nullptr;
     a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
-    rc = da_gemm_f64(a, s);
+    a.gate = gate.flags; a.gate_want = gate.want;
+    rc = gemm_real(a, s);
     if (rc) return rc;
   }
   return DA_OK;
@@ -455,50 +590,51 @@ int cholqr_pass(double* P0, double* G, double* L, double* W, int batch, int rows
 // upper triangle and half of the diagonal: the Cholesky factor of G = I + E is R = I + up(E) + O(E^2), so
 // P V = P R^-1 + O(E^2).
 __global__ __launch_bounds__(256) void polish_factor_kernel(const float* __restrict__ G, float* __restrict__ V,
-                                                            long long rr, int r) {
+                                                            long long rr, int r, const int* __restrict__ bad,
+                                                            const int* gate, int want) {
   const long long b = blockIdx.y;
+  if (!orth_gate_open(gate, want, (int)b)) return;
   const int i = blockIdx.x;
   const float* g = G + b * rr + (long long)i * r;
   float* v = V + b * rr + (long long)i * r;
+  const int* bd = bad ? bad + b * r : nullptr;
+  const bool row_bad = bd && bd[i];
   for (int j = threadIdx.x; j < r; j += 256) {
     const float x = g[j];
-    v[j] = i < j ? -x : (i == j ? 1.5f - 0.5f * x : 0.f);
+    const bool drop = row_bad || (bd && bd[j]);   // dropped columns neither receive nor give a correction
+    v[j] = drop ? (i == j ? 1.f : 0.f) : (i < j ? -x : (i == j ? 1.5f - 0.5f * x : 0.f));
   }
 }
 
 // U = up(G - I) in bf16 (see polish_factor_kernel): the factor of the correction product P U, which only has
-// to be known to the relative accuracy of bf16 because it is itself of the size of the defect.
+// to be known to the relative accuracy of bf16 because it is itself of the size of the defect.  Rows and columns
+// of dropped columns (`bad`, may be null) are left out of the correction.
 __global__ __launch_bounds__(256) void polish_correction_kernel(const float* __restrict__ G, bf16_t* __restrict__ U,
-                                                                long long rr, int r) {
+                                                                long long rr, int r, const int* __restrict__ bad,
+                                                                const int* gate, int want) {
   const long long b = blockIdx.y;
+  if (!orth_gate_open(gate, want, (int)b)) return;
   const int i = blockIdx.x;
   const float* g = G + b * rr + (long long)i * r;
   bf16_t* u = U + b * rr + (long long)i * r;
+  const int* bd = bad ? bad + b * r : nullptr;
+  const bool row_bad = bd && bd[i];
   for (int j = threadIdx.x; j < r; j += 256) {
     const float x = g[j];
-    u[j] = f2bf(i < j ? x : (i == j ? 0.5f * (x - 1.f) : 0.f));
+    const bool drop = row_bad || (bd && bd[j]);
+    u[j] = f2bf(drop ? 0.f : (i < j ? x : (i == j ? 0.5f * (x - 1.f) : 0.f)));
   }
 }
 
-// The last polishing pass of an iterate that exists in fp32 and in bf16:  out <- in - in_bf16 U(in^T in).
-// The Gram product is fp32 as in polish_pass; the correction product runs on the bf16 matrix cores (its
+// The last polishing pass of an iterate that exists in fp32 and in bf16:  out <- in - in_bf16 U(in^T in), with
+// U built from the Gram matrix G (already computed).  The correction product runs on the bf16 matrix cores (its
 // relative error 2^-8 times the defect E of `in` adds 4e-3 E to the result, next to the pass's own O(E^2)).
-int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_dtype, float* G, bf16_t* U, int batch,
-                     int rows, int r, bool g_cleared, hipStream_t s) {
+int correction_bf16(const float* in, const bf16_t* in_low, void* out, int out_dtype, const float* G, bf16_t* U,
+                    const int* bad, int batch, int rows, int r, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
-  Gemm32Desc g{};
-  g.batch = batch;
-  g.A = in; g.B = in; g.C = G;
-  g.sA = pr; g.sB = pr; g.sC = rr;
-  g.lda = r; g.ldb = r; g.ldc = r;
-  g.M = r; g.N = r; g.K = rows;
-  g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
-  g.split_k = -1;
-  g.c_is_zero = g_cleared ? 1 : 0;
-  int rc = da_gemm_f32s(g, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(polish_correction_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, U, rr, r);
-  rc = da_launch_status();
+  hipLaunchKernelGGL(polish_correction_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, U, rr, r, bad,
+                     gate.flags, gate.want);
+  int rc = da_launch_status();
   if (rc) return rc;
   GemmDesc c{};
   c.batch = batch;
@@ -510,28 +646,18 @@ int polish_pass_bf16(const float* in, const bf16_t* in_low, void* out, int out_d
   c.sE = pr; c.lde = r;
   c.M = rows; c.N = r; c.K = r;
   c.epilogue = DA_EPI_AXPBY; c.s0 = 1.f; c.s1 = -1.f; c.faithful = 0;
+  c.gate = gate.flags; c.gate_want = gate.want;
   return da_gemm_bf16(c, s);
 }
 
-// One polishing pass in fp32:  out <- in V(in^T in).  `in` (fp32) and `out` (fp32, or the caller's dtype for
-// the last pass) are different buffers; one Gram product, one elementwise pass over r x r, one product with
-// the triangular V -- no serial chain.
-int polish_pass(const float* in, void* out, int out_store, float* G, float* V, int batch, int rows, int r,
-                bool g_cleared, hipStream_t s) {
+// The same in fp32 throughout:  out <- in V(G)  with the triangular V (ranks that are not multiples of 8, and
+// intermediate passes).  `in` and `out` are different buffers.
+int correction_f32(const float* in, void* out, int out_store, const float* G, float* V, const int* bad, int batch,
+                   int rows, int r, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
-  Gemm32Desc g{};
-  g.batch = batch;
-  g.A = in; g.B = in; g.C = G;
-  g.sA = pr; g.sB = pr; g.sC = rr;
-  g.lda = r; g.ldb = r; g.ldc = r;
-  g.M = r; g.N = r; g.K = rows;
-  g.a_kstrided = 1; g.b_kstrided = 1; g.symmetric = 1; g.alpha = 1.0; g.beta = 0.0;
-  g.split_k = -1;
-  g.c_is_zero = g_cleared ? 1 : 0;
-  int rc = da_gemm_f32s(g, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(polish_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, V, rr, r);
-  rc = da_launch_status();
+  hipLaunchKernelGGL(polish_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, V, rr, r, bad,
+                     gate.flags, gate.want);
+  const int rc = da_launch_status();
   if (rc) return rc;
   // out = in V: V is upper triangular, so column tile j only sums k < 64 (j + 1)
   Gemm32Desc a{};
@@ -540,57 +666,304 @@ int polish_pass(const float* in, void* out, int out_store, float* G, float* V, i
   a.B = V; a.sB = rr; a.ldb = r; a.b_kstrided = 1;
   a.C = static_cast<float*>(out); a.c_store = out_store; a.sC = pr; a.ldc = r;
   a.M = rows; a.N = r; a.K = r; a.alpha = 1.0; a.beta = 0.0; a.k_tri = 1;
+  a.gate = gate.flags; a.gate_want = gate.want;
   return da_gemm_f32s(a, s);
 }
 
+int zero_cols(void* out, int dtype, const int* bad, const int* info, int batch, int rows, int r, DaGate gate,
+              hipStream_t s) {
+  const long long n = (long long)rows * r;
+  long long blocks = (n + 255) / 256;
+  if (blocks > 1024) blocks = 1024;
+  const dim3 grid((unsigned)blocks, (unsigned)batch);
+  if (dtype == DA_BF16)
+    hipLaunchKernelGGL(zero_cols_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(out), bad, rows, r, info,
+                       gate.flags, gate.want);
+  else
+    hipLaunchKernelGGL(zero_cols_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(out), bad, rows, r, info,
+                       gate.flags, gate.want);
+  return da_launch_status();
+}
+
+// ---- the fp32 pass on the bf16 matrix cores (bf16 P: its products with bf16 factors are exact in fp32) ----
+
+// Row i of G[b] = sum of `n_hh` slabs + sum of `n_hl` slabs and their transposes (the cross terms h^T l + l^T h of
+// a matrix held as h + l), in slab order; padded diagonal and row defects as in gram_finish_kernel.
+__global__ __launch_bounds__(256) void gram16_finish_kernel(const float* __restrict__ part, int n_hh, int n_hl,
+                                                            long long slab, float* __restrict__ G, long long rr, int r,
+                                                            int r_live, float* __restrict__ rowdef) {
+  const int b = blockIdx.y, i = blockIdx.x;
+  float* g = G + b * rr + (long long)i * r;
+  float acc = 0.f;
+  for (int j = threadIdx.x; j < r; j += 256) {
+    float v = 0.f;
+    for (int q = 0; q < n_hh; ++q) v += part[q * slab + b * rr + (long long)i * r + j];
+    for (int q = n_hh; q < n_hh + n_hl; ++q)
+      v += part[q * slab + b * rr + (long long)i * r + j] + part[q * slab + b * rr + (long long)j * r + i];
+    if (i >= r_live && j == i) v = 1.f;
+    g[j] = v;
+    const float e = v - (i == j ? 1.f : 0.f);
+    acc += e * e;
+  }
+  if (rowdef) {
+    __shared__ float red[256];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) rowdef[(long long)b * r + i] = red[0];
+  }
+}
+
+// G = H^T H (+ H^T Lo + Lo^T H when Lo is given), fp32, from bf16 operands: up to four products (K slices x
+// {H^T H, H^T Lo}) run as the groups of one launch and leave fp32 slabs that the finish kernel adds in order.
+int gram16(const bf16_t* H, const bf16_t* Lo, float* G, float* part, int batch, int rows, int r, int r_live,
+           float* rowdef, hipStream_t s) {
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  const int kinds = Lo ? 2 : 1;
+  const long long tiles = (long long)batch * ((r + 255) / 256) * ((r + 255) / 256);
+  int nsl = (int)((256 + tiles - 1) / tiles);
+  if (nsl > DA_MAX_GROUPS / kinds) nsl = DA_MAX_GROUPS / kinds;
+  if (nsl > rows / 256) nsl = rows / 256 > 0 ? rows / 256 : 1;
+  const int ks = ((rows + nsl - 1) / nsl + 63) / 64 * 64;   // rows per slice, a multiple of the stage depth
+  nsl = (rows + ks - 1) / ks;
+  GemmDesc g[DA_MAX_GROUPS];
+  int n = 0;
+  for (int kind = 0; kind < kinds; ++kind)
+    for (int q = 0; q < nsl; ++q) {
+      const int k0 = q * ks, kn = rows - k0 < ks ? rows - k0 : ks;
+      GemmDesc& d = g[n];
+      d = GemmDesc{};
+      d.batch = batch;
+      d.A = H + (long long)k0 * r; d.sA = pr; d.lda = r; d.a_kstrided = 1;
+      d.B = (kind == 0 ? H : Lo) + (long long)k0 * r; d.sB = pr; d.ldb = r; d.b_kstrided = 1;
+      d.C = part + (long long)n * rr * batch; d.sC = rr; d.ldc = r; d.c_dtype = DA_F32;
+      d.M = r; d.N = r; d.K = kn;
+      d.epilogue = DA_EPI_STORE; d.s1 = 1.f; d.faithful = 0;
+      ++n;
+    }
+  int rc = da_gemm_bf16_grouped(g, n, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(gram16_finish_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, part, nsl, Lo ? nsl : 0,
+                     rr * batch, G, rr, r, r_live, rowdef);
+  return da_launch_status();
+}
+
+// T = identity (r x r per matrix)
+__global__ __launch_bounds__(256) void eye_kernel(float* __restrict__ T, long long rr, int r) {
+  const long long b = blockIdx.y;
+  const int i = blockIdx.x;
+  for (int j = threadIdx.x; j < r; j += 256) T[b * rr + (long long)i * r + j] = i == j ? 1.f : 0.f;
+}
+
+// Tcat[k][0 .. r) = bf16(T[k][:]), Tcat[k][r .. 2r) = bf16(T[k][:] - that): T to 16 bits as two bf16 factors
+__global__ __launch_bounds__(256) void split_factor_kernel(const float* __restrict__ T, bf16_t* __restrict__ Tcat,
+                                                           long long rr, int r) {
+  const long long b = blockIdx.y;
+  const int k = blockIdx.x;
+  const float* t = T + b * rr + (long long)k * r;
+  bf16_t* o = Tcat + b * 2 * rr + (long long)k * 2 * r;
+  for (int j = threadIdx.x; j < r; j += 256) {
+    const float v = t[j];
+    const bf16_t h = f2bf(v);
+    o[j] = h;
+    o[r + j] = f2bf(v - bf2f(h));
+  }
+}
+
+// C2 (rows x 2r, fp32) holds P T_hi | P T_lo: their sum as h + l (two bf16 matrices, 16 bits together)
+__global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict__ C2, bf16_t* __restrict__ H,
+                                                        bf16_t* __restrict__ Lo, long long pr, int r) {
+  const long long b = blockIdx.y;
+  const float* c = C2 + b * 2 * pr;
+  for (long long e = ((long long)blockIdx.x * 256 + threadIdx.x) * 4; e < pr; e += (long long)gridDim.x * 1024) {
+    const long long row = e / r;
+    const int col = (int)(e - row * r);   // r is a multiple of 8: the four elements share the row
+    const float4 a = *reinterpret_cast<const float4*>(c + row * 2 * r + col);
+    const float4 d = *reinterpret_cast<const float4*>(c + row * 2 * r + r + col);
+    const float v[4] = {a.x + d.x, a.y + d.y, a.z + d.z, a.w + d.w};
+    bf16_t h[4], l[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      h[q] = f2bf(v[q]);
+      l[q] = f2bf(v[q] - bf2f(h[q]));
+    }
+    *reinterpret_cast<uint2*>(H + b * pr + e) = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+    *reinterpret_cast<uint2*>(Lo + b * pr + e) = make_uint2((uint32_t)l[0] | ((uint32_t)l[1] << 16), (uint32_t)l[2] | ((uint32_t)l[3] << 16));
+  }
+}
+
+// The fp32 CholeskyQR pass of a bf16 P with its large products on the bf16 matrix cores:
+//   G = P^T P (exact products, fp32 sums), blocked Cholesky G = R^T R in fp32, T = R^-1 explicitly (the block
+//   recurrence of the triangular solve applied to the identity), P1 = P T with T as two bf16 factors (T to 16
+//   bits: P1 stays an exact triangular recombination of P's columns, so its thin-QR factor is P's), kept as
+//   h + l (bf16 each); then G2 = P1^T P1 = h^T h + h^T l + l^T h for the defect and the polishing pass.
+int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, int r_live, hipStream_t s) {
+  const int NB = DA_CHOL_NB;
+  const int nblk = (r + NB - 1) / NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  const DaGate all{nullptr, 0};
+  float* G = reinterpret_cast<float*>(w.G);
+  float* L = reinterpret_cast<float*>(w.L);
+  float* W = reinterpret_cast<float*>(w.W);
+  float* T = W + rr * batch;                          // second half of W's room
+  bf16_t* Tcat = reinterpret_cast<bf16_t*>(w.L);      // over the factor L, which is dead once W is complete
+  float* C2 = reinterpret_cast<float*>(w.P0);         // rows x 2r fp32 = the room of the fp64 copy
+  bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
+  float* part = reinterpret_cast<float*>(w.part);
+  int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, s);
+  if (rc) return rc;
+  for (int j = 0; j < nblk; ++j) {
+    const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
+    rc = da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s);
+    if (rc) return rc;
+    if (rest <= 0) break;
+    Gemm32Desc u{};
+    u.batch = batch;
+    u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
+    u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+    u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
+    u.E = u.C; u.sE = rr; u.lde = r;
+    u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
+    rc = da_gemm_f32s(u, s);
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(eye_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, rr, r);
+  rc = da_launch_status();
+  if (rc) return rc;
+  for (int j = 0; j < nblk; ++j) {
+    const int o = j * NB, nb = r - o < NB ? r - o : NB;
+    Gemm32Desc a{};
+    a.batch = batch;
+    a.A = T; a.sA = rr; a.lda = r; a.a_kstrided = 0;
+    a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
+    a.C = T + o; a.sC = rr; a.ldc = r;
+    // rows below block j of T are zero in these columns (T is upper triangular): only rows < o + nb are needed
+    a.M = o + nb; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
+    rc = da_gemm_f32s(a, s);
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(split_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, Tcat, rr, r);
+  rc = da_launch_status();
+  if (rc) return rc;
+  GemmDesc c{};
+  c.batch = batch;
+  c.A = P; c.sA = pr; c.lda = r; c.a_kstrided = 0;
+  c.B = Tcat; c.sB = 2 * rr; c.ldb = 2 * r; c.b_kstrided = 1;
+  c.C = C2; c.sC = 2 * pr; c.ldc = 2 * r; c.c_dtype = DA_F32;
+  c.M = rows; c.N = 2 * r; c.K = r;
+  c.epilogue = DA_EPI_STORE; c.s1 = 1.f; c.faithful = 0;
+  rc = da_gemm_bf16(c, s);
+  if (rc) return rc;
+  long long blocks = (pr / 4 + 255) / 256;
+  const long long cap = 16384 / batch > 0 ? 16384 / batch : 1;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)(blocks < 1 ? 1 : blocks), (unsigned)batch), dim3(256), 0, s, C2,
+                     w.Ph, Lo, pr, r);
+  rc = da_launch_status();
+  if (rc) return rc;
+  return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, s);
+}
+
+// Defect ||P^T P - I||_F up to which the closed-form polishing pass is trusted after the fp32 pass: it leaves
+// about 3 E^2, i.e. 1e-5.
+constexpr float FAST_TOL = 2e-3f;
+
 }  // namespace
 
-// The first pass is a blocked CholeskyQR in fp64: the Gram matrix squares P's condition number (up to
-// 4e12 on the optimizer's inputs).  Its result is orthonormal to E = eps64 * cond(P)^2 <= 1e-4, and for
-// such a matrix the second CholeskyQR pass has a closed form to O(E^2) <= 1e-8 -- below fp32 round-off,
-// which is all the output dtype (fp32 or bf16) can hold: R^-1 = I - up(P^T P - I).  So the later passes
-// are two fp32 products and no factorisation at all; the last one stores the output dtype.
+// Thin-QR Q factor of each P (same column space, orthonormal columns, up to column signs).
+//   passes == 2 (the optimizer's case): a blocked CholeskyQR pass in fp32, the Gram matrix of its result (which
+//   measures the defect E = ||P^T P - I||_F it left: eps32 * cond(P)^2) and, for a small defect, the closed form of
+//   a second CholeskyQR pass: R^-1 = I - up(P^T P - I) + O(E^2).  Matrices for which the fp32 pass failed or left
+//   too large a defect are flagged on the device, and the same sequence in fp64 then runs for those alone (every
+//   launch of it returns at once for the others; no host synchronisation): the Gram matrix squares P's condition
+//   number, up to 4e12 on the optimizer's full-rank inputs.  After the fp64 pass, columns whose row of
+//   P^T P - I is not small came from pivots at round-off level (a numerically rank-deficient P): they are zeroed
+//   and reported in `info` like a non-positive pivot.
+//   passes == 1: the fp64 pass alone.  passes == 3: fp64 pass and two polishing passes.
 // Columns r_live .. r-1 of P, if any, must be zero on entry and are zero on return (a caller pads the
 // rank to a multiple of 8 this way); the polishing passes multiply them by finite factors only.
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
                       void* ws, int* info, hipStream_t s) {
   if (passes < 1 || batch > 65535 || r_live < 1 || r_live > r || r - r_live > 63) return DA_ERR_ARG;
-  const long long pr = (long long)rows * r, rr = (long long)r * r;
-  double* P0 = static_cast<double*>(ws);
-  double* G = P0 + pr * batch;
-  double* L = G + rr * batch;
-  double* W = L + rr * batch;
-  float* P0f = reinterpret_cast<float*>(W + rr * batch);
-  bf16_t* P0h = reinterpret_cast<bf16_t*>(P0f + pr * batch);
-  // the Gram products are split over K when they have few tiles: their output is cleared by the conversion
-  // launch that precedes them rather than by one of its own
-  const bool split = da_auto_split(da_gram_blocks(r, batch), rows) > 1;
-  int rc = da_cvt_to_f64(P, dtype, P0, pr * batch, split ? G : nullptr, rr * batch, s);
+  const long long pr = (long long)rows * r;
+  const OrthWs w(ws, batch, rows, r);
+  static const bool force64 = getenv("DION_AMD_ORTH_FP64") != nullptr;
+  const bool low = (r & 7) == 0;   // the bf16 correction product moves 16-byte chunks
+  // (a P that is square or nearly so is a full-rank factor: its condition number is beyond fp32 as a rule)
+  const bool fast = passes == 2 && !force64 && rows >= 4 * r;
+  static const bool no16 = getenv("DION_AMD_ORTH_NO_BF16") != nullptr;
+  const bool fast16 = fast && dtype == DA_BF16 && low && !no16;
+  const DaGate all{nullptr, 0};
+  int rc;
+  if (fast) {
+    // ---- fp32 pass on every matrix
+    float* G = reinterpret_cast<float*>(w.G);
+    float* L = reinterpret_cast<float*>(w.L);
+    float* W = reinterpret_cast<float*>(w.W);
+    rc = da_fill_int(w.info32, batch, 0, s);
+    if (rc) return rc;
+    if (fast16) {
+      rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, s);
+      if (rc) return rc;
+    } else {
+      rc = da_cvt_to_f32(P, dtype, w.Pf, pr, batch, all, s);
+      if (rc) return rc;
+      rc = cholqr_pass<float>(w.Pf, G, L, W, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.info32, all, s);
+      if (rc) return rc;
+      if (low) {
+        rc = da_cvt_f32_to_bf16(w.Pf, w.Ph, pr, batch, all, s);
+        if (rc) return rc;
+      }
+      rc = gram<float>(w.Pf, G, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, all, s);
+      if (rc) return rc;
+    }
+    hipLaunchKernelGGL(decide_fast_kernel, dim3((unsigned)batch), dim3(64), 0, s, w.rowdef, w.info32, w.need, r,
+                       FAST_TOL * FAST_TOL);
+    rc = da_launch_status();
+    if (rc) return rc;
+    const DaGate good{w.need, 0};
+    if (low) rc = correction_bf16(w.Pf, w.Ph, out, dtype, G, reinterpret_cast<bf16_t*>(L), nullptr, batch, rows, r, good, s);
+    else rc = correction_f32(w.Pf, out, da_store_of(dtype), G, L, nullptr, batch, rows, r, good, s);
+    if (rc) return rc;
+  }
+  // ---- fp64 pass: on the flagged matrices, or on all of them
+  const DaGate gate = fast ? DaGate{w.need, 1} : all;
+  rc = da_cvt_to_f64(P, dtype, w.P0, pr, batch, gate, s);
   if (rc) return rc;
-  rc = cholqr_pass(P0, G, L, W, batch, rows, r, r_live, split, info, s);
+  rc = cholqr_pass<double>(w.P0, w.G, w.L, w.W, w.part, batch, rows, r, r_live, info, gate, s);
   if (rc) return rc;
-  if (passes == 1) return da_cvt_from_f64(P0, out, dtype, pr * batch, s);
+  if (passes == 1) return da_cvt_from_f64(w.P0, out, dtype, pr, batch, gate, s);
+  float* Gf = reinterpret_cast<float*>(w.G);
   // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products
-  // (the bf16 product moves 16-byte chunks: r a multiple of 8, else the all-fp32 form below)
-  const bool low = passes == 2 && (r & 7) == 0;
-  // the fp32 Gram matrix of the first polishing pass goes where G was: cleared here for its split-K product
-  rc = da_cvt_f64_to_f32(P0, P0f, low ? P0h : nullptr, pr * batch, split ? reinterpret_cast<float*>(G) : nullptr,
-                         rr * batch, s);
+  const bool last_low = passes == 2 && low;
+  rc = da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate, s);
   if (rc) return rc;
-  if (low)
-    return polish_pass_bf16(P0f, P0h, out, dtype, reinterpret_cast<float*>(G), reinterpret_cast<bf16_t*>(L), batch,
-                            rows, r, split, s);
-  const float* cur = P0f;
-  float* Gf = reinterpret_cast<float*>(G);
-  float* Vf = reinterpret_cast<float*>(L);
+  const float* cur = w.Pf;
   for (int pass = 1; pass < passes; ++pass) {
     const bool last = pass + 1 == passes;
-    // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
-    float* other = cur == P0f ? reinterpret_cast<float*>(P0) : P0f;
-    rc = polish_pass(cur, last ? out : static_cast<void*>(other), last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf, Vf,
-                     batch, rows, r, split && pass == 1, s);
+    rc = gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s);
     if (rc) return rc;
-    cur = other;
+    const int* bad = nullptr;
+    if (pass == 1) {
+      hipLaunchKernelGGL(decide_cols_kernel, dim3((unsigned)batch), dim3(256), 0, s, w.rowdef, w.bad, info, r,
+                         gate.flags, gate.want);
+      rc = da_launch_status();
+      if (rc) return rc;
+      bad = w.bad;
+    }
+    if (last && last_low) {
+      rc = correction_bf16(cur, w.Ph, out, dtype, Gf, reinterpret_cast<bf16_t*>(w.L), bad, batch, rows, r, gate, s);
+    } else {
+      // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
+      float* other = cur == w.Pf ? reinterpret_cast<float*>(w.P0) : w.Pf;
+      rc = correction_f32(cur, last ? out : static_cast<void*>(other), last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf,
+                          reinterpret_cast<float*>(w.L), bad, batch, rows, r, gate, s);
+      cur = other;
+    }
+    if (rc) return rc;
   }
-  return DA_OK;
+  return zero_cols(out, dtype, w.bad, info, batch, rows, r, gate, s);
 }

@@ -174,24 +174,28 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
                                      : static_cast<const char*>(d.E) + (long long)b * d.sE * CSZ;
   const int lr = lane / CPR, c8 = (lane % CPR) * 8;
   const bool col_ok = FULL || wn0 + c8 < dN;
-  // E for one band is fetched up front (its latency overlaps the LDS staging of the accumulators)
-  // and the next band's E is requested before the current band is finished.
-  u32x4_t ev[NPASS][NV];
-  auto load_e = [&](int band) {
+  // E is requested up to three bands ahead (registers that the K loop's fragments no longer need), so that a
+  // tile's epilogue pays one memory latency and not one per band; an fp32 E (twice the registers) one band ahead.
+  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (C::TMI < 3 ? C::TMI : 3);
+  u32x4_t ev[DEPTH][NPASS][NV];
+  auto load_e = [&](int band, u32x4_t (&dst)[NPASS][NV]) {
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
       const int m = wm0 + band * 32 + pass * RPP + lr;
       const u32x4_t z = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int h = 0; h < NV; ++h) ev[pass][h] = z;
+      for (int h = 0; h < NV; ++h) dst[pass][h] = z;
       if (col_ok && (FULL || m < dM)) {
         const char* Ep = Ebase + ((long long)m * lde + wn0 + c8) * CSZ;
 #pragma unroll
-        for (int h = 0; h < NV; ++h) ev[pass][h] = ldg16(Ep + 16 * h);
+        for (int h = 0; h < NV; ++h) dst[pass][h] = ldg16(Ep + 16 * h);
       }
     }
   };
-  if (HAS_E) load_e(0);
+  if (HAS_E) {
+#pragma unroll
+    for (int q = 0; q < DEPTH; ++q) load_e(q, ev[q]);
+  }
 #pragma unroll
   for (int i = 0; i < C::TMI; ++i) {
     {
@@ -210,8 +214,8 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
 #pragma unroll
       for (int pass = 0; pass < NPASS; ++pass)
 #pragma unroll
-        for (int h = 0; h < NV; ++h) ec[pass][h] = ev[pass][h];
-      if (i + 1 < C::TMI) load_e(i + 1);
+        for (int h = 0; h < NV; ++h) ec[pass][h] = ev[i % DEPTH][pass][h];
+      if (i + DEPTH < C::TMI) load_e(i + DEPTH, ev[i % DEPTH]);
     }
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
@@ -343,6 +347,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const int wm = wave / C::WGN, wn = wave % C::WGN;
   const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0);
   const int b = tile.b, ti = tile.ti, tj = tile.tj;
+  if (d.gate && (d.gate[b] != 0) != (d.gate_want != 0)) return;   // (before any barrier: the whole workgroup leaves)
   const int m0 = ti * BT, n0 = tj * BT;
   const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) + d.a_off : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
   const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;

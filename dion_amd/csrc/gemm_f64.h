@@ -16,22 +16,26 @@ struct RealGemmDesc {
   int a_kstrided, b_kstrided, symmetric;
   int lower_only;  // 1 (M == N): only tiles on or below the diagonal are computed and stored
   double alpha, beta;
-  int split_k;   // > 1: K is cut into that many slices whose partial products are added atomically into a
-                 // zeroed C (no E term); the summation order, and so the last bits, vary run to run.
-                 // < 0: the launcher picks the slice count for the tile it chooses and clears C itself
+  int split_k;   // > 1: K is cut into that many slices (no E term); slice s writes its partial product to
+                 // C + s * split_stride and the caller adds the slices in a fixed order (da_auto_split tells it
+                 // how many there are).  < 0: the launcher picks the slice count for the tile it chooses
+  long long split_stride;   // elements between the outputs of consecutive K slices (>= batch * sC)
+  // Optional per-matrix switch: with `gate` set, matrix b is computed only if (gate[b] != 0) == (gate_want != 0);
+  // the workgroups of the other matrices return at once.
+  const int* gate;
+  int gate_want;
   // Storage of C when it is not T (DA_STORE_*): the pointer then addresses elements of that dtype (cast to T*
   // by the caller), ldc and sC count its elements and the result is rounded once at the store.  A converted C
   // excludes E, split_k and the symmetric form.
   int c_store;
   int k_tri;     // 1: B is block lower triangular -- output column tile j only sums k < 64 (j + 1)
-  int c_is_zero; // 1: the caller has cleared C (batch * sC elements): an auto-split product need not do it
 };
 #define DA_STORE_NATIVE 0
 #define DA_STORE_BF16 1
 #define DA_STORE_F32 2
 inline int da_store_of(int dtype) { return dtype == DA_BF16 ? DA_STORE_BF16 : DA_STORE_F32; }
 // Slices of K an auto-split product (split_k < 0) of `blocks` output tiles uses: few tiles with a long K are
-// sliced until ~512 workgroups exist.  > 1 means the product adds into a cleared C.
+// sliced until ~512 workgroups exist.  > 1 means the product leaves that many partial results.
 inline int da_auto_split(long long blocks, int K) {
   const int max_split = K / 256 > 0 ? K / 256 : 1;
   const long long sp = (512 + blocks - 1) / blocks;
@@ -48,14 +52,19 @@ typedef RealGemmDesc<float> Gemm32Desc;
 // The same kernel in fp32 (v_mfma_f32_16x16x4_f32): the products of the polishing passes, whose input is
 // already orthonormal to 1e-4 or better, do not need fp64.
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s);
-// dst (f32) <- src (f64); `low`, if not null, receives the same values in bf16; `zero`, if not null, nz floats
-// cleared in the same launch
-int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, float* zero, long long nz, hipStream_t s);
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s);
 
-// dst (f64) <- src (bf16 / f32), and back; contiguous element counts per call.
-int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, double* zero, long long nz, hipStream_t s);
-int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s);
+// Conversions of `batch` matrices of `per` contiguous elements each; matrix b is converted only if `gate` is null
+// or (gate[b] != 0) == (gate_want != 0).
+struct DaGate { const int* flags; int want; };
+// dst (f64 / f32) <- src (bf16 / f32)
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long per, int batch, DaGate gate, hipStream_t s);
+int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long per, int batch, DaGate gate, hipStream_t s);
+// dst (bf16 / f32) <- src (f64)
+int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long per, int batch, DaGate gate, hipStream_t s);
+// dst (f32) <- src (f64 / f32; dst may be null for an f32 source); `low`, if not null, receives the same values in bf16
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
+int da_cvt_f32_to_bf16(const float* src, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
 
 // Block-column step j = o / 64 of the blocked lower Cholesky G = L L^T of each r x r matrix
 // G[b] (o a multiple of 64; nb = 64 except for a ragged last block): factors the nb x nb diagonal
@@ -63,8 +72,11 @@ int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hi
 // the panel L[o+nb.., o..o+nb] into Lmat[b], and row block j of W[b] (D_j = L_jj^-1 on the
 // diagonal, -D_j L[j, c] left of it).  A non-positive or non-finite pivot zeroes that column (of
 // L_jj and of D_j) and records (o + column + 1) in info[b] if it is the matrix's first failure.
+// `gate`: as in RealGemmDesc.
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, hipStream_t s);
+                 int batch, DaGate gate, hipStream_t s);
+int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
+                     int batch, DaGate gate, hipStream_t s);
 
 #define DA_CHOL_NB 64
 

@@ -76,6 +76,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
   const int per_batch = tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
   const int split = blockIdx.y;  // split-K slice
   const int b = blockIdx.x / per_batch;
+  if (d.gate && (d.gate[b] != 0) != (d.gate_want != 0)) return;
   int t = blockIdx.x - b * per_batch;
   int ti, tj;
   if (tri) {
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
         }
     return;
   }
-  T* C = d.C + (long long)b * d.sC;
+  T* C = d.C + (long long)b * d.sC + (long long)split * d.split_stride;   // each K slice has an output of its own
   const T* E = d.E ? d.E + (long long)b * d.sE : nullptr;
   const bool mirror = SYM && (ti != tj);
 #pragma unroll
@@ -226,22 +227,11 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
         const int n = n0 + wn * WT + j * 16 + (lane & 15);
         if (m < d.M && n < d.N) {
           T o = (T)d.alpha * acc[i][j][v];
-          if (gridDim.y > 1) {  // split-K: partial sums meet in a zeroed C
-            atomicAdd(C + (long long)m * d.ldc + n, o);
-            if (mirror) atomicAdd(C + (long long)n * d.ldc + m, o);
-          } else {
-            if (E) o += (T)d.beta * E[(long long)m * d.lde + n];
-            C[(long long)m * d.ldc + n] = o;
-            if (mirror) C[(long long)n * d.ldc + m] = o;
-          }
+          if (E) o += (T)d.beta * E[(long long)m * d.lde + n];
+          C[(long long)m * d.ldc + n] = o;
+          if (mirror) C[(long long)n * d.ldc + m] = o;
         }
       }
-}
-
-template <typename R>
-__global__ void fill_f64_kernel(R* p, long long n, R v) {
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = v;
 }
 
 template <typename T, int BTt>
@@ -267,52 +257,56 @@ int launch(const RealGemmDesc<T>& d, hipStream_t s) {
   const long long blocks = blocks_of<T, BTt>(d);
   const bool auto_split = d.split_k < 0 && !d.E && d.c_store == DA_STORE_NATIVE;
   int split = d.split_k > 1 && !d.E ? d.split_k : 1;
-  if (auto_split) {
-    split = da_auto_split(blocks, d.K);
-    if (split > 1 && !d.c_is_zero) {
-      // the slices add into C: clear it (the batches of C are contiguous here)
-      const long long n = (long long)d.sC * (d.batch - 1) + (long long)(d.M - 1) * d.ldc + d.N;
-      hipLaunchKernelGGL(fill_f64_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d.C, n, T(0));
-      const int rc = da_launch_status();
-      if (rc) return rc;
-    }
-  }
+  if (auto_split) split = da_auto_split(blocks, d.K);
+  if (split > 1 && d.split_stride < (long long)d.sC * d.batch) return DA_ERR_ARG;
   return launch_bt<T, A_KS, B_KS, SYM, BTt>(d, split, s);
 }
 
-// (`zero`, if not null: nz elements cleared in the same launch -- the output of the split-K product that follows)
-template <typename T, typename R>
-__global__ __launch_bounds__(256) void cvt_to_f64_kernel(const T* __restrict__ src, R* __restrict__ dst,
-                                                         long long n, R* __restrict__ zero, long long nz) {
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
-    dst[i] = (R)ld_as_float<T>(src + i);
-  if (zero)
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nz; i += (long long)gridDim.x * 256) zero[i] = R(0);
+// Element-wise conversions of `batch` matrices of `per` contiguous elements; blockIdx.y = matrix.
+__device__ __forceinline__ bool gate_open(const int* flags, int want, int b) {
+  return !flags || (flags[b] != 0) == (want != 0);
 }
 
 template <typename T, typename R>
-__global__ __launch_bounds__(256) void cvt_from_f64_kernel(const R* __restrict__ src, T* __restrict__ dst,
-                                                           long long n) {
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+__global__ __launch_bounds__(256) void cvt_up_kernel(const T* __restrict__ src, R* __restrict__ dst, long long per,
+                                                     const int* gate, int want) {
+  const long long b = blockIdx.y;
+  if (!gate_open(gate, want, (int)b)) return;
+  src += b * per; dst += b * per;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < per; i += (long long)gridDim.x * 256)
+    dst[i] = (R)ld_as_float<T>(src + i);
+}
+
+template <typename T, typename R>
+__global__ __launch_bounds__(256) void cvt_down_kernel(const R* __restrict__ src, T* __restrict__ dst, long long per,
+                                                       const int* gate, int want) {
+  const long long b = blockIdx.y;
+  if (!gate_open(gate, want, (int)b)) return;
+  src += b * per; dst += b * per;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < per; i += (long long)gridDim.x * 256)
     st_from_float<T>(dst + i, (float)src[i]);
 }
 
-// fp64 -> fp32, and (if `low` is given) the same values rounded once more to bf16
-__global__ __launch_bounds__(256) void cvt_f64_to_f32_kernel(const double* __restrict__ src, float* __restrict__ dst,
-                                                              bf16_t* __restrict__ low, long long n,
-                                                              float* __restrict__ zero, long long nz) {
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+// R (fp64 / fp32) -> fp32 (unless dst is null) and, if `low` is given, the same values rounded once more to bf16
+template <typename R>
+__global__ __launch_bounds__(256) void cvt_f32_low_kernel(const R* __restrict__ src, float* __restrict__ dst,
+                                                          bf16_t* __restrict__ low, long long per, const int* gate,
+                                                          int want) {
+  const long long b = blockIdx.y;
+  if (!gate_open(gate, want, (int)b)) return;
+  src += b * per;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < per; i += (long long)gridDim.x * 256) {
     const float v = (float)src[i];
-    dst[i] = v;
-    if (low) low[i] = f2bf(v);
+    if (dst) dst[b * per + i] = v;
+    if (low) low[b * per + i] = f2bf(v);
   }
-  if (zero)
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nz; i += (long long)gridDim.x * 256) zero[i] = 0.f;
 }
 
-inline unsigned cvt_blocks(long long n) {
-  long long b = (n + 255) / 256;
-  return (unsigned)(b > 8192 ? 8192 : (b < 1 ? 1 : b));
+inline dim3 cvt_grid(long long per, int batch) {
+  long long b = (per + 255) / 256;
+  const long long cap = 8192 / batch > 0 ? 8192 / batch : 1;
+  if (b > cap) b = cap;
+  return dim3((unsigned)(b < 1 ? 1 : b), (unsigned)batch);
 }
 
 template <typename T>
@@ -333,24 +327,12 @@ int gemm_real(const RealGemmDesc<T>& d, hipStream_t s) {
 }
 
 template <typename R>
-int cvt_to(const void* src, int src_dtype, R* dst, long long n, R* zero, long long nz, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
+int cvt_up(const void* src, int src_dtype, R* dst, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   if (src_dtype == DA_BF16)
-    hipLaunchKernelGGL((cvt_to_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, n, zero, nz);
+    hipLaunchKernelGGL((cvt_up_kernel<bf16_t, R>), cvt_grid(per, batch), dim3(256), 0, s, static_cast<const bf16_t*>(src), dst, per, g.flags, g.want);
   else if (src_dtype == DA_F32)
-    hipLaunchKernelGGL((cvt_to_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, static_cast<const float*>(src), dst, n, zero, nz);
-  else
-    return DA_ERR_DTYPE;
-  return da_launch_status();
-}
-
-template <typename R>
-int cvt_from(const R* src, void* dst, int dst_dtype, long long n, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
-  if (dst_dtype == DA_BF16)
-    hipLaunchKernelGGL((cvt_from_f64_kernel<bf16_t, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), n);
-  else if (dst_dtype == DA_F32)
-    hipLaunchKernelGGL((cvt_from_f64_kernel<float, R>), dim3(cvt_blocks(n)), dim3(256), 0, s, src, static_cast<float*>(dst), n);
+    hipLaunchKernelGGL((cvt_up_kernel<float, R>), cvt_grid(per, batch), dim3(256), 0, s, static_cast<const float*>(src), dst, per, g.flags, g.want);
   else
     return DA_ERR_DTYPE;
   return da_launch_status();
@@ -361,12 +343,29 @@ int cvt_from(const R* src, void* dst, int dst_dtype, long long n, hipStream_t s)
 int da_gemm_f64(const Gemm64Desc& d, hipStream_t s) { return gemm_real<double>(d, s); }
 int da_gemm_f32s(const Gemm32Desc& d, hipStream_t s) { return gemm_real<float>(d, s); }
 
-int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long n, double* zero, long long nz, hipStream_t s) {
-  return cvt_to<double>(src, src_dtype, dst, n, zero, nz, s);
+int da_cvt_to_f64(const void* src, int src_dtype, double* dst, long long per, int batch, DaGate g, hipStream_t s) {
+  return cvt_up<double>(src, src_dtype, dst, per, batch, g, s);
 }
-int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long n, hipStream_t s) { return cvt_from<double>(src, dst, dst_dtype, n, s); }
-int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long n, float* zero, long long nz, hipStream_t s) {
-  if (n <= 0) return DA_ERR_ARG;
-  hipLaunchKernelGGL(cvt_f64_to_f32_kernel, dim3(cvt_blocks(n)), dim3(256), 0, s, src, dst, low, n, zero, nz);
+int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long per, int batch, DaGate g, hipStream_t s) {
+  return cvt_up<float>(src, src_dtype, dst, per, batch, g, s);
+}
+int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  if (dst_dtype == DA_BF16)
+    hipLaunchKernelGGL((cvt_down_kernel<bf16_t, double>), cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), per, g.flags, g.want);
+  else if (dst_dtype == DA_F32)
+    hipLaunchKernelGGL((cvt_down_kernel<float, double>), cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<float*>(dst), per, g.flags, g.want);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  hipLaunchKernelGGL(cvt_f32_low_kernel<double>, cvt_grid(per, batch), dim3(256), 0, s, src, dst, low, per, g.flags, g.want);
+  return da_launch_status();
+}
+int da_cvt_f32_to_bf16(const float* src, bf16_t* low, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  hipLaunchKernelGGL(cvt_f32_low_kernel<float>, cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<float*>(nullptr), low, per, g.flags, g.want);
   return da_launch_status();
 }
