@@ -82,6 +82,78 @@ def test_orthonormalize_batch_and_rank_deficient(dev):
     assert torch.equal(orthonormalize(P[0].to(dev)), Q[0])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_orthonormalize_numerically_rank_deficient(dev, dtype):
+    """P = A B of rank 96 < r = 128: the dependent columns have pivots at round-off level of either sign.  They must
+    not come back as scaled noise: the result is finite, every column is a unit vector or zero, the kept columns
+    are orthonormal, and `info` reports the first dropped column."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(3)
+    rows, r, k = 1024, 128, 96
+    P = (torch.randn(rows, k, dtype=torch.float64) @ torch.randn(k, r, dtype=torch.float64)).to(dtype)
+    Q, info = orthonormalize(P.to(dev), return_info=True)
+    assert torch.isfinite(Q).all()
+    Qd = Q.double().cpu()
+    norms = Qd.norm(dim=0)
+    kept = norms > 0.5
+    tol = 1e-3 if dtype == torch.float32 else 3e-2
+    assert ((norms[kept] - 1).abs() <= tol).all() and (norms[~kept] == 0).all()
+    if dtype == torch.float32:
+        assert int(info.item()) != 0
+        assert int(kept.sum()) >= k - 2 and int(kept.sum()) <= k + 2
+    else:
+        # rounded to bf16 the dependent columns carry 2^-9 of independent noise: P has full rank with a condition
+        # number of a few thousand, and keeping every column is as valid as dropping the noisy ones
+        assert (int(info.item()) != 0) == (int(kept.sum()) < r)
+    Qk = Qd[:, kept]
+    assert (Qk.T @ Qk - torch.eye(Qk.shape[1], dtype=torch.float64)).norm().item() <= (ORTH_TOL if dtype == torch.float32 else 0.3)
+    # the kept columns span P's column space
+    resid = P.double() - Qk @ (Qk.T @ P.double())
+    assert (resid.norm() / P.double().norm()).item() <= (1e-4 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,r", [(768, 192), (3072, 512)])
+def test_orthonormalize_fp32_first_pass_agrees_with_the_fp64_pass(dev, dtype, rows, r):
+    """A well-conditioned factor takes the fp32 pass (two passes asked for, rows >= 4 r); three passes always run the
+    fp64 pass.  Same thin-QR factor either way."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(4)
+    P = torch.randn(4, rows, r).to(dtype).to(dev)
+    Qa, ia = orthonormalize(P, passes=2, return_info=True)
+    Qb, ib = orthonormalize(P, passes=3, return_info=True)
+    assert ia.abs().sum().item() == 0 and ib.abs().sum().item() == 0
+    d = rel_fro(Qa.double().cpu(), Qb.double().cpu())
+    print(f"fp32-first vs fp64 pass, {rows}x{r} {dtype}: {d:.2e}")
+    assert d <= (2e-5 if dtype == torch.float32 else 4e-3)
+    Qd = Qa[0].double().cpu()
+    orth = (Qd.T @ Qd - torch.eye(r, dtype=torch.float64)).norm().item()
+    assert orth <= (2e-5 if dtype == torch.float32 else 5e-2 * (r ** 0.5) / 8)
+
+
+def test_dion_step_with_a_rank_deficient_gradient_stays_bounded(dev):
+    """First step from zero momentum with a gradient of rank 8 < r = 64: B Q has rank 8."""
+    from dion_amd import Dion
+
+    torch.manual_seed(6)
+    m, n = 512, 256
+    p = torch.nn.Parameter((torch.randn(m, n) * 0.02).to(dev))
+    opt = Dion([p], rank_fraction=0.25, lr=0.01, mu=0.95, weight_decay=0.0)
+    x0 = p.detach().clone()
+    for _ in range(3):
+        p.grad = ((torch.randn(m, 8) @ torch.randn(8, n)) * 1e-3).to(dev)
+        opt.step()
+    torch.cuda.synchronize()
+    st = opt.state[p]
+    assert torch.isfinite(p).all() and torch.isfinite(st["momentum"]).all() and torch.isfinite(st["Q"]).all()
+    # an orthonormal P bounds the update: ||P Qn^T||_F <= sqrt(r), scaled by lr * sqrt(m / n)
+    step_bound = 0.01 * (m / n) ** 0.5 * (64 ** 0.5) * 1.05
+    assert (p.detach() - x0).norm().item() <= 3 * step_bound
+    assert st["momentum"].norm().item() <= 3 * (1e-3 * 8 ** 0.5 * (m * n) ** 0.5) * 1.5
+
+
 def _run_dion(dev, shapes, rank_fraction, steps, x_dtype, m_dtype, q_dtype, seed_q=2, seed_g=3, lr=0.01, mu=0.95, wd=0.01,
               check=None):
     from dion_amd import Dion, DionMixedPrecisionConfig
