@@ -52,9 +52,12 @@ _SIGNATURES = {
     "dion_amd_muon_workspace_bytes": (_sz, [_i, _i, _i]),
     "dion_amd_orthonormalize_workspace_bytes": (_sz, [_i, _i, _i]),
     "dion_amd_orthonormalize": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "dion_amd_orthonormalize_method": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "dion_amd_dion_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "dion_amd_dion_step": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i,
                                 _vp, _vp, _sz, _vp]),
+    "dion_amd_dion_step_qr": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i, _i,
+                                   _vp, _vp, _sz, _vp]),
     "dion_amd_profile_enable": (_i, [_i]),
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),
@@ -172,6 +175,8 @@ class Workspace:
             self._buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         return self._buf
 
+
+QR_METHODS = {"rcqr": 0, "qr": 1, "cqr": 2}   # DION_AMD_QR_*
 
 PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
               "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt", "dion_ef_upd")

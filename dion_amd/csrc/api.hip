@@ -637,7 +637,14 @@ size_t dion_amd_orthonormalize_workspace_bytes(int batch, int rows, int r) {
 
 int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
                             int* info, void* workspace, size_t workspace_bytes, void* stream) {
+  return dion_amd_orthonormalize_method(P, out, dtype, batch, rows, r, passes, DA_QR_AUTO, info, workspace,
+                                        workspace_bytes, stream);
+}
+
+int dion_amd_orthonormalize_method(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
+                                   int qr_method, int* info, void* workspace, size_t workspace_bytes, void* stream) {
   if (!P || !out || !workspace || batch <= 0 || rows <= 0 || r <= 0 || passes < 1 || passes > 3) return DA_ERR_ARG;
+  if (qr_method < 0 || qr_method > 2) return DA_ERR_ARG;
   if (!dtype_ok(dtype)) return DA_ERR_DTYPE;
   if (r > rows) return DA_ERR_ARG;
   if (workspace_bytes < dion_amd_orthonormalize_workspace_bytes(batch, rows, r)) return DA_ERR_WORKSPACE;
@@ -648,13 +655,22 @@ int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int 
   int rc = da_fill_int(inf, batch, 0, s);
   if (rc) return rc;
   DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-  return da_orthonormalize(P, out, dtype, batch, rows, r, r, passes, workspace, inf, s);
+  return da_orthonormalize(P, out, dtype, batch, rows, r, r, passes, qr_method, workspace, inf, s);
 }
 
 int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
                        int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
                        float scaled_lr, float eps, int faithful, int power_iters, int* info, void* workspace,
                        size_t workspace_bytes, void* stream) {
+  return dion_amd_dion_step_qr(X, G, M, Q, batch, m, n, rank, x_dtype, g_dtype, m_dtype, q_dtype, ef_alpha, decay,
+                               scaled_lr, eps, faithful, power_iters, DA_QR_AUTO, info, workspace, workspace_bytes, stream);
+}
+
+int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
+                          int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
+                          float scaled_lr, float eps, int faithful, int power_iters, int qr_method, int* info,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+  if (qr_method < 0 || qr_method > 2) return DA_ERR_ARG;
   if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || rank <= 0) return DA_ERR_ARG;
   if (power_iters < 1 || power_iters > 64) return DA_ERR_ARG;
   if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype) || !dtype_ok(m_dtype) || !dtype_ok(q_dtype)) return DA_ERR_DTYPE;
@@ -729,7 +745,7 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
       // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
       {
         DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-        rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, orth_ws, linfo, s);
+        rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, qr_method, orth_ws, linfo, s);
         if (rc) return rc;
         // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
         rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);

@@ -29,8 +29,12 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
 // column (0 = success); failed columns come out as zeros.  Columns r_live .. r-1 of P are zero
 // padding (r_live == r: none) and stay zero.
 size_t da_orth_workspace_bytes(int batch, int rows, int r);
+// method: how the first pass is chosen (the reference's qr_method, dion/dion_reference.py:733-789)
+#define DA_QR_AUTO 0   // "rcqr": CholeskyQR in fp32, its measured defect sends a matrix on to the fp64 pass
+#define DA_QR_FP64 1   // "qr": the fp64 pass for every matrix
+#define DA_QR_CQR 2    // "cqr": one CholeskyQR pass in fp32 and nothing else; a failed factorisation falls back to DA_QR_AUTO's fp64 pass
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
-                      void* ws, int* info, hipStream_t s);
+                      int method, void* ws, int* info, hipStream_t s);
 
 // Error feedback and weight update in one pass (dion_fused.hip), bf16 factors:
 //   M[b] <- M[b] + ef_alpha P[b] R[b]^T,  X[b] <- decay X[b] - scaled_lr P[b] Qn[b]^T   (R P^T, Qn P^T when `transposed`)

@@ -800,7 +800,8 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
 //   recurrence of the triangular solve applied to the identity), P1 = P T with T as two bf16 factors (T to 16
 //   bits: P1 stays an exact triangular recombination of P's columns, so its thin-QR factor is P's), kept as
 //   h + l (bf16 each); then G2 = P1^T P1 = h^T h + h^T l + l^T h for the defect and the polishing pass.
-int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, int r_live, hipStream_t s) {
+int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, int r_live, bool second_gram,
+                hipStream_t s) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
@@ -863,8 +864,24 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)(blocks < 1 ? 1 : blocks), (unsigned)batch), dim3(256), 0, s, C2,
                      w.Ph, Lo, pr, r);
   rc = da_launch_status();
-  if (rc) return rc;
+  if (rc || !second_gram) return rc;
   return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, s);
+}
+
+// bf16 copy of the matrices whose gate is open
+__global__ __launch_bounds__(256) void copy_bf16_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst,
+                                                        long long per, const int* gate, int want) {
+  const long long b = blockIdx.y;
+  if (!orth_gate_open(gate, want, (int)b)) return;
+  const uint4* s4 = reinterpret_cast<const uint4*>(src + b * per);
+  uint4* d4 = reinterpret_cast<uint4*>(dst + b * per);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < per / 8; i += (long long)gridDim.x * 256) d4[i] = s4[i];
+}
+
+// need[b] = the fp32 factorisation of matrix b met a pivot that was not positive
+__global__ void decide_cqr_kernel(const int* __restrict__ info32, int* __restrict__ need, int batch) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < batch) need[b] = info32[b] != 0 ? 1 : 0;
 }
 
 // Defect ||P^T P - I||_F up to which the closed-form polishing pass is trusted after the fp32 pass: it leaves
@@ -886,19 +903,49 @@ constexpr float FAST_TOL = 2e-3f;
 // Columns r_live .. r-1 of P, if any, must be zero on entry and are zero on return (a caller pads the
 // rank to a multiple of 8 this way); the polishing passes multiply them by finite factors only.
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
-                      void* ws, int* info, hipStream_t s) {
+                      int method, void* ws, int* info, hipStream_t s) {
   if (passes < 1 || batch > 65535 || r_live < 1 || r_live > r || r - r_live > 63) return DA_ERR_ARG;
+  if (method != DA_QR_AUTO && method != DA_QR_FP64 && method != DA_QR_CQR) return DA_ERR_ARG;
   const long long pr = (long long)rows * r;
   const OrthWs w(ws, batch, rows, r);
   static const bool force64 = getenv("DION_AMD_ORTH_FP64") != nullptr;
   const bool low = (r & 7) == 0;   // the bf16 correction product moves 16-byte chunks
   // (a P that is square or nearly so is a full-rank factor: its condition number is beyond fp32 as a rule)
-  const bool fast = passes == 2 && !force64 && rows >= 4 * r;
+  const bool cqr = passes == 2 && method == DA_QR_CQR;
+  const bool fast = cqr || (passes == 2 && method == DA_QR_AUTO && !force64 && rows >= 4 * r);
   static const bool no16 = getenv("DION_AMD_ORTH_NO_BF16") != nullptr;
   const bool fast16 = fast && dtype == DA_BF16 && low && !no16;
   const DaGate all{nullptr, 0};
   int rc;
-  if (fast) {
+  if (cqr) {
+    // ---- "cqr": the fp32 CholeskyQR pass is the result (reference dion/dion_reference.py:752-758)
+    rc = da_fill_int(w.info32, batch, 0, s);
+    if (rc) return rc;
+    if (fast16) {
+      rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, false, s);
+    } else {
+      rc = da_cvt_to_f32(P, dtype, w.Pf, pr, batch, all, s);
+      if (rc) return rc;
+      rc = cholqr_pass<float>(w.Pf, reinterpret_cast<float*>(w.G), reinterpret_cast<float*>(w.L),
+                              reinterpret_cast<float*>(w.W), reinterpret_cast<float*>(w.part), batch, rows, r, r_live,
+                              w.info32, all, s);
+    }
+    if (rc) return rc;
+    hipLaunchKernelGGL(decide_cqr_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, w.info32, w.need, batch);
+    rc = da_launch_status();
+    if (rc) return rc;
+    const DaGate good{w.need, 0};
+    if (fast16) {
+      long long blocks = (pr / 8 + 255) / 256;
+      if (blocks > 1024) blocks = 1024;
+      hipLaunchKernelGGL(copy_bf16_kernel, dim3((unsigned)(blocks < 1 ? 1 : blocks), (unsigned)batch), dim3(256), 0, s, w.Ph,
+                         static_cast<bf16_t*>(out), pr, good.flags, good.want);
+      rc = da_launch_status();
+    } else {
+      rc = da_cvt_from_f32(w.Pf, out, dtype, pr, batch, good, s);
+    }
+    if (rc) return rc;
+  } else if (fast) {
     // ---- fp32 pass on every matrix
     float* G = reinterpret_cast<float*>(w.G);
     float* L = reinterpret_cast<float*>(w.L);
@@ -906,7 +953,7 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     rc = da_fill_int(w.info32, batch, 0, s);
     if (rc) return rc;
     if (fast16) {
-      rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, s);
+      rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, true, s);
       if (rc) return rc;
     } else {
       rc = da_cvt_to_f32(P, dtype, w.Pf, pr, batch, all, s);

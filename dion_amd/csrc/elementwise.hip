@@ -17,7 +17,8 @@
 
 namespace {
 
-constexpr int TS = 64;  // tile edge; 256 threads, 16 elements (two 8-wide chunks) per thread
+constexpr int TS = 64;  // tile edge of the transposing passes; 256 threads, 16 elements (two 8-wide chunks) per thread
+constexpr int RT = 32, CT = 256;   // tile of the passes that keep the orientation: 32 rows x 256 columns
 
 template <typename T> struct Vec8;
 template <> struct Vec8<bf16_t> {
@@ -134,6 +135,55 @@ __global__ __launch_bounds__(256) void stage_wide_kernel(StageArgs<TG, TM, TW> a
   TW* W = a.use_wtab ? static_cast<TW*>(a.wtab.p[b]) : a.wide + (long long)b * mw * a.ldw;
 
   float ss = 0.f;
+  if (!TALL) {
+    // No transpose: a tile is RT rows x CT columns, a wavefront's 16-byte accesses cover whole 512-byte row
+    // segments, and all of a thread's loads are requested before the first is used.
+    const int tiles_cw = (a.cols + CT - 1) / CT;
+    const int wi = blockIdx.x / tiles_cw, wj = blockIdx.x % tiles_cw;
+    constexpr int NC = RT * CT / 8 / 256;   // chunks per thread
+    float g[NC][8], m[NC][8];
+    bool ok[NC];
+#pragma unroll
+    for (int it = 0; it < NC; ++it) {
+      const int c = tid + 256 * it;
+      const int i = wi * RT + c / (CT / 8), j = wj * CT + (c % (CT / 8)) * 8;
+      ok[it] = i < a.rows && j < a.cols;
+      if (ok[it]) {
+        Vec8<TG>::load_nt(G + (long long)i * a.ld + j, g[it]);
+        if (a.muon) Vec8<TM>::load_nt(M + (long long)i * a.cols + j, m[it]);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NC; ++it) {
+      if (!ok[it]) continue;
+      const int c = tid + 256 * it;
+      const int i = wi * RT + c / (CT / 8), j = wj * CT + (c % (CT / 8)) * 8;
+      float u[8];
+      if (a.muon) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float ge = Vec8<TM>::round(g[it][e]);             // G.to(M.dtype)
+          float me = Vec8<TM>::round(m[it][e] * a.mu);            // M *= mu
+          me = Vec8<TM>::round(me + ge);                          // M += G
+          m[it][e] = me;
+          float ue = me;
+          if (a.nesterov) ue = Vec8<TM>::round(Vec8<TM>::round(me * a.mu) + ge);  // U = M*mu; U += G
+          u[e] = Vec8<TW>::round(ue);                             // U.to(bf16)
+        }
+        Vec8<TM>::store_nt(M + (long long)i * a.cols + j, m[it]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[e] = Vec8<TW>::round(g[it][e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += u[e] * u[e];
+      Vec8<TW>::store(W + (long long)i * a.ldw + j, u);
+    }
+    if (!a.partials) return;   // (uniform over the grid)
+    const float s = block_sum(ss, red);
+    if (tid == 0) a.partials[(long long)b * gridDim.x + blockIdx.x] = s;
+    return;
+  }
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int c = tid + 256 * it;        // chunk id within tile: 64 rows x 8 chunks
@@ -219,18 +269,46 @@ __global__ __launch_bounds__(256) void norm_finish_kernel(const float* partials,
   }
 }
 
+// x / d for a divisor shared by many elements: with rd = RN(1 / d), one residual step on the estimate x * rd gives
+// the correctly rounded quotient (three fused operations instead of the dozen of a full division; the pass is
+// otherwise bound by its arithmetic).  |x| <= d here (d is the matrix's Frobenius norm plus eps), so nothing
+// overflows; a divisor whose reciprocal is zero or not finite takes the plain division (the caller's branch).
+__device__ __forceinline__ float div_by(float x, float d, float rd) {
+  const float q = x * rd;
+  const float rem = __builtin_fmaf(-q, d, x);
+  return __builtin_fmaf(rem, rd, q);
+}
+
 template <typename TW>
 __global__ __launch_bounds__(256) void normalize_kernel(TW* W, long long per_matrix, const float* divisor) {
   const int b = blockIdx.y;
   const float d = divisor[b];
+  const float rd = 1.f / d;
+  const bool fast = __builtin_isfinite(rd) && rd != 0.f;   // (the same for the whole matrix)
   TW* p = W + (long long)b * per_matrix;
-  for (long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 8; i < per_matrix;
-       i += (long long)gridDim.x * 256 * 8) {
-    float v[8];
-    Vec8<TW>::load(p + i, v);
+  // four 16-byte chunks per thread and trip, all requested before the first is used
+  for (long long i0 = (long long)blockIdx.x * 8192; i0 < per_matrix; i0 += (long long)gridDim.x * 8192) {
+    float v[4][8];
+    bool ok[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = v[e] / d;
-    Vec8<TW>::store(p + i, v);
+    for (int q = 0; q < 4; ++q) {
+      const long long i = i0 + (q * 256 + threadIdx.x) * 8;
+      ok[q] = i < per_matrix;
+      if (ok[q]) Vec8<TW>::load(p + i, v[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (!ok[q]) continue;
+      const long long i = i0 + (q * 256 + threadIdx.x) * 8;
+      if (fast) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] = div_by(v[q][e], d, rd);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[q][e] = v[q][e] / d;
+      }
+      Vec8<TW>::store(p + i, v[q]);
+    }
   }
 }
 
@@ -260,6 +338,42 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
   const int mw = TALL ? a.cols : a.rows, nw = TALL ? a.rows : a.cols;
   const TW* W = a.use_wtab ? static_cast<const TW*>(a.wtab.p[b]) : a.wide + (long long)b * mw * a.ldw;
 
+  if (!TALL) {
+    const int tiles_cw = (a.cols + CT - 1) / CT;
+    const int wi = blockIdx.x / tiles_cw, wj = blockIdx.x % tiles_cw;
+    constexpr int NC = RT * CT / 8 / 256;
+    float u[NC][8], x[NC][8];
+    bool ok[NC];
+#pragma unroll
+    for (int it = 0; it < NC; ++it) {
+      const int c = tid + 256 * it;
+      const int i = wi * RT + c / (CT / 8), j = wj * CT + (c % (CT / 8)) * 8;
+      ok[it] = i < a.rows && j < a.cols;
+      if (ok[it]) {
+        Vec8<TW>::load(W + (long long)i * a.ldw + j, u[it]);
+        if (a.muon) Vec8<TX>::load_nt(X + (long long)i * a.ld + j, x[it]);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NC; ++it) {
+      if (!ok[it]) continue;
+      const int c = tid + 256 * it;
+      const int i = wi * RT + c / (CT / 8), j = wj * CT + (c % (CT / 8)) * 8;
+      TX* xp = X + (long long)i * a.ld + j;
+      if (a.muon) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xd = Vec8<TX>::round(x[it][e] * a.decay);    // X *= 1 - lr*wd
+          const float t = Vec8<TW>::round(u[it][e] * a.step);      // U * adjusted_lr (U's dtype)
+          x[it][e] = xd - t;                                       // X -= U ; rounded by the store
+        }
+        Vec8<TX>::store_nt(xp, x[it]);
+      } else {
+        Vec8<TX>::store(xp, u[it]);
+      }
+    }
+    return;
+  }
   if (TALL) {
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
@@ -309,7 +423,8 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
 
 template <typename TG, typename TM, typename TW>
 int stage_launch(const StageArgs<TG, TM, TW>& a, int batch, bool tall, hipStream_t s) {
-  const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
+  const int tiles = tall ? ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS)
+                         : ((a.rows + RT - 1) / RT) * ((a.cols + CT - 1) / CT);
   dim3 grid(tiles, batch);
   if (tall) hipLaunchKernelGGL((stage_wide_kernel<TG, TM, TW, true>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((stage_wide_kernel<TG, TM, TW, false>), grid, dim3(256), 0, s, a);
@@ -329,16 +444,21 @@ int stage_dispatch_w(const DaStage& d, hipStream_t s) {
 template <typename TX, typename TW>
 int unstage_launch(const DaUnstage& d, hipStream_t s) {
   UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon, d.use_wtab, d.wtab};
-  const int tiles = ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS);
+  const bool tall = d.rows > d.cols && !d.use_wtab;
+  const int tiles = tall ? ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS)
+                         : ((a.rows + RT - 1) / RT) * ((a.cols + CT - 1) / CT);
   dim3 grid(tiles, d.batch);
-  if (d.rows > d.cols && !d.use_wtab) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
+  if (tall) hipLaunchKernelGGL((unstage_kernel<TX, TW, true>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((unstage_kernel<TX, TW, false>), grid, dim3(256), 0, s, a);
   return da_launch_status();
 }
 
 }  // namespace
 
-int da_stage_tiles(int rows, int cols) { return ((rows + TS - 1) / TS) * ((cols + TS - 1) / TS); }
+// Workgroups (and partial sums of squares) per matrix of da_stage_wide: transposing tiles for a tall source.
+int da_stage_tiles(int rows, int cols) {
+  return rows > cols ? ((rows + TS - 1) / TS) * ((cols + TS - 1) / TS) : ((rows + RT - 1) / RT) * ((cols + CT - 1) / CT);
+}
 
 int da_stage_wide(const DaStage& d, hipStream_t s) {
   if (d.batch <= 0 || d.batch > DA_MAX_PTRS) return DA_ERR_LIMIT;
@@ -359,7 +479,7 @@ int da_norm_finish(const float* partials, int tiles, int batch, float eps, int b
 
 int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor, hipStream_t s) {
   if (per_matrix & 7) return DA_ERR_ALIGN;
-  long long blocks = (per_matrix / 8 + 255) / 256;
+  long long blocks = (per_matrix + 8191) / 8192;
   if (blocks > 2048) blocks = 2048;
   dim3 grid((unsigned)blocks, batch);
   if (w_dtype == DA_BF16)

@@ -65,6 +65,8 @@ int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long per, 
 // dst (f32) <- src (f64 / f32; dst may be null for an f32 source); `low`, if not null, receives the same values in bf16
 int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
 int da_cvt_f32_to_bf16(const float* src, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
+// dst (bf16 / f32) <- src (f32)
+int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, int batch, DaGate gate, hipStream_t s);
 
 // Block-column step j = o / 64 of the blocked lower Cholesky G = L L^T of each r x r matrix
 // G[b] (o a multiple of 64; nb = 64 except for a ragged last block): factors the nb x nb diagonal

@@ -359,6 +359,16 @@ int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long per, 
     return DA_ERR_DTYPE;
   return da_launch_status();
 }
+int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  if (dst_dtype == DA_BF16)
+    hipLaunchKernelGGL((cvt_down_kernel<bf16_t, float>), cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<bf16_t*>(dst), per, g.flags, g.want);
+  else if (dst_dtype == DA_F32)
+    hipLaunchKernelGGL((cvt_down_kernel<float, float>), cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<float*>(dst), per, g.flags, g.want);
+  else
+    return DA_ERR_DTYPE;
+  return da_launch_status();
+}
 int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate g, hipStream_t s) {
   if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   hipLaunchKernelGGL(cvt_f32_low_kernel<double>, cvt_grid(per, batch), dim3(256), 0, s, src, dst, low, per, g.flags, g.want);

@@ -290,14 +290,20 @@ class Dion(Optimizer):
                     crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
                     Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
                 ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
-                rc = lib.dion_amd_dion_step(
+                # Cholesky QR only after the warm-up, when the factors are well conditioned
+                # (reference dion/dion_reference.py:296-299)
+                qr_method = self._qr_method
+                if qr_method == "cqr" and group["step"] <= self._cqr_warmup_steps:
+                    qr_method = "rcqr"
+                rc = lib.dion_amd_dion_step_qr(
                     _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
                     len(plist), m, n, r,
                     _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
                     ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
+                    _lib.QR_METHODS[qr_method],
                     info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
                 )
-                _lib.check(rc, "dion_amd_dion_step")
+                _lib.check(rc, "dion_amd_dion_step_qr")
                 for dst, padded in crops:
                     _lib.crop_back(dst, padded)
                 del Xs, Gs, Ms, Qs, crops
@@ -329,17 +335,35 @@ class Dion(Optimizer):
         )
 
 
+def generate_random_sketch_matrix(P: Tensor, oversample: float = 1.25, shard_mesh_dim=None) -> Tensor:
+    """The sketch of the reference's randomised Cholesky QR (dion/dion.py:1221-1263) for a batch P of shape
+    (..., m, r): S of shape (..., k, m) with k = oversample * r rounded up to a multiple of 128 and entries
+    N(0, 1/k) in P's dtype, drawn from torch's generator for P's device.  The device orthonormaliser draws no
+    sketch (its "rcqr" preconditions with an fp32 CholeskyQR pass instead), so nothing in `Dion.step()` calls this;
+    it is here for callers of the reference's helper.  One GPU: `shard_mesh_dim` must be None."""
+    assert P.ndim >= 3, "P must have batch dimension"
+    if shard_mesh_dim is not None:
+        raise TypeError("Must use DTensor parameters for sharded random sketch.")
+    m, r = P.size(-2), P.size(-1)
+    k = math.ceil(oversample * r / 128.0) * 128
+    std = math.sqrt(1.0 / k)
+    return torch.empty((*P.shape[:-2], k, m), device=P.device, dtype=P.dtype).normal_(std=std)
+
+
 class DionReference(Dion):
     """Counterpart of the reference's per-matrix class (`dion.DionReference`, dion/dion_reference.py:64-365) on one
     GPU: the same constructor, which also takes `power_iters` >= 1 and `qr_method` in {"qr", "cqr", "rcqr"}
     (dion/dion_reference.py:131-134), and the same update (`dion_update`, dion/dion_reference.py:613-687; its
     `power_iteration`, 690-730, repeats P = orth(B Q), Q = B^T P with the unnormalised Q).
 
-    All three `qr_method` names run the device orthonormaliser: Householder QR, Cholesky QR and randomised
-    Cholesky QR (dion/dion_reference.py:733-789) are three ways to the same thin-QR factor, which they return with
-    different column signs; M and X do not see those signs and Q carries them consistently.  So `cqr_warmup_steps`
-    and the fall-back from a failed Cholesky factorisation to the randomised method (752-758, 296-299) have nothing
-    left to switch between: the factorisation here is in fp64 and its status is in `cholesky_info()`.
+    `qr_method` selects the device orthonormaliser's first pass as the reference selects its factorisation
+    (dion/dion_reference.py:733-789): "rcqr" -- CholeskyQR in fp32, and in fp64 for the matrices whose measured
+    defect asks for it (the robust default, standing where the reference preconditions with a random sketch);
+    "qr" -- the fp64 pass for every matrix (standing for Householder QR); "cqr" -- one fp32 CholeskyQR pass and
+    nothing else, used after `cqr_warmup_steps` steps only (296-299), with the fall-back for a failed
+    factorisation taken per matrix on the device (752-758).  All three return the thin-QR factor with a positive
+    diagonal of R; the reference's Householder-based variants differ from it by column signs, which M and X do
+    not see and Q carries consistently.  The status of the factorisations is in `cholesky_info()`.
     `state["Q"]` is updated in place rather than replaced by a new tensor."""
 
     _REFERENCE_OPTIONS = True

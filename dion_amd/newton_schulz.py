@@ -146,10 +146,12 @@ def gemm(A: Tensor, B: Tensor, *, a_kstrided=False, b_kstrided=False, E: Tensor 
     return out if A.ndim == 3 else out[0]
 
 
-def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False):
-    """Thin-QR Q factor of P (rows x r) or a batch of them on the device (one CholeskyQR pass in fp64, then
-    `passes - 1` fp32 polishing passes); counterpart of `orthogonalize` (reference dion/dion.py:1267-1308),
-    equal up to column signs."""
+def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False, qr_method: str = "rcqr"):
+    """Thin-QR Q factor of P (rows x r) or a batch of them on the device; counterpart of `orthogonalize`
+    (reference dion/dion.py:1267-1308, dion/dion_reference.py:733-789), equal up to column signs.
+    qr_method: "rcqr" -- CholeskyQR in fp32, in fp64 for the matrices whose measured defect asks for it, then a
+    polishing pass; "qr" -- the fp64 pass for every matrix; "cqr" -- one fp32 CholeskyQR pass and nothing else
+    (fp64 pass only if the factorisation fails)."""
     lib = _lib.load()
     _lib.require_gpu(P, "orthonormalize")
     P3 = (P if P.ndim == 3 else P.unsqueeze(0)).contiguous()
@@ -159,8 +161,9 @@ def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False):
     nbytes = lib.dion_amd_orthonormalize_workspace_bytes(batch, rows, r)
     ws = _workspace.get(nbytes, P.device)
     with torch.cuda.device(P.device):
-        rc = lib.dion_amd_orthonormalize(P3.data_ptr(), out.data_ptr(), _lib.dtype_code(P.dtype), batch, rows, r,
-                                         passes, info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(P.device))
-    _lib.check(rc, "dion_amd_orthonormalize")
+        rc = lib.dion_amd_orthonormalize_method(P3.data_ptr(), out.data_ptr(), _lib.dtype_code(P.dtype), batch, rows, r,
+                                                passes, _lib.QR_METHODS[qr_method], info.data_ptr(), ws.data_ptr(),
+                                                ws.numel(), _lib.stream_ptr(P.device))
+    _lib.check(rc, "dion_amd_orthonormalize_method")
     out = out if P.ndim == 3 else out[0]
     return (out, info) if return_info else out

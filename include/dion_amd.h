@@ -231,16 +231,35 @@ size_t dion_amd_orthonormalize_workspace_bytes(int batch, int rows, int r);
 /* Replaces orthogonalize (reference dion/dion.py:1267-1308; per-matrix variants
  * dion/dion_reference.py:733-789): thin-QR Q factor of each of `batch` contiguous matrices
  * P_b (rows x r, rows >= r, dtype bf16 or f32), written to out_b (same layout; may alias P).
- * Method: CholeskyQR2.  The first pass (Gram matrix, blocked Cholesky factorisation,
- * triangular solve) runs in fp64 on the device; each further pass (`passes` - 1 of them) is
- * the first-order form of a CholeskyQR pass on an almost orthonormal matrix,
- * P <- P (I - up(P^T P - I)) in fp32, which squares the remaining defect ||P^T P - I||.
- * No host synchronisation.  The factor equals the reference's Householder / randomised
- * Cholesky QR result up to column signs (Cholesky's diagonal is positive).
- * info (device, `batch` ints, may be NULL): 0, or 1 + the first column whose pivot was not
- * positive -- the analogue of torch.linalg.cholesky_ex's info; such columns come out as 0. */
+ * Method (passes == 2, the optimizer's case): a blocked CholeskyQR pass (Gram matrix, Cholesky
+ * factorisation, triangular solve) in fp32 -- for a bf16 P with its large products on the bf16 matrix
+ * cores --, then the Gram matrix of the result, which measures the defect ||P^T P - I||_F the pass left.
+ * Where that is at most 2e-3, the first-order form of a second CholeskyQR pass,
+ * P <- P (I - up(P^T P - I)), finishes the matrix; the others (and all matrices with rows < 4 r) take the
+ * same pass in fp64, flagged and selected on the device: no host synchronisation.
+ * passes == 1: the fp64 pass alone; passes == 3: fp64 pass and two polishing passes (each squares the
+ * remaining defect).  The factor equals the reference's Householder / randomised Cholesky QR result up to
+ * column signs (Cholesky's diagonal is positive).
+ * info (device, `batch` ints, may be NULL): 0, or 1 + the first column whose pivot was not positive or
+ * whose result was not a unit vector orthogonal to the others (a pivot at round-off level: P is
+ * numerically rank deficient) -- the analogue of torch.linalg.cholesky_ex's info; such columns come out as 0. */
 int dion_amd_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
                             int* info, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same with the reference's choice of method (`qr_method` of dion/dion_reference.py:733-789, and the
+ * fall-back of 752-758), as far as it has a counterpart on the device.  All three yield the thin-QR factor with a
+ * positive diagonal of R (the reference's Householder-based variants differ from it by column signs):
+ *   DION_AMD_QR_AUTO ("rcqr", what dion_amd_orthonormalize does): a CholeskyQR pass in fp32 first; matrices for
+ *     which it fails or leaves ||P^T P - I||_F > 2e-3 go through the fp64 pass; closed-form polishing pass.
+ *   DION_AMD_QR_FP64 ("qr"): the fp64 pass and the polishing pass for every matrix.
+ *   DION_AMD_QR_CQR  ("cqr"): one CholeskyQR pass in fp32 and nothing else (defect eps32 * cond(P)^2, as in the
+ *     reference); a matrix whose factorisation meets a non-positive pivot falls back to the fp64 pass, on the
+ *     device, as the reference falls back to the randomised method.  Needs passes == 2. */
+#define DION_AMD_QR_AUTO 0
+#define DION_AMD_QR_FP64 1
+#define DION_AMD_QR_CQR 2
+int dion_amd_orthonormalize_method(const void* P, void* out, int dtype, int batch, int rows, int r, int passes,
+                                   int qr_method, int* info, void* workspace, size_t workspace_bytes, void* stream);
 
 size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype);
 
@@ -269,6 +288,15 @@ int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, voi
                        float ef_alpha, float decay, float scaled_lr, float eps, int faithful,
                        int power_iters,
                        int* info, void* workspace, size_t workspace_bytes, void* stream);
+
+/* dion_amd_dion_step with the orthonormaliser's method chosen by the caller (DION_AMD_QR_*): the per-matrix
+ * reference class's `qr_method` (reference dion/dion_reference.py:131-134, 296-299). */
+int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, void* const* Q,
+                          int batch, int m, int n, int r,
+                          int x_dtype, int g_dtype, int m_dtype, int q_dtype,
+                          float ef_alpha, float decay, float scaled_lr, float eps, int faithful,
+                          int power_iters, int qr_method,
+                          int* info, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Measurement hooks (no counterpart in the reference; used by the benchmark only)

@@ -213,3 +213,19 @@ def test_zero_padding_helpers():
     out = [torch.zeros(2, 3), torch.zeros(2, 3)]
     _lib.crop_back(out, big)
     assert torch.equal(out[0], mats[0] + 1) and torch.equal(out[1], mats[1])
+
+
+def test_generate_random_sketch_matrix_shape_and_scale():
+    """reference dion/dion.py:1221-1263: (..., k, m) with k = oversample * r rounded up to a multiple of 128, N(0, 1/k)."""
+    from dion_amd.dion import generate_random_sketch_matrix
+
+    torch.manual_seed(0)
+    S = generate_random_sketch_matrix(torch.zeros(3, 1000, 200), oversample=1.25)
+    assert S.shape == (3, 256, 1000) and S.dtype == torch.float32
+    assert abs(S.std().item() - (1.0 / 256) ** 0.5) <= 2e-4 and abs(S.mean().item()) <= 2e-4
+    S = generate_random_sketch_matrix(torch.zeros(1, 64, 512, dtype=torch.bfloat16), oversample=1.0)
+    assert S.shape == (1, 512, 64) and S.dtype == torch.bfloat16
+    with pytest.raises(AssertionError):
+        generate_random_sketch_matrix(torch.zeros(10, 4))
+    with pytest.raises(TypeError):
+        generate_random_sketch_matrix(torch.zeros(1, 10, 4), shard_mesh_dim=0)

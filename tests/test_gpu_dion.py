@@ -391,3 +391,36 @@ def test_dion_reference_class(dev, qr_method, power_iters):
         DionReference(params, power_iters=0)
     with pytest.raises(ValueError):
         DionReference(params, qr_method="svd")
+
+
+def test_orthonormalize_methods(dev):
+    """The three `qr_method`s of the per-matrix reference class (dion/dion_reference.py:733-789) on the device: "cqr" is
+    one CholeskyQR pass in fp32 and leaves a defect of about eps32 * cond(P)^2 (as the reference's does); "rcqr" and
+    "qr" are orthonormal to round-off; all three are the same thin-QR factor."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(8)
+    rows, r = 2048, 256
+    U, _ = torch.linalg.qr(torch.randn(rows, r, dtype=torch.float64))
+    V, _ = torch.linalg.qr(torch.randn(r, r, dtype=torch.float64))
+    P = ((U * torch.logspace(0, -2.5, r, dtype=torch.float64)) @ V.T).float()     # cond ~ 300
+    Qh, _ = torch.linalg.qr(P.double())
+    eye = torch.eye(r, dtype=torch.float64)
+    res = {}
+    for method in ("rcqr", "qr", "cqr"):
+        Q, info = orthonormalize(P.to(dev), qr_method=method, return_info=True)
+        assert int(info.item()) == 0
+        Qd = Q.double().cpu()
+        res[method] = ((Qd.T @ Qd - eye).norm().item(), rel_fro(_sign_align(Qd, Qh), Qh))
+        print(f"{method}: ||QtQ-I|| = {res[method][0]:.2e}, vs Householder {res[method][1]:.2e}")
+    assert res["rcqr"][0] <= 2e-5 and res["qr"][0] <= 2e-5
+    assert 1e-5 <= res["cqr"][0] <= 5e-2          # eps32 * cond^2 ~ 5e-3: visibly a single fp32 pass
+    assert res["rcqr"][1] <= 5e-4 and res["qr"][1] <= 1e-5 and res["cqr"][1] <= 5e-2
+    # "cqr" on a factor whose Cholesky factorisation fails: the fall-back runs on the device and reports the column
+    Pz = torch.randn(2, 512, 64)
+    Pz[1, :, 17] = 0.0
+    Q, info = orthonormalize(Pz.to(dev), qr_method="cqr", return_info=True)
+    assert info.cpu().tolist() == [0, 18] and torch.isfinite(Q).all() and torch.count_nonzero(Q[1][:, 17]) == 0
+    Q1 = Q[1].double().cpu()
+    keep = [j for j in range(64) if j != 17]
+    assert (Q1[:, keep].T @ Q1[:, keep] - torch.eye(63, dtype=torch.float64)).norm().item() <= ORTH_TOL

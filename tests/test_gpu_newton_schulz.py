@@ -137,3 +137,26 @@ def test_muon_reference_import_path(dev):
     assert torch.equal(keller(G, steps=3), newton_schulz(G, epsilon=1e-7, coeffs=(NS_KELLER_COEFFS,) * 3))
     with pytest.raises(AssertionError):
         keller(G.unsqueeze(0))
+
+
+@pytest.mark.parametrize("shape", [(768, 768), (256, 1024), (1024, 256), (3, 384, 640)])
+def test_frobenius_normalisation_is_bit_exact(dev, shape):
+    """Zero iterations leave X / (||X||_F + eps) (reference dion/muon.py:633-638): same bf16 values as the op-by-op
+    evaluation, division included, whenever the two norms round to the same bf16 number (sums in another order)."""
+    from dion_amd.newton_schulz import newton_schulz
+    from oracle import newton_schulz as ON
+
+    torch.manual_seed(9)
+    G = torch.randn(shape)
+    got = newton_schulz(G.to(dev), coeffs=()).cpu()
+    ref = ON.ns5(G, coeffs=())
+    assert got.dtype == torch.bfloat16 and got.shape == ref.shape
+    mism = (got != ref).float().mean().item()
+    print(f"normalisation {shape}: {mism:.2e} of the elements differ")
+    X = G.bfloat16()
+    n_ref = X.norm(dim=(-2, -1)) + 1e-7
+    n_f64 = (X.double().norm(dim=(-2, -1)).float().bfloat16() + 1e-7)
+    if torch.equal(n_ref, n_f64):
+        assert mism == 0.0
+    else:
+        assert rel_fro(got, ref) <= 8e-3   # the norms themselves differ by one bf16 ulp
