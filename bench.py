@@ -53,7 +53,7 @@ WORKLOADS = {
     "scalar_gpt_small": dict(kind="scalar", shapes=[(50304, 768)] * 2 + [(768,)] * 25, seed=6,
                              desc="Lion on the GPT-small embedding and norms, AdamW on lm_head (50304x768 each), bf16"),
 }
-GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd")
+GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")
 
 
 def make_problem(shapes, seed, dtype, device="cpu"):
@@ -171,12 +171,15 @@ def summarize(name, wl, res):
         # products read and write an m x n matrix; each also moves its m' x r and n' x r factors.
         import math
 
-        rd = upd = 0.0
+        rd = upd = fused = 0.0
         for m, n in shapes:
             r = min(math.ceil(wl["rank_fraction"] * min(m, n)), m, n)   # reference dion/dion.py:672-676
             rd += 2.0 * (m * n + (m + n) * r)
             upd += 2.0 * (2 * m * n + (m + n) * r)
-        for name, nbytes in (("dion_bq", rd), ("dion_btp", rd), ("dion_ef", upd), ("dion_upd", upd)):
+            # error feedback and weight update as one pass: M and X read and written once, P, R and Q_new read
+            fused += 2.0 * (4 * m * n + (max(m, n) + 2 * min(m, n)) * r)
+        for name, nbytes in (("dion_bq", rd), ("dion_btp", rd), ("dion_ef", upd), ("dion_upd", upd),
+                             ("dion_ef_upd", fused)):
             k = out["kernels"].get(name)
             if k and k["ms_per_step"] > 0:
                 rate = nbytes / (k["ms_per_step"] * 1e-3)
@@ -214,7 +217,7 @@ def roofline_of(res, kind, workload=None):
                     frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4), traffic=None, avg_launch_ms=round(ms / n, 5),
                     bytes_per_launch=work / n)
     cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
-                         else ("dion_bq", "dion_btp", "dion_ef", "dion_upd")) if k in prof]
+                         else ("dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")) if k in prof]
     dom = max(cands, key=lambda k: prof[k][1])
     n, ms, work = prof[dom]
     achieved = work / (ms * 1e-3) / 1e12
@@ -289,6 +292,28 @@ def device_info(dev):
     return info
 
 
+def stream_ceiling(dev):
+    """What a plain streaming kernel reaches on this GPU in this run (an in-place scale by torch: one read and one
+    write per element), at the size of one GPT-small bucket and at 2 GiB: the practical ceiling next to the 8 TB/s
+    the HBM-bound passes are priced against."""
+    import torch
+
+    out = {}
+    for label, n in (("108MiB", 48 * 768 * 768 * 2), ("2GiB", 1 << 30)):
+        x = torch.ones(n, dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            x.mul_(1.0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            x.mul_(1.0)
+        e1.record()
+        torch.cuda.synchronize()
+        out[label] = round(4.0 * n / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9, 1)
+        del x
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -342,6 +367,7 @@ def main():
         "roofline": roofline_of(res, wl["kind"], args.workload),
         "device": device_info(dev),
     }
+    out["device"]["streaming_kernel_gbps"] = stream_ceiling(dev)
     out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
     if not args.no_extra:
         extra = {}

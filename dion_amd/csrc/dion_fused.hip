@@ -29,8 +29,7 @@ constexpr int STAGE = 3 * OPND;          // P, R, Qn
 constexpr int RING = 2 * STAGE;
 constexpr int EPITCH = 64 + 4;           // floats per staged accumulator row (16-byte aligned, conflict-free)
 constexpr int ESTG = 32 * EPITCH * 4;    // bytes per wavefront: one 32-row band
-constexpr int SINK = RING + 4 * ESTG;    // 256 bytes per wavefront that nothing reads (see touch_tile)
-constexpr int SMEM = SINK + 8 * 256;
+constexpr int SMEM = RING + 4 * ESTG;
 constexpr int NPIECE = 8;                // epilogue pieces per tile: 2 outputs x 2 bands x 2 halves
 constexpr int PREFETCH = 2;              // pieces whose M / X values are requested ahead
 
@@ -44,7 +43,6 @@ struct FusedArgs {
   int tiles_s, tiles_d;
   int r, ldo, total;
   float ef_alpha, decay, neg_lr;
-  int touch;              // 1: request the M / X lines of a tile at the start of its K loop
 };
 
 struct FTile { int b, ts, td; };
@@ -88,35 +86,6 @@ __device__ __forceinline__ void dma_stage(const FusedArgs& a, const FTile& f, in
   for (int i = 0; i < 4; ++i) dma16(b1, doff + i * dstep, l + OPND + i * 4096);
 #pragma unroll
   for (int i = 0; i < 4; ++i) dma16(b2, doff + i * dstep, l + 2 * OPND + i * 4096);
-}
-
-// Pull the 128 x 128 tiles of M and X that the group will update after this K loop towards the GPU's caches: one
-// dword per 128-byte line, sent to a scratch corner of LDS (a direct-to-LDS load has no register destination that
-// would have to stay reserved while the load is in flight).  The loads stay in flight (2 or 3 per lane); the
-// epilogue's own loads then find the lines in L2 or the Infinity Cache instead of paying the HBM latency between
-// two barriers.  Offsets within a matrix are 32-bit (checked by the launcher).
-__device__ __forceinline__ void touch4(const char* base, unsigned off, unsigned l) {
-  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
-  const unsigned long long u = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(a >> 32)) << 32) |
-                               (unsigned)__builtin_amdgcn_readfirstlane((int)a);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 4\n\tglobal_load_lds_dword %0, %1"
-               :
-               : "v"(off), "s"(u), "s"(__builtin_amdgcn_readfirstlane((int)l))
-               : "memory");
-}
-
-template <bool XF32>
-__device__ __forceinline__ void touch_tile(const char* Mb, const char* Xb, int ldo, int m0, int n0, int gw, int lane,
-                                           unsigned sink) {
-  const int idx = gw * 64 + lane;             // 256 lanes of the group: row idx / 2, half idx % 2
-  const unsigned row_off = (unsigned)(m0 + (idx >> 1)) * (unsigned)ldo + (unsigned)n0;
-  touch4(Mb, row_off * 2u + (idx & 1) * 128u, sink);
-  if (!XF32) {
-    touch4(Xb, row_off * 2u + (idx & 1) * 128u, sink);
-  } else {
-    touch4(Xb, row_off * 4u + (idx & 1) * 256u, sink);
-    touch4(Xb, row_off * 4u + (idx & 1) * 256u + 128u, sink);
-  }
 }
 
 // The two 16-row passes of piece (band, half) of one output: M / X values of the wavefront's 64 x 64 sub-tile.
@@ -272,15 +241,7 @@ __global__ __launch_bounds__(512) void dion_ef_update_kernel(FusedArgs a) {
         DA_MMA(fr1, fr2, fc1, fc2);
         __builtin_amdgcn_sched_barrier(0);
         if (more) {
-          if (kt == 0 && a.touch) {
-            // (issued after the stage's loads: loads return in order, so the stage is in LDS once all but these are back)
-            touch_tile<XF32>(Mb, Xb, a.ldo, (DUAL_A ? mine.td : mine.ts) * FT, (DUAL_A ? mine.ts : mine.td) * FT, gw, lane,
-                             lds_addr(lds) + SINK + wave * 256);
-            if (XF32) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-          } else {
-            dma_wait();
-          }
+          dma_wait();
         } else {
           // the epilogue of this tile starts right after the barrier: request its first M values now (2 loads per
           // piece); loads return in order, so the stage is complete once all but these are back
@@ -374,8 +335,6 @@ int da_dion_ef_update(const void* P, const void* R, const void* Qn, const DaPtrT
   if (total > 0x7fffffffLL) return DA_ERR_LIMIT;
   a.total = (int)total;
   a.ef_alpha = ef_alpha; a.decay = decay; a.neg_lr = -scaled_lr;
-  static const bool no_touch = getenv("DION_AMD_FUSED_NO_TOUCH") != nullptr;
-  a.touch = no_touch ? 0 : 1;
   const bool xf = x_dtype == DA_F32;
   if (transposed) return xf ? launch<true, true>(a, s) : launch<true, false>(a, s);
   return xf ? launch<false, true>(a, s) : launch<false, false>(a, s);
