@@ -34,7 +34,7 @@ template <> __device__ __forceinline__ float rsqrt_seed<float>(float p) { return
 template <typename T>
 __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G, T* __restrict__ Lmat,
                                                         T* __restrict__ Wmat, long long sG, int r, int o, int nb,
-                                                        int below, int* __restrict__ info, const int* gate,
+                                                        int below, int* __restrict__ info, int fresh, const int* gate,
                                                         int gate_want) {
   typedef typename Mfma<T>::acc_t acc_t;
   __shared__ T dinv4[4][4];            // inverse of the current diagonal 4 x 4 factor (lower)
@@ -200,7 +200,8 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
             w[(long long)i * r + j] = j <= i ? y[ii][jj] : T(0);
           }
         }
-      if (tid == 0 && first_bad != 0 && info[b] == 0) info[b] = first_bad;
+      // (`fresh`: the first block column of a factorisation starts the matrix's status word)
+      if (tid == 0 && (fresh || (first_bad != 0 && info[b] == 0))) info[b] = first_bad;
       continue;
     }
     // 64 x 64 x 64 product on the matrix cores: C[m][n] = sum_k opa[k][m] * opb[k][n]
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
 
 template <typename T>
 int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, int* info, int batch, DaGate gate,
-              hipStream_t s) {
+              bool fresh, hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   const int rest = r - o - nb;
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
@@ -289,7 +290,7 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
     configured = true;
   }
   hipLaunchKernelGGL(chol_step_kernel<T>, dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb, below, info,
-                     gate.flags, gate.want);
+                     fresh ? 1 : 0, gate.flags, gate.want);
   return da_launch_status();
 }
 
@@ -297,9 +298,10 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
 
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
                  int batch, DaGate gate, hipStream_t s) {
-  return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, s);
+  return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, false, s);
 }
 int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s) {
-  return chol_step<float>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, s);
+  // the fp32 pass keeps its status in a word of its own, which its first block column initialises
+  return chol_step<float>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, o == 0, s);
 }

@@ -609,11 +609,36 @@ __global__ __launch_bounds__(256) void polish_factor_kernel(const float* __restr
 // U = up(G - I) in bf16 (see polish_factor_kernel): the factor of the correction product P U, which only has
 // to be known to the relative accuracy of bf16 because it is itself of the size of the defect.  Rows and columns
 // of dropped columns (`bad`, may be null) are left out of the correction.
+// `decide` (if given): every workgroup first evaluates the matrix's verdict after the fp32 pass -- the pass failed or
+// left a defect ||P^T P - I||_F above tol (sum of the rows' squared defects, in a fixed order) -- and returns if
+// the matrix goes on to the fp64 pass; the workgroup of row 0 records the verdict for the launches that follow.
+struct FastVerdict {
+  const float* rowdef;
+  const int* info32;
+  int* need;
+  float tol2;
+};
+
 __global__ __launch_bounds__(256) void polish_correction_kernel(const float* __restrict__ G, bf16_t* __restrict__ U,
                                                                 long long rr, int r, const int* __restrict__ bad,
-                                                                const int* gate, int want) {
+                                                                const int* gate, int want, FastVerdict decide) {
   const long long b = blockIdx.y;
-  if (!orth_gate_open(gate, want, (int)b)) return;
+  if (decide.need) {
+    __shared__ float red[256];
+    float s = 0.f;
+    for (int j = threadIdx.x; j < r; j += 256) s += decide.rowdef[b * r + j];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+      __syncthreads();
+    }
+    const bool need = decide.info32[b] != 0 || !(red[0] <= decide.tol2);
+    if (blockIdx.x == 0 && threadIdx.x == 0) decide.need[b] = need ? 1 : 0;
+    if (need) return;
+  } else if (!orth_gate_open(gate, want, (int)b)) {
+    return;
+  }
   const int i = blockIdx.x;
   const float* g = G + b * rr + (long long)i * r;
   bf16_t* u = U + b * rr + (long long)i * r;
@@ -630,10 +655,10 @@ __global__ __launch_bounds__(256) void polish_correction_kernel(const float* __r
 // U built from the Gram matrix G (already computed).  The correction product runs on the bf16 matrix cores (its
 // relative error 2^-8 times the defect E of `in` adds 4e-3 E to the result, next to the pass's own O(E^2)).
 int correction_bf16(const float* in, const bf16_t* in_low, void* out, int out_dtype, const float* G, bf16_t* U,
-                    const int* bad, int batch, int rows, int r, DaGate gate, hipStream_t s) {
+                    const int* bad, int batch, int rows, int r, DaGate gate, FastVerdict decide, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   hipLaunchKernelGGL(polish_correction_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, G, U, rr, r, bad,
-                     gate.flags, gate.want);
+                     gate.flags, gate.want, decide);
   int rc = da_launch_status();
   if (rc) return rc;
   GemmDesc c{};
@@ -919,8 +944,6 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   int rc;
   if (cqr) {
     // ---- "cqr": the fp32 CholeskyQR pass is the result (reference dion/dion_reference.py:752-758)
-    rc = da_fill_int(w.info32, batch, 0, s);
-    if (rc) return rc;
     if (fast16) {
       rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, false, s);
     } else {
@@ -950,8 +973,6 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
     float* G = reinterpret_cast<float*>(w.G);
     float* L = reinterpret_cast<float*>(w.L);
     float* W = reinterpret_cast<float*>(w.W);
-    rc = da_fill_int(w.info32, batch, 0, s);
-    if (rc) return rc;
     if (fast16) {
       rc = fast16_pass(static_cast<const bf16_t*>(P), w, batch, rows, r, r_live, true, s);
       if (rc) return rc;
@@ -967,13 +988,18 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
       rc = gram<float>(w.Pf, G, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, all, s);
       if (rc) return rc;
     }
-    hipLaunchKernelGGL(decide_fast_kernel, dim3((unsigned)batch), dim3(64), 0, s, w.rowdef, w.info32, w.need, r,
-                       FAST_TOL * FAST_TOL);
-    rc = da_launch_status();
-    if (rc) return rc;
     const DaGate good{w.need, 0};
-    if (low) rc = correction_bf16(w.Pf, w.Ph, out, dtype, G, reinterpret_cast<bf16_t*>(L), nullptr, batch, rows, r, good, s);
-    else rc = correction_f32(w.Pf, out, da_store_of(dtype), G, L, nullptr, batch, rows, r, good, s);
+    if (low) {
+      // (the verdict is part of the correction factor's launch)
+      const FastVerdict verdict{w.rowdef, w.info32, w.need, FAST_TOL * FAST_TOL};
+      rc = correction_bf16(w.Pf, w.Ph, out, dtype, G, reinterpret_cast<bf16_t*>(L), nullptr, batch, rows, r, good, verdict, s);
+    } else {
+      hipLaunchKernelGGL(decide_fast_kernel, dim3((unsigned)batch), dim3(64), 0, s, w.rowdef, w.info32, w.need, r,
+                         FAST_TOL * FAST_TOL);
+      rc = da_launch_status();
+      if (rc) return rc;
+      rc = correction_f32(w.Pf, out, da_store_of(dtype), G, L, nullptr, batch, rows, r, good, s);
+    }
     if (rc) return rc;
   }
   // ---- fp64 pass: on the flagged matrices, or on all of them
@@ -1002,7 +1028,8 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
       bad = w.bad;
     }
     if (last && last_low) {
-      rc = correction_bf16(cur, w.Ph, out, dtype, Gf, reinterpret_cast<bf16_t*>(w.L), bad, batch, rows, r, gate, s);
+      rc = correction_bf16(cur, w.Ph, out, dtype, Gf, reinterpret_cast<bf16_t*>(w.L), bad, batch, rows, r, gate,
+                           FastVerdict{nullptr, nullptr, nullptr, 0.f}, s);
     } else {
       // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
       float* other = cur == w.Pf ? reinterpret_cast<float*>(w.P0) : w.Pf;
