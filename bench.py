@@ -314,6 +314,70 @@ def stream_ceiling(dev):
     return out
 
 
+def tile_trace(dev):
+    """Time line of single bf16 GEMM launches (`--tile-trace`): per output tile, when its workgroup started, finished
+    its K loop and finished its epilogue, and on which CU.  Prints one summary line per product: mean duration of the
+    two phases, the gap until the CU's next workgroup, and how many tiles were in their epilogue at 40 instants of the
+    launch (all-or-nothing values mean that the CUs run in lockstep)."""
+    import ctypes
+
+    import numpy as np
+    import torch
+    from dion_amd import _lib
+    from dion_amd.newton_schulz import gemm
+
+    lib = _lib.load()
+    torch.manual_seed(0)
+
+    def report(name, ntiles):
+        ntiles = min(ntiles, 65536)
+        buf = np.zeros((ntiles, 4), dtype=np.uint64)
+        _lib.check(lib.dion_amd_tile_trace_read(ctypes.c_void_p(buf.ctypes.data), ntiles), "dion_amd_tile_trace_read")
+        t0, t1, t2 = (buf[:, i].astype(np.int64) for i in range(3))
+        hw = buf[:, 3]
+        xcc = (hw >> np.uint64(32)).astype(np.int64)
+        h = (hw & np.uint64(0xffffffff)).astype(np.int64)
+        cu = ((xcc * 8 + ((h >> 13) & 7)) * 2 + ((h >> 12) & 1)) * 16 + ((h >> 8) & 15)
+        gaps = []
+        for c in np.unique(cu):
+            idx = np.where(cu == c)[0]
+            o = idx[np.argsort(t0[idx])]
+            gaps += ((t0[o][1:] - t2[o][:-1]) / 100.0).tolist()
+        ts = np.linspace(t0.min(), t2.max(), 40)
+        in_epi = [int(((t1 <= x) & (t2 > x)).sum()) for x in ts]
+        print(json.dumps(dict(
+            product=name, tiles=int(ntiles), cus=int(len(np.unique(cu))), launch_us=round((t2.max() - t0.min()) / 100.0, 1),
+            k_loop_us=round(float(((t1 - t0) / 100.0).mean()), 2), epilogue_us=round(float(((t2 - t1) / 100.0).mean()), 2),
+            gap_us=round(float(np.mean(gaps)), 2) if gaps else None, tiles_in_epilogue_at_40_instants=in_epi)))
+
+    def run(name, fn, ntiles):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        lib.dion_amd_tile_trace_enable(1)
+        fn()
+        lib.dion_amd_tile_trace_enable(0)
+        report(name, ntiles)
+
+    bf = torch.bfloat16
+    # Dion error feedback M <- M - 0.05 P R^T, in place, 4 x (28672 x 8192), rank 512 and rank 64
+    for r in (512, 64):
+        P = (torch.randn(4, 28672, r, device=dev) * 0.03).to(bf)
+        R = (torch.randn(4, 8192, r, device=dev) * 0.03).to(bf)
+        M = torch.randn(4, 28672, 8192, device=dev).to(bf)
+        run(f"M + a P R^T, 4 x 28672x8192, rank {r}", lambda: gemm(P, R, E=M, s0=1.0, s1=-0.05, out=M, faithful=True),
+            4 * 112 * 32)
+        del P, R, M
+    # Newton-Schulz X' = aX + BX: 24 x (768 x 3072) and 4 x (4096 x 4096)
+    for b, m, n in ((24, 768, 3072), (4, 4096, 4096)):
+        X = (torch.randn(b, m, n, device=dev) * 0.03).to(bf)
+        B = (torch.randn(b, m, m, device=dev) * 0.03).to(bf)
+        Y = torch.empty_like(X)
+        run(f"X' = aX + BX, {b} x {m}x{n}", lambda: gemm(B, X, b_kstrided=True, E=X, s0=3.0, s1=1.0, out=Y, faithful=True),
+            b * (m // 256) * (n // 256))
+        del X, B, Y
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -322,6 +386,8 @@ def main():
     ap.add_argument("--workload", default="muon_gpt_small", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tile-trace", action="store_true",
+                    help="instead of a workload: time lines of single bf16 GEMM launches (one JSON line per product)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three plain 512 MiB device copies (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -336,6 +402,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.tile_trace:
+        tile_trace(dev)
+        return
     if args.calibrate_copy:
         src = torch.ones(512 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -58,6 +58,8 @@ _SIGNATURES = {
                                 _vp, _vp, _sz, _vp]),
     "dion_amd_dion_step_qr": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i, _i,
                                    _vp, _vp, _sz, _vp]),
+    "dion_amd_tile_trace_enable": (_i, [_i]),
+    "dion_amd_tile_trace_read": (_i, [_vp, _i]),
     "dion_amd_profile_enable": (_i, [_i]),
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),

@@ -39,6 +39,7 @@ struct GemmArgs {
   GemmDesc d[DA_MAX_GROUPS];
   int start[DA_MAX_GROUPS + 1];
   int n;
+  int trace;   // 1: every workgroup records its time stamps (measurement hook)
 };
 
 template <int BT_, int WGM_, int WGN_>
@@ -326,8 +327,17 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
 //   !FULL: bounds-checked 16-byte loads into registers (out-of-range chunks zero filled),
 //     written to LDS after the stage's MFMAs.
 // ---------------------------------------------------------------------------------------
+// Measurement hook: per workgroup (tile) of the last traced launch, the 100 MHz counter at the start, after the
+// K loop and at the end, and the hardware id of the CU it ran on.
+constexpr int DA_TRACE_TILES = 65536;
+__device__ unsigned long long da_tile_trace[4 * DA_TRACE_TILES];
+bool g_tile_trace = false;
+
 template <typename C, bool A_KS, bool B_KS, bool SYM, bool FULL>
 __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
+  const bool trace = args.trace && blockIdx.x < DA_TRACE_TILES;
+  unsigned long long ts0 = 0, ts1 = 0;
+  if (trace) ts0 = __builtin_amdgcn_s_memrealtime();
   // which of the grouped products this workgroup belongs to (groups own contiguous block ranges)
   int grp = 0;
 #pragma unroll
@@ -493,7 +503,18 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
 #undef DA_MMA
 #undef DA_FREAD2
 #undef DA_MMA2
+  if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
   epilogue<C, SYM, FULL>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
+  if (trace) {
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned hw = __builtin_amdgcn_s_getreg(4 | (31 << 11));      // HW_ID: CU, shader array, shader engine
+      const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11));     // XCC_ID
+      unsigned long long* t = da_tile_trace + 4 * (size_t)blockIdx.x;
+      t[0] = ts0; t[1] = ts1; t[2] = __builtin_amdgcn_s_memrealtime();
+      t[3] = ((unsigned long long)xcc << 32) | hw;
+    }
+  }
 }
 
 // Bytes from the first to the last element a workgroup reads of one operand (BT rows, all of K).
@@ -535,6 +556,7 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   }
   GemmArgs args{};
   args.n = n;
+  args.trace = g_tile_trace ? 1 : 0;
   const bool full = all_interior(d, n, BT);
   long long blocks = 0;
   for (int g = 0; g < n; ++g) {
@@ -648,3 +670,15 @@ int da_gemm_bf16_plan(const GemmDesc& d) {
 }
 
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) { return da_gemm_bf16_grouped(&d, 1, stream); }
+
+// ---- measurement hook: time stamps of the tiles of the bf16 GEMM launches (see include/dion_amd.h)
+extern "C" int dion_amd_tile_trace_enable(int on) {
+  g_tile_trace = on != 0;
+  return DA_OK;
+}
+extern "C" int dion_amd_tile_trace_read(void* dst, int tiles) {
+  if (!dst || tiles <= 0 || tiles > DA_TRACE_TILES) return DA_ERR_ARG;
+  DA_HIP_CHECK(hipDeviceSynchronize());
+  DA_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(da_tile_trace), (size_t)tiles * 4 * sizeof(unsigned long long)));
+  return DA_OK;
+}

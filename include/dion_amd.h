@@ -327,6 +327,14 @@ int dion_amd_profile_reset(void);
  * summed work. */
 int dion_amd_profile_read(int kind, long long* launches, double* total_ms, double* total_work);
 
+/* Time line of a bf16 GEMM launch (no counterpart in the reference; used by the benchmark only).  While enabled,
+ * every workgroup of a bf16 GEMM launch -- one output tile each -- records three readings of the GPU's 100 MHz
+ * counter (start, end of its K loop, end of its epilogue) and the hardware id of the CU it ran on.  `read` waits
+ * for the device and copies the records of the first `tiles` workgroups (at most 65536) of the most recent such
+ * launch to HOST memory: four 64-bit words per tile (t_start, t_k_loop_done, t_end, (XCC id << 32) | HW_ID). */
+int dion_amd_tile_trace_enable(int on);
+int dion_amd_tile_trace_read(void* host_dst, int tiles);
+
 #ifdef __cplusplus
 }
 #endif
