@@ -189,20 +189,16 @@ def summarize(name, wl, res):
 
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.000 and
 # WRITE_SIZE x 1.000, in KiB, the factors being what the same counters read for a plain 512 MiB copy);
-# the runs used the workload named in the key with three 512 MiB copies first (--calibrate-copy).  Keyed by (workload, kernel).
+# the runs used the workload named in the key with three 512 MiB copies first (--calibrate-copy).  Keyed by
+# (workload, kernel); measured 2026-11-25 on the kernels of this revision (profiles/*_hbm_traffic.md hold the runs);
+# a kernel kind that is not listed has not been measured since it last changed and reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("muon_gpt_small", "ns_axpy"): 683634 * 1024,
-    # error feedback / weight update of the Llama-3-70B layer: mean over the 2-matrix and the 1-matrix bucket
-    ("dion_llama70b_layer", "dion_ef"): 1896506 * 1024,
-    ("dion_llama70b_layer", "dion_upd"): 1896506 * 1024,
+    ("muon_gpt_small", "ns_axpy"): 676308 * 1024,
     # one Llama-3-8B layer: the grouped X' = aX + BX launch over its four buckets
-    ("muon_llama8b_layer", "ns_axpy"): 3443298 * 1024,
-    # Dion on the GPT-small matrices (every bucket's error-feedback / update launch moves the same bytes)
-    ("dion_gpt_small_r025", "dion_ef"): 138008 * 1024,
-    ("dion_gpt_small_r025", "dion_upd"): 138008 * 1024,
-    ("dion_gpt_small_r025", "dion_btp"): 85195 * 1024,   # mean of the 48-matrix launch and the two K-sliced ones
-    ("dion_gpt_small_r1", "dion_ef"): 219424 * 1024,
-    ("dion_gpt_small_r1", "dion_upd"): 219424 * 1024,
+    ("muon_llama8b_layer", "ns_axpy"): 3435386 * 1024,
+    # error feedback + weight update in one pass: mean over the buckets of the workload
+    ("dion_gpt_small_r025", "dion_ef_upd"): 277687 * 1024,
+    ("dion_llama70b_layer", "dion_ef_upd"): 4027315 * 1024,
 }
 
 
