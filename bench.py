@@ -327,7 +327,7 @@ def tile_trace(dev):
 
     def report(name, ntiles):
         ntiles = min(ntiles, 65536)
-        buf = np.zeros((ntiles, 4), dtype=np.uint64)
+        buf = np.zeros((ntiles, 6), dtype=np.uint64)
         _lib.check(lib.dion_amd_tile_trace_read(ctypes.c_void_p(buf.ctypes.data), ntiles), "dion_amd_tile_trace_read")
         t0, t1, t2 = (buf[:, i].astype(np.int64) for i in range(3))
         hw = buf[:, 3]
@@ -339,12 +339,16 @@ def tile_trace(dev):
             idx = np.where(cu == c)[0]
             o = idx[np.argsort(t0[idx])]
             gaps += ((t0[o][1:] - t2[o][:-1]) / 100.0).tolist()
+        mhz = (buf[:, 5].astype(np.int64) - buf[:, 4].astype(np.int64)) / np.maximum(t2 - t0, 1) * 100.0
         ts = np.linspace(t0.min(), t2.max(), 40)
         in_epi = [int(((t1 <= x) & (t2 > x)).sum()) for x in ts]
         print(json.dumps(dict(
             product=name, tiles=int(ntiles), cus=int(len(np.unique(cu))), launch_us=round((t2.max() - t0.min()) / 100.0, 1),
             k_loop_us=round(float(((t1 - t0) / 100.0).mean()), 2), epilogue_us=round(float(((t2 - t1) / 100.0).mean()), 2),
-            gap_us=round(float(np.mean(gaps)), 2) if gaps else None, tiles_in_epilogue_at_40_instants=in_epi)))
+            gap_us=round(float(np.mean(gaps)), 2) if gaps else None,
+            shader_clock_mhz=dict(mean=round(float(mhz.mean())), p10=round(float(np.percentile(mhz, 10))),
+                                  p90=round(float(np.percentile(mhz, 90)))),
+            tiles_in_epilogue_at_40_instants=in_epi)))
 
     def run(name, fn, ntiles):
         for _ in range(3):

@@ -328,16 +328,20 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
 //     written to LDS after the stage's MFMAs.
 // ---------------------------------------------------------------------------------------
 // Measurement hook: per workgroup (tile) of the last traced launch, the 100 MHz counter at the start, after the
-// K loop and at the end, and the hardware id of the CU it ran on.
+// K loop and at the end, the hardware id of the CU it ran on, and the shader-clock counter at the start and the end.
 constexpr int DA_TRACE_TILES = 65536;
-__device__ unsigned long long da_tile_trace[4 * DA_TRACE_TILES];
+constexpr int DA_TRACE_WORDS = 6;
+__device__ unsigned long long da_tile_trace[DA_TRACE_WORDS * DA_TRACE_TILES];
 bool g_tile_trace = false;
 
 template <typename C, bool A_KS, bool B_KS, bool SYM, bool FULL>
 __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const bool trace = args.trace && blockIdx.x < DA_TRACE_TILES;
-  unsigned long long ts0 = 0, ts1 = 0;
-  if (trace) ts0 = __builtin_amdgcn_s_memrealtime();
+  unsigned long long ts0 = 0, ts1 = 0, tc0 = 0;
+  if (trace) {
+    ts0 = __builtin_amdgcn_s_memrealtime();
+    tc0 = __builtin_amdgcn_s_memtime();
+  }
   // which of the grouped products this workgroup belongs to (groups own contiguous block ranges)
   int grp = 0;
 #pragma unroll
@@ -510,9 +514,10 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
     if (tid == 0) {
       const unsigned hw = __builtin_amdgcn_s_getreg(4 | (31 << 11));      // HW_ID: CU, shader array, shader engine
       const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11));     // XCC_ID
-      unsigned long long* t = da_tile_trace + 4 * (size_t)blockIdx.x;
+      unsigned long long* t = da_tile_trace + DA_TRACE_WORDS * (size_t)blockIdx.x;
       t[0] = ts0; t[1] = ts1; t[2] = __builtin_amdgcn_s_memrealtime();
       t[3] = ((unsigned long long)xcc << 32) | hw;
+      t[4] = tc0; t[5] = __builtin_amdgcn_s_memtime();
     }
   }
 }
@@ -679,6 +684,6 @@ extern "C" int dion_amd_tile_trace_enable(int on) {
 extern "C" int dion_amd_tile_trace_read(void* dst, int tiles) {
   if (!dst || tiles <= 0 || tiles > DA_TRACE_TILES) return DA_ERR_ARG;
   DA_HIP_CHECK(hipDeviceSynchronize());
-  DA_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(da_tile_trace), (size_t)tiles * 4 * sizeof(unsigned long long)));
+  DA_HIP_CHECK(hipMemcpyFromSymbol(dst, HIP_SYMBOL(da_tile_trace), (size_t)tiles * DA_TRACE_WORDS * sizeof(unsigned long long)));
   return DA_OK;
 }

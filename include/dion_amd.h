@@ -331,7 +331,9 @@ int dion_amd_profile_read(int kind, long long* launches, double* total_ms, doubl
  * every workgroup of a bf16 GEMM launch -- one output tile each -- records three readings of the GPU's 100 MHz
  * counter (start, end of its K loop, end of its epilogue) and the hardware id of the CU it ran on.  `read` waits
  * for the device and copies the records of the first `tiles` workgroups (at most 65536) of the most recent such
- * launch to HOST memory: four 64-bit words per tile (t_start, t_k_loop_done, t_end, (XCC id << 32) | HW_ID). */
+ * launch to HOST memory: six 64-bit words per tile (t_start, t_k_loop_done, t_end, (XCC id << 32) | HW_ID, and the
+ * shader-clock counter at the start and at the end: its difference over that of the 100 MHz counter is the clock the
+ * CU ran at). */
 int dion_amd_tile_trace_enable(int on);
 int dion_amd_tile_trace_read(void* host_dst, int tiles);
 
