@@ -1,7 +1,7 @@
-// One block-column step of the batched, blocked fp64 Cholesky used by the CholeskyQR
+// One block-column step of the batched, blocked Cholesky (fp64 or fp32) used by the CholeskyQR
 // orthonormalisation, fused into a single launch: every workgroup factors the (<= 64) x (<= 64)
-// diagonal block in registers and inverts the triangular factor (redundantly -- the factor is the
-// serial part; a few workgroups per matrix repeat it rather than wait for one), then they share
+// diagonal block on the matrix cores and inverts the triangular factor (redundantly -- the factor is
+// the serial part; a few workgroups per matrix repeat it rather than wait for one), then they share
 // the 64 x 64 pieces of what depends on it:
 //   role 0            : stores L_jj and its inverse D_j (the diagonal block of W, see below),
 //   roles 1 .. below  : one 64-row tile of the panel   L[i, j] = A[i, j] D_j^T,
@@ -21,15 +21,23 @@ namespace {
 constexpr int NB = DA_CHOL_NB;
 constexpr int LP = NB + 1;   // LDS pitch of the operand tiles (doubles): transposed stores stay nearly conflict-free
 
-// 256 threads as a 16 x 16 grid; thread (bi, bj) keeps the 4 x 4 blocks of the working matrix
-// and of the inverse-in-progress at block position (bi, bj) in registers.  Right-looking with
-// 4-wide block columns: per block step the diagonal owner factors and inverts its 4 x 4 block
-// in registers, the column owners form their L blocks (A_ic * L_cc^-T), the row owners of the
-// inverse form X_c = L_cc^-1 * Y_c, both are published through LDS, and every thread applies
-// the two rank-4 updates.  Two barriers per 4 columns.
+// The 64 x 64 diagonal block S and the inverse-in-progress Y live in matrix-core accumulators: wavefront w of
+// the four holds tile row w (rows 16 w .. 16 w + 15) of both as 16 x 16 tiles.  Right-looking with 4-wide block
+// columns.  Per block step every wavefront reads the published block column of S (64 x 4) and row block of Y
+// (4 x 64) from LDS and repeats the serial part on its own SIMD instead of waiting for one owner: the 4 x 4
+// diagonal factor (the same instructions in every lane), then lane = row forms its row of the L block column
+// by forward substitution and lane = column its column of X = L_cc^-1 Y_c (rows 4 cb .. 4 cb + 3 of the inverse,
+// final after this).  Both go to LDS as MFMA operands, the two rank-4 updates S -= L_c L_c^T, Y -= L_c X are
+// v_mfma_*_16x16x4 instructions on the wavefront's own tiles, and the wavefronts publish the next block column / row
+// block.  One workgroup barrier per 4 columns; the published blocks and the operands are double-buffered.
 template <typename T> __device__ __forceinline__ T rsqrt_seed(T p);
 template <> __device__ __forceinline__ double rsqrt_seed<double>(double p) { return __builtin_amdgcn_rsq(p); }
 template <> __device__ __forceinline__ float rsqrt_seed<float>(float p) { return __builtin_amdgcn_rsqf(p); }
+// a positive normal number (false for NaN, infinities, zero and denormals, which the estimate does not handle)
+__device__ __forceinline__ bool usable_pivot(double p) { return __builtin_amdgcn_class(p, 0x100); }
+__device__ __forceinline__ bool usable_pivot(float p) { return __builtin_amdgcn_classf(p, 0x100); }
+
+template <typename T> struct Quad { T v[4]; };
 
 template <typename T>
 __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G, T* __restrict__ Lmat,
@@ -37,201 +45,191 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
                                                         int below, int* __restrict__ info, int fresh, const int* gate,
                                                         int gate_want) {
   typedef typename Mfma<T>::acc_t acc_t;
-  __shared__ T dinv4[4][4];            // inverse of the current diagonal 4 x 4 factor (lower)
-  __shared__ T lcol[NB][4];            // rows > 4cb+3: L[i][4cb .. 4cb+3]
-  __shared__ T xrow[4][NB];            // rows 4cb .. 4cb+3 of L^-1
-  __shared__ int first_bad;
+  typedef Quad<T> quad_t;
+  __shared__ __attribute__((aligned(16))) T scol[2][4][NB];     // published block column of S: [column][row]
+  __shared__ __attribute__((aligned(16))) quad_t yrow[2][NB];   // published row block of Y:    [column] -> 4 rows
+  __shared__ __attribute__((aligned(16))) quad_t lops[2][NB];   // L block column as MFMA operand (0 in finished rows)
+  __shared__ __attribute__((aligned(16))) quad_t xops[2][NB];   // X, [column] -> 4 rows
   extern __shared__ __attribute__((aligned(16))) unsigned char opnd_raw[];   // two k-major 64 x 64 operand tiles
   T* const opnd = reinterpret_cast<T*>(opnd_raw);
   const int b = blockIdx.y, tid = threadIdx.x;
   if (gate && (gate[b] != 0) != (gate_want != 0)) return;
-  const int bi = tid >> 4, bj = tid & 15;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lc = lane & 15, lg = lane >> 4;
+  // D_j transposed (dT[k][x] = D[x][k], zero outside the nb x nb lower triangle) and, for role 0, L_jj (in `op`)
+  T* const dT = opnd;
+  T* const op = opnd + NB * LP;
   const T* g = G + (long long)b * sG + (long long)o * r + o;
-  T a[4][4], y[4][4];
+  acc_t S[4], Y[4];
 #pragma unroll
-  for (int ii = 0; ii < 4; ++ii)
+  for (int tj = 0; tj < 4; ++tj)
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const int i = bi * 4 + ii, j = bj * 4 + jj;
+    for (int v = 0; v < 4; ++v) {
+      const int i = wave * 16 + Mfma<T>::row(v, lane), j = tj * 16 + lc;
       // identity padding beyond nb keeps the padded part inert
-      a[ii][jj] = (i < nb && j < nb) ? g[(long long)i * r + j] : (i == j ? T(1) : T(0));
-      y[ii][jj] = (i == j) ? T(1) : T(0);
+      S[tj][v] = (tj <= wave && i < nb && j < nb) ? g[(long long)i * r + j] : (i == j ? T(1) : T(0));
+      Y[tj][v] = (i == j) ? T(1) : T(0);
     }
-  if (tid == 0) first_bad = 0;
+  // The workgroups of one matrix share its roles round-robin (role 0: L_jj, D_j and the status word; 1 .. below:
+  // panel tiles; the rest: W tiles).  The operand tile of a product does not depend on this step's factor: it is
+  // requested now, 16 elements per thread, and the next one while the previous product runs.
+  const int nroles = 1 + below + o / NB;
+  T pre[16];
+  auto fetch = [&](int role) {
+    const bool panel = role <= below;
+    const int row0 = o + nb + (role - 1) * NB;
+    const int rows_ok = r - row0 < NB ? r - row0 : NB;
+    const T* src = panel ? G + (long long)b * sG + (long long)row0 * r + o
+                         : Lmat + (long long)b * sG + (long long)o * r + (role - 1 - below) * NB;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int e = tid + 256 * t, hi = e >> 6, lo = e & 63;
+      const bool in = panel ? (hi < rows_ok && lo < nb) : hi < nb;
+      pre[t] = in ? src[(long long)hi * r + lo] : T(0);
+    }
+  };
+  int role = blockIdx.x == 0 ? (int)gridDim.x : (int)blockIdx.x;   // this workgroup's first product
+  if (role < nroles) fetch(role);
+  if (tid < 2 * NB) {
+    // columns right of the diagonal tile of a row block are never published: they read as zero
+    quad_t z;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) z.v[k] = T(0);
+    yrow[tid >> 6][tid & 63] = z;
+  }
   __syncthreads();
 
-  for (int cb = 0; cb < NB / 4; ++cb) {
-    if (bi == cb && bj == cb) {
-      // unblocked Cholesky of the 4 x 4 diagonal block and its inverse, in registers
-      T di[4];
+  // Block q (columns / rows 4 q .. 4 q + 3) of the current S and Y into buffer `buf`.
+  auto publish = [&](int q, int buf) {
+    const int tq = q >> 2, qq = q & 3;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const T p = a[c][c];
-        const bool ok = p > T(0) && p < (sizeof(T) == 8 ? T(1.0e300) : T(1.0e37));  // false for NaN as well
-        // 1/sqrt(p) from the hardware estimate plus two Newton steps (full fp64 accuracy), then
-        // sqrt(p) = p * rsqrt(p): this thread is the critical path of the whole factorisation and
-        // the library sqrt + divide are four times as long
-        T rs = ok ? rsqrt_seed<T>(p) : T(0);
-        rs = rs * (T(1.5) - T(0.5) * p * rs * rs);
-        rs = rs * (T(1.5) - T(0.5) * p * rs * rs);
-        const T d = ok ? p * rs : T(0);
-        di[c] = ok ? rs : T(0);
-        if (!ok && cb * 4 + c < nb && first_bad == 0) first_bad = o + cb * 4 + c + 1;
-        a[c][c] = d;
+    for (int tj = 0; tj < 4; ++tj) {
+      if (tj == tq && tj <= wave && (lc >> 2) == qq) {
 #pragma unroll
-        for (int i = c + 1; i < 4; ++i) a[i][c] *= di[c];
-#pragma unroll
-        for (int i = c + 1; i < 4; ++i)
-#pragma unroll
-          for (int j = c + 1; j <= i; ++j) a[i][j] -= a[i][c] * a[j][c];
+        for (int v = 0; v < 4; ++v) scol[buf][lc & 3][wave * 16 + Mfma<T>::row(v, lane)] = S[tj][v];
       }
-      T inv[4][4];
+      if (wave == tq && tj <= wave) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          T t = (i == j) ? T(1) : T(0);
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            if (k >= j && k < i) t -= a[i][k] * inv[k][j];
-          inv[i][j] = j <= i ? t * di[i] : T(0);
+        for (int v = 0; v < 4; ++v) {
+          const int rr = Mfma<T>::row(v, lane);
+          if ((rr >> 2) == qq) yrow[buf][tj * 16 + lc].v[rr & 3] = Y[tj][v];
         }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (j > i) a[i][j] = T(0);
-          dinv4[i][j] = inv[i][j];
-        }
-    }
-    __syncthreads();
-    if (bj == cb && bi > cb) {
-      // L_ic = A_ic * L_cc^-T : row ii of the block times the transposed inverse
-      T l[4][4];
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          T t = T(0);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) t += a[ii][k] * dinv4[jj][k];
-          l[ii][jj] = t;
-        }
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          a[ii][jj] = l[ii][jj];
-          lcol[bi * 4 + ii][jj] = l[ii][jj];
-        }
-    }
-    if (bi == cb) {
-      // X_c = L_cc^-1 * Y_c  (rows 4cb .. 4cb+3 of the inverse are final after this)
-      T x[4][4];
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          T t = T(0);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) t += dinv4[ii][k] * y[k][jj];
-          x[ii][jj] = t;
-        }
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          y[ii][jj] = x[ii][jj];
-          xrow[ii][bj * 4 + jj] = x[ii][jj];
-        }
-    }
-    __syncthreads();
-    if (bi > cb) {
-      T li[4][4];
-#pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) li[ii][k] = lcol[bi * 4 + ii][k];
-      if (bj > cb) {
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const T lj = lcol[bj * 4 + jj][k];
-#pragma unroll
-            for (int ii = 0; ii < 4; ++ii) a[ii][jj] -= li[ii][k] * lj;
-          }
       }
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const T xk = xrow[k][bj * 4 + jj];
-#pragma unroll
-          for (int ii = 0; ii < 4; ++ii) y[ii][jj] -= li[ii][k] * xk;
-        }
     }
-  }
+  };
+  publish(0, 0);
+  __syncthreads();
 
-  // D_j (zero outside its nb x nb lower triangle), transposed: dT[k][x] = D[x][k]
-  T* dT = opnd;
-  T* op = opnd + NB * LP;
+  constexpr int NEWTON = sizeof(T) == 8 ? 2 : 0;   // the hardware estimate is good to 1 ulp in fp32, ~2^-27 in fp64
+  int bad = 0;                                     // first failed pivot (every lane computes the same)
+  for (int cb = 0; cb < NB / 4; ++cb) {
+    const int buf = cb & 1, k0 = cb * 4;
+    quad_t sv;                             // lane = row: S[lane][k0 ..]
 #pragma unroll
-  for (int ii = 0; ii < 4; ++ii)
+    for (int k = 0; k < 4; ++k) sv.v[k] = scol[buf][k][lane];
+    const quad_t yv = yrow[buf][lane];     // lane = column: Y[k0 ..][lane]
+    T a[4][4];
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const int i = bi * 4 + ii, j = bj * 4 + jj;
-      dT[j * LP + i] = (i < nb && j <= i) ? y[ii][jj] : T(0);
-    }
-  const int lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-  const int nroles = 1 + below + o / NB;
-  // the workgroups of one matrix share its roles round-robin
-  for (int role = blockIdx.x; role < nroles; role += gridDim.x) {
-    if (role == 0) {
-      T* l = Lmat + (long long)b * sG + (long long)o * r + o;
-      T* w = Wmat + (long long)b * sG + (long long)o * r + o;
+      const quad_t d = *reinterpret_cast<const quad_t*>(&scol[buf][jj][k0]);   // the same address in every lane
 #pragma unroll
-      for (int ii = 0; ii < 4; ++ii)
+      for (int ii = 0; ii < 4; ++ii) a[ii][jj] = d.v[ii];
+    }
+    // unblocked Cholesky of the 4 x 4 diagonal block: a[i][j], j < i becomes L_cc, di[] the inverse diagonal
+    T di[4];
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const int i = bi * 4 + ii, j = bj * 4 + jj;
-          if (i < nb && j < nb) {
-            l[(long long)i * r + j] = j <= i ? a[ii][jj] : T(0);
-            w[(long long)i * r + j] = j <= i ? y[ii][jj] : T(0);
-          }
-        }
-      // (`fresh`: the first block column of a factorisation starts the matrix's status word)
-      if (tid == 0 && (fresh || (first_bad != 0 && info[b] == 0))) info[b] = first_bad;
-      continue;
+    for (int c = 0; c < 4; ++c) {
+      const T p = a[c][c];
+      const bool ok = usable_pivot(p);
+      // 1/sqrt(p) from the hardware estimate plus Newton steps: this chain is the critical path of the whole
+      // factorisation and the library sqrt + divide are four times as long
+      T rs = ok ? rsqrt_seed<T>(p) : T(0);
+#pragma unroll
+      for (int it = 0; it < NEWTON; ++it) rs = rs * (T(1.5) - T(0.5) * p * rs * rs);
+      di[c] = ok ? rs : T(0);
+      bad = (!ok && bad == 0 && k0 + c < nb) ? o + k0 + c + 1 : bad;
+#pragma unroll
+      for (int i = c + 1; i < 4; ++i) a[i][c] *= di[c];
+#pragma unroll
+      for (int i = c + 1; i < 4; ++i)
+#pragma unroll
+        for (int j = c + 1; j <= i; ++j) a[i][j] -= a[i][c] * a[j][c];
     }
-    // 64 x 64 x 64 product on the matrix cores: C[m][n] = sum_k opa[k][m] * opb[k][n]
-    const bool panel = role <= below;
-    int row0, col0, rows_ok, cols_ok;
-    __syncthreads();   // `op` may still be read by the previous role's MFMAs; dT is complete after it
-    if (panel) {
-      // L[i, j] = A[i, j] D^T :  opa[k][m] = A[row0 + m][o + k],  opb = dT
-      row0 = o + nb + (role - 1) * NB;
-      col0 = o;
-      rows_ok = r - row0 < NB ? r - row0 : NB;
-      cols_ok = nb;
-      const T* src = G + (long long)b * sG + (long long)row0 * r + o;
-      for (int e = tid; e < NB * NB; e += 256) {
-        const int m = e >> 6, k = e & 63;
-        op[k * LP + m] = (m < rows_ok && k < nb) ? src[(long long)m * r + k] : T(0);
+    // row `lane` of the L block column and column `lane` of X, by forward substitution with L_cc
+    T l[4], x[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      T tl = sv.v[k], tx = yv.v[k];
+#pragma unroll
+      for (int m = 0; m < k; ++m) {
+        tl -= l[m] * a[k][m];
+        tx -= a[k][m] * x[m];
       }
-    } else {
-      // W[j, c] = -D L[j, c] :  opa = dT,  opb[k][n] = L[o + k][col0 + n]
-      row0 = o;
-      col0 = (role - 1 - below) * NB;   // col0 + 64 <= o
-      rows_ok = nb;
-      cols_ok = NB;
-      const T* src = Lmat + (long long)b * sG + (long long)o * r + col0;
-      for (int e = tid; e < NB * NB; e += 256) {
-        const int k = e >> 6, n = e & 63;
-        op[k * LP + n] = k < nb ? src[(long long)k * r + n] : T(0);
+      l[k] = tl * di[k];
+      x[k] = tx * di[k];
+    }
+    quad_t lo, xo, lfin;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      lo.v[k] = lane > k0 + 3 ? l[k] : T(0);               // finished rows take no part in the updates
+      lfin.v[k] = lane >= k0 + k ? l[k] : T(0);            // L_jj: zero above the diagonal
+      xo.v[k] = (lane <= k0 + k && k0 + k < nb) ? x[k] : T(0);
+    }
+    lops[buf][lane] = lo;     // (every wavefront writes the same values; each reads back after its own writes)
+    xops[buf][lane] = xo;
+    if (wave == (cb & 3)) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) dT[lane * LP + k0 + k] = lane < nb ? xo.v[k] : T(0);
+      if (blockIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) op[lane * LP + k0 + k] = lfin.v[k];
       }
     }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (wave * 16 + 15 > k0 + 3) {
+      const T aop = -lops[buf][wave * 16 + lc].v[lg];
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        if (tj <= wave && tj * 16 + 15 > k0 + 3) S[tj] = Mfma<T>::mma(aop, lops[buf][tj * 16 + lc].v[lg], S[tj]);
+        if (tj <= wave && tj * 16 <= k0 + 3) Y[tj] = Mfma<T>::mma(aop, xops[buf][tj * 16 + lc].v[lg], Y[tj]);
+      }
+    }
+    if (cb + 1 < NB / 4) publish(cb + 1, buf ^ 1);
     __syncthreads();
+  }
+
+  // ---- the 64 x 64 x 64 products that depend on the factor: C[m][n] = sum_k opa[k][m] * opb[k][n]
+  if (blockIdx.x == 0) {
+    T* l = Lmat + (long long)b * sG + (long long)o * r + o;
+    T* w = Wmat + (long long)b * sG + (long long)o * r + o;
+    for (int e = tid; e < NB * NB; e += 256) {
+      const int i = e >> 6, j = e & 63;
+      if (i < nb && j < nb) {
+        l[(long long)i * r + j] = op[i * LP + j];
+        w[(long long)i * r + j] = dT[j * LP + i];
+      }
+    }
+    // (`fresh`: the first block column of a factorisation starts the matrix's status word)
+    if (tid == 0 && (fresh || (bad != 0 && info[b] == 0))) info[b] = bad;
+  }
+  const int wm = wave >> 1, wn = wave & 1;
+  while (role < nroles) {
+    const bool panel = role <= below;
+    __syncthreads();   // `op` may still be read (role 0's copy, the previous product's MFMAs)
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int e = tid + 256 * t;
+      // panel: opa[k][m] = A[row0 + m][o + k] (element e = (m, k));  W: opb[k][n] = L[o + k][col0 + n] (e = (k, n))
+      op[panel ? (e & 63) * LP + (e >> 6) : (e >> 6) * LP + (e & 63)] = pre[t];
+    }
+    const int next = role + (int)gridDim.x;
+    if (next < nroles) fetch(next);   // in flight during this role's product
+    __syncthreads();
+    const int row0 = panel ? o + nb + (role - 1) * NB : o;
+    const int col0 = panel ? o : (role - 1 - below) * NB;   // (W: col0 + 64 <= o)
+    const int rows_ok = panel ? (r - row0 < NB ? r - row0 : NB) : nb;
+    const int cols_ok = panel ? nb : NB;
     const T* opa = panel ? op : dT;
     const T* opb = panel ? dT : op;
     acc_t acc[2][2];
@@ -265,6 +263,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
           const int n = wn * 32 + j * 16 + (lane & 15);
           if (m < rows_ok && n < cols_ok) dst[(long long)m * r + n] = sign * acc[i][j][v];
         }
+    role = next;
   }
 }
 
