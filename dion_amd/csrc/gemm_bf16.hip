@@ -73,7 +73,10 @@ struct StageAddr {
   long long gstep, tstep;   // per chunk and per stage, in elements
   int l, lstep;
   int row, col;             // first chunk's (row within tile, k offset) resp. (k row, row offset)
-  __device__ __forceinline__ StageAddr(const bf16_t* base, int ld, int row0, int tid) {
+  // `dim`: extent of the operand in the tile's row direction (M or N); the direct-to-LDS addresses of a
+  // k-strided operand keep their 16-byte chunks inside it (an edge tile then fetches a neighbouring chunk for the
+  // columns it does not own: finite values that the bounds-checked epilogue never stores).
+  __device__ __forceinline__ StageAddr(const bf16_t* base, int ld, int row0, int tid, int dim) {
     constexpr int NW = C::NT / 64;
     const int lane = tid & 63, wave = tid >> 6;
     if (!KS) {
@@ -100,7 +103,9 @@ struct StageAddr {
       lstep = (C::NT / CPR) * (C::BT * 2);                 // NT / CPR = 16: swizzle term unchanged
       const int drow = wave * RPB + lane / CPR;
       dbase = reinterpret_cast<const char*>(base + row0);
-      doff = (unsigned)(drow * ld + ks_swizzle(lane % CPR, drow) * 8) * 2u;
+      int dcol = ks_swizzle(lane % CPR, drow) * 8;
+      if (row0 + dcol > dim - 8) dcol = dim - 8 - row0;
+      doff = (unsigned)(drow * ld + dcol) * 2u;
       dstep = (unsigned)(NW * RPB * ld) * 2u;              // NW * RPB = 16
     }
   }
@@ -320,22 +325,27 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
 }
 
 // ---------------------------------------------------------------------------------------
-// One kernel, two K loops.
-//   FULL: every tile is interior (M, N multiples of BT, K a multiple of 64).  Stages are
+// One kernel, two K loops, three modes.
+//   DA_LOOP_INTERIOR: every tile is interior (M, N multiples of BT, K a multiple of 64).  Stages are
 //     fetched with direct-to-LDS loads issued one stage ahead; the only wait is the
-//     vmcnt(0) in front of the per-stage barrier.
-//   !FULL: bounds-checked 16-byte loads into registers (out-of-range chunks zero filled),
+//     vmcnt(0) in front of the per-stage barrier.  No bounds checks anywhere.
+//   DA_LOOP_EDGE: the same K loop for products whose ragged dimension belongs to a k-strided operand (its chunks
+//     are kept inside the matrix) and whose other operand has whole tiles; the epilogue checks bounds.  Dion's
+//     rank-r products at a rank that is not a multiple of the tile edge (r = 192).
+//   DA_LOOP_CHECKED: bounds-checked 16-byte loads into registers (out-of-range chunks zero filled),
 //     written to LDS after the stage's MFMAs.
 // ---------------------------------------------------------------------------------------
 // Measurement hook: per workgroup (tile) of the last traced launch, the 100 MHz counter at the start, after the
 // K loop and at the end, the hardware id of the CU it ran on, and the shader-clock counter at the start and the end.
+constexpr int DA_LOOP_CHECKED = 0, DA_LOOP_INTERIOR = 1, DA_LOOP_EDGE = 2;
 constexpr int DA_TRACE_TILES = 65536;
 constexpr int DA_TRACE_WORDS = 6;
 __device__ unsigned long long da_tile_trace[DA_TRACE_WORDS * DA_TRACE_TILES];
 bool g_tile_trace = false;
 
-template <typename C, bool A_KS, bool B_KS, bool SYM, bool FULL>
+template <typename C, bool A_KS, bool B_KS, bool SYM, int MODE>
 __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
+  constexpr bool FULL = MODE != DA_LOOP_CHECKED;   // the direct-to-LDS K loop
   const bool trace = args.trace && blockIdx.x < DA_TRACE_TILES;
   unsigned long long ts0 = 0, ts1 = 0, tc0 = 0;
   if (trace) {
@@ -374,8 +384,8 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  StageAddr<C, A_KS> sa(A, d.lda, m0, tid);
-  StageAddr<C, B_KS> sb(B, d.ldb, n0, tid);
+  StageAddr<C, A_KS> sa(A, d.lda, m0, tid, d.M);
+  StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
   const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
   const int KT = (d.K + BK - 1) / BK;
   bf16x8_t fa[TMI], fb[TNJ];
@@ -508,7 +518,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
 #undef DA_FREAD2
 #undef DA_MMA2
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
-  epilogue<C, SYM, FULL>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
+  epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
   if (trace) {
     __syncthreads();
     if (tid == 0) {
@@ -539,6 +549,22 @@ bool all_interior(const GemmDesc* d, int n, int bt) {
   return true;
 }
 
+// Whether the direct-to-LDS K loop can run with edge tiles: K whole stages, every k-contiguous operand in whole
+// tiles (its rows are fetched unconditionally), every k-strided operand at least one chunk wide (multiples of 8
+// by the alignment contract), 32-bit offsets as above.
+bool edge_loop_ok(const GemmDesc* d, int n, int bt) {
+  for (int g = 0; g < n; ++g) {
+    if (d[g].K % BK) return false;
+    if (!d[g].a_kstrided && d[g].M % bt) return false;
+    if (!d[g].b_kstrided && d[g].N % bt) return false;
+    if (d[g].a_kstrided && (d[g].M < 8 || d[g].M % 8)) return false;
+    if (d[g].b_kstrided && (d[g].N < 8 || d[g].N % 8)) return false;
+    if (da_tile_span_bytes(d[g].a_kstrided != 0, bt, d[g].lda, d[g].K) >= (1LL << 32)) return false;
+    if (da_tile_span_bytes(d[g].b_kstrided != 0, bt, d[g].ldb, d[g].K) >= (1LL << 32)) return false;
+  }
+  return true;
+}
+
 template <typename C>
 long long tiles_of(const GemmDesc& d) {
   const long long tm = (d.M + C::BT - 1) / C::BT, tn = (d.N + C::BT - 1) / C::BT;
@@ -551,11 +577,13 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   constexpr int stage2 = 2 * (Tile<BT, A_KS>::bytes + Tile<BT, B_KS>::bytes);
   constexpr int epi = (C::NT / 64) * 32 * (C::WCOLS + 4) * 4;
   constexpr int smem = stage2 > epi ? stage2 : epi;
-  auto kfull = gemm_bf16_kernel<C, A_KS, B_KS, SYM, true>;
-  auto kgen = gemm_bf16_kernel<C, A_KS, B_KS, SYM, false>;
+  auto kfull = gemm_bf16_kernel<C, A_KS, B_KS, SYM, DA_LOOP_INTERIOR>;
+  auto kedge = gemm_bf16_kernel<C, A_KS, B_KS, SYM, (A_KS || B_KS) && !SYM ? DA_LOOP_EDGE : DA_LOOP_CHECKED>;
+  auto kgen = gemm_bf16_kernel<C, A_KS, B_KS, SYM, DA_LOOP_CHECKED>;
   static bool configured = false;  // benign race: the attribute calls are idempotent
   if (!configured) {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kfull), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kedge), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kgen), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
@@ -563,6 +591,8 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   args.n = n;
   args.trace = g_tile_trace ? 1 : 0;
   const bool full = all_interior(d, n, BT);
+  static const bool edge_on = [] { const char* e = getenv("DION_AMD_NO_EDGE_LOOP"); return !(e && atoi(e)); }();
+  const bool edge = !full && edge_on && (A_KS || B_KS) && !SYM && edge_loop_ok(d, n, BT);
   long long blocks = 0;
   for (int g = 0; g < n; ++g) {
     args.d[g] = d[g];
@@ -573,7 +603,7 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
     if (blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
   }
   for (int g = n; g <= DA_MAX_GROUPS; ++g) args.start[g] = (int)blocks;
-  hipLaunchKernelGGL(full ? kfull : kgen, dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
+  hipLaunchKernelGGL(full ? kfull : (edge ? kedge : kgen), dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
   return da_launch_status();
 }
 
@@ -638,7 +668,10 @@ int choose_tile(const GemmDesc* d, int n) {
   if (forced == 128 || forced == 256) return forced;
   bool fits_big = true;
   for (int g = 0; g < n; ++g) fits_big = fits_big && d[g].M >= 256 && d[g].N >= 256;
-  const bool full_big = all_interior(d, n, 256), full_small = all_interior(d, n, 128);
+  // (either form of the direct-to-LDS K loop counts)
+  const bool may_edge = !d[0].symmetric && (d[0].a_kstrided || d[0].b_kstrided);
+  const bool full_big = all_interior(d, n, 256) || (may_edge && edge_loop_ok(d, n, 256));
+  const bool full_small = all_interior(d, n, 128) || (may_edge && edge_loop_ok(d, n, 128));
   const double cost_big = launch_cost<Big>(d, n, 256, 4.0);
   const double cost_small = launch_cost<Small>(d, n, 512, 3.0);
   return fits_big && (full_big || !full_small) && cost_big <= cost_small ? 256 : 128;
