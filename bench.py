@@ -199,6 +199,14 @@ MEASURED_TRAFFIC_BYTES = {
     # error feedback + weight update in one pass: mean over the buckets of the workload
     ("dion_gpt_small_r025", "dion_ef_upd"): 277687 * 1024,
     ("dion_llama70b_layer", "dion_ef_upd"): 4027315 * 1024,
+    # mean over the three buckets (two launches of the non-transposed kernel, one of the transposed one)
+    ("dion_gpt_small_r1", "dion_ef_upd"): 446671 * 1024,
+    # the 16-matrix and the 8-matrix bucket: mean of the two launches
+    ("dion_llama70b_mlp", "dion_ef_upd"): 33113826 * 1024,
+    # the grouped X' = aX + BX launch over all 224 matrices
+    ("muon_llama8b", "ns_axpy"): 105288904 * 1024,
+    # mean of the AdamW launch (lm_head) and the Lion launch (embedding, norms)
+    ("scalar_gpt_small", "scalar_opt"): 452944 * 1024,
 }
 
 
@@ -210,7 +218,8 @@ def roofline_of(res, kind, workload=None):
         n, ms, work = prof["scalar_opt"]
         achieved = work / (ms * 1e-3) / 1e9
         return dict(bound="hbm", kernel="scalar_opt", achieved=round(achieved, 1), peak=PEAK_HBM_BPS / 1e9, unit="GB/s",
-                    frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4), traffic=None, avg_launch_ms=round(ms / n, 5),
+                    frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4),
+                    traffic=MEASURED_TRAFFIC_BYTES.get((workload, "scalar_opt")), avg_launch_ms=round(ms / n, 5),
                     bytes_per_launch=work / n)
     cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
                          else ("dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")) if k in prof]
