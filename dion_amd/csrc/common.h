@@ -101,6 +101,12 @@ struct GemmDesc {
   // (gate[b] != 0) == (gate_want != 0); the workgroups of the other matrices return at once.
   const int* gate;
   int gate_want;
+  // bf16 kernel, optional.  a_kwrap > 0: A has only a_kwrap columns (a multiple of 64 that divides K; A k-contiguous)
+  // and is read again from its first column every a_kwrap steps of k: C = A [B_0; B_1; ...] = sum_i A B_i in one
+  // accumulation.  c2_off != 0 (bf16 C, plain store): the part of s1 * acc that the bf16 value stored in C leaves
+  // over is rounded to bf16 as well and stored c2_off elements after C -- the result as two bf16 matrices.
+  int a_kwrap;
+  long long c2_off;
 };
 
 // Epilogues.  With `faithful` set the rounding points of the reference's separate

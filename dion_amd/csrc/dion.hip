@@ -784,17 +784,19 @@ __global__ __launch_bounds__(256) void eye_kernel(float* __restrict__ T, long lo
 }
 
 // Tcat[k][0 .. r) = bf16(T[k][:]), Tcat[k][r .. 2r) = bf16(T[k][:] - that): T to 16 bits as two bf16 factors
+// `stacked`: [T_hi; T_lo] (2r x r) instead of [T_hi | T_lo] (r x 2r)
 __global__ __launch_bounds__(256) void split_factor_kernel(const float* __restrict__ T, bf16_t* __restrict__ Tcat,
-                                                           long long rr, int r) {
+                                                           long long rr, int r, int stacked) {
   const long long b = blockIdx.y;
   const int k = blockIdx.x;
   const float* t = T + b * rr + (long long)k * r;
-  bf16_t* o = Tcat + b * 2 * rr + (long long)k * 2 * r;
+  bf16_t* o = Tcat + b * 2 * rr + (long long)k * (stacked ? r : 2 * r);
+  const long long lo = stacked ? rr : r;
   for (int j = threadIdx.x; j < r; j += 256) {
     const float v = t[j];
     const bf16_t h = f2bf(v);
     o[j] = h;
-    o[r + j] = f2bf(v - bf2f(h));
+    o[lo + j] = f2bf(v - bf2f(h));
   }
 }
 
@@ -871,9 +873,26 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
     rc = da_gemm_f32s(a, s);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(split_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, Tcat, rr, r);
+  // P1 = P T_hi + P T_lo.  With whole 64-deep stages (r a multiple of 64) it is ONE accumulation over the stacked
+  // factor [T_hi; T_lo], P read twice along k, and the product leaves the kernel as h + l; otherwise the two
+  // products go side by side into an fp32 matrix and a pass of its own adds and splits them.
+  const bool stacked = r % 64 == 0 && rows % 128 == 0 && (Lo - w.Ph) % 8 == 0;
+  hipLaunchKernelGGL(split_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, Tcat, rr, r,
+                     stacked ? 1 : 0);
   rc = da_launch_status();
   if (rc) return rc;
+  if (stacked) {
+    GemmDesc c{};
+    c.batch = batch;
+    c.A = P; c.sA = pr; c.lda = r; c.a_kstrided = 0; c.a_kwrap = r;
+    c.B = Tcat; c.sB = 2 * rr; c.ldb = r; c.b_kstrided = 1;
+    c.C = w.Ph; c.sC = pr; c.ldc = r; c.c_dtype = DA_BF16; c.c2_off = Lo - w.Ph;
+    c.M = rows; c.N = r; c.K = 2 * r;
+    c.epilogue = DA_EPI_STORE; c.s1 = 1.f; c.faithful = 0;
+    rc = da_gemm_bf16(c, s);
+    if (rc || !second_gram) return rc;
+    return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, s);
+  }
   GemmDesc c{};
   c.batch = batch;
   c.A = P; c.sA = pr; c.lda = r; c.a_kstrided = 0;

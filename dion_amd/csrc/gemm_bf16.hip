@@ -171,6 +171,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
   // the descriptor lives in the kernel-argument segment: fields read inside the band loop would be fetched
   // again after every store (scalar load + a full wait in the middle of the band), so they are copied first
   const float s0 = d.s0, s1 = d.s1;
+  const long long c2 = (!HAS_E && !FAITHFUL && !SYM && !CF32) ? d.c2_off * 2 : 0;   // bytes to the second output
   const int dM = d.M, dN = d.N;
   const long long ldc = d.ldc, lde = d.lde;
   const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
@@ -261,6 +262,13 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
             }
           }
           stg16(Cp, pk);
+          if (!HAS_E && !FAITHFUL && !SYM && c2) {
+            // what the stored bf16 leaves of s1 * acc, as a second bf16 matrix
+            u32x4_t lo;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) lo[q] = cvt_pk_bf16(s1 * v[2 * q] - lo_f(pk[q]), s1 * v[2 * q + 1] - hi_f(pk[q]));
+            stg16(Cp + c2, lo);
+          }
         }
         if (SYM && mirror) {  // keep the final values for the transposed store
           *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
@@ -426,9 +434,11 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
         dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
     koff_a += (unsigned)(sa.tstep * 2);                                                            \
+    if (koff_a == wrap_a) koff_a = 0;                                                              \
     koff_b += (unsigned)(sb.tstep * 2);                                                            \
   } while (0)
     unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB: checked by the launcher)
+    const unsigned wrap_a = (unsigned)d.a_kwrap * 2u;   // A read again from its first column (0: never, koff_a > 0 here)
     DA_DMA(lds);
     dma_wait();
     __syncthreads();
@@ -603,6 +613,9 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
     if (blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
   }
   for (int g = n; g <= DA_MAX_GROUPS; ++g) args.start[g] = (int)blocks;
+  if (!full && !edge)   // the bounds-checked K loop walks A with a pointer: no wrap-around there
+    for (int g = 0; g < n; ++g)
+      if (d[g].a_kwrap) return DA_ERR_ARG;
   hipLaunchKernelGGL(full ? kfull : (edge ? kedge : kgen), dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
   return da_launch_status();
 }
@@ -629,6 +642,9 @@ int check_desc(const GemmDesc& d) {
   if (d.a_kstrided && (d.M & 7)) return DA_ERR_ALIGN;
   if (((uintptr_t)d.A | (uintptr_t)d.B | (uintptr_t)d.C | (uintptr_t)d.E) & 15) return DA_ERR_ALIGN;
   if (d.symmetric && (d.M != d.N || d.a_kstrided || d.b_kstrided)) return DA_ERR_ARG;
+  if (d.a_kwrap && (d.a_kwrap < 0 || d.a_kstrided || d.a_kwrap % BK || d.K % d.a_kwrap)) return DA_ERR_ARG;
+  if (d.c2_off && (d.c_dtype != DA_BF16 || d.epilogue != DA_EPI_STORE || d.faithful || d.symmetric || (d.c2_off & 7)))
+    return DA_ERR_ARG;
   return DA_OK;
 }
 
