@@ -683,7 +683,9 @@ int choose_tile(const GemmDesc* d, int n) {
   static const int forced = [] { const char* e = getenv("DION_AMD_TILE"); return e ? atoi(e) : 0; }();
   if (forced == 128 || forced == 256) return forced;
   bool fits_big = true;
-  for (int g = 0; g < n; ++g) fits_big = fits_big && d[g].M >= 256 && d[g].N >= 256;
+  // (a 192-wide product fills three quarters of a 256-tile: still cheaper than one and a half 128-tiles -- rank-192
+  // P = BQ 34 -> 29.5 us per GPT-small bucket)
+  for (int g = 0; g < n; ++g) fits_big = fits_big && d[g].M >= 192 && d[g].N >= 192;
   // (either form of the direct-to-LDS K loop counts)
   const bool may_edge = !d[0].symmetric && (d[0].a_kstrided || d[0].b_kstrided);
   const bool full_big = all_interior(d, n, 256) || (may_edge && edge_loop_ok(d, n, 256));
