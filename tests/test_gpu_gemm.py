@@ -70,7 +70,10 @@ def test_ns_line_2(dev, m, dtype):
 @pytest.mark.parametrize("a_ks", [False, True])
 @pytest.mark.parametrize("b_ks", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M,N,K,batch", [(256, 384, 512, 1), (136, 72, 200, 3), (1024, 1024, 192, 2)])
+@pytest.mark.parametrize("M,N,K,batch", [(256, 384, 512, 1), (136, 72, 200, 3), (1024, 1024, 192, 2),
+                                         # ragged dimension on a k-strided operand, everything else in whole tiles:
+                                         # the direct-to-LDS K loop with a bounds-checked epilogue (Dion's rank 192)
+                                         (768, 192, 768, 2), (192, 192, 1024, 2), (200, 320, 128, 1)])
 def test_gemm_layouts(dev, a_ks, b_ks, dtype, M, N, K, batch):
     from dion_amd.newton_schulz import gemm
 
