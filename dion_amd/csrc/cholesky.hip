@@ -8,6 +8,9 @@
 //   roles above that  : one 64-column tile of          W[j, c] = -D_j L[j, c],  c < j,
 // where W is the block-lower-triangular matrix with which the triangular solve of P becomes one
 // in-place GEMM per block column:  P[:, j] <- P[:, 0 .. j] W[j, 0 .. j]^T.
+// A second form of the kernel (INV) writes, instead of W's row block, row block j of T = L^-1 itself:
+//   T[j, j] = D_j,   T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c],   c < j,
+// for the callers that need the inverse factor as a matrix.
 // No host synchronisation: a failed pivot is recorded in a device-side info word, mirroring
 // torch.linalg.cholesky_ex's `info`.
 #include "gemm_f64.h"
@@ -39,11 +42,11 @@ __device__ __forceinline__ bool usable_pivot(float p) { return __builtin_amdgcn_
 
 template <typename T> struct Quad { T v[4]; };
 
-template <typename T>
+template <typename T, bool INV>
 __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G, T* __restrict__ Lmat,
-                                                        T* __restrict__ Wmat, long long sG, int r, int o, int nb,
-                                                        int below, int* __restrict__ info, int fresh, const int* gate,
-                                                        int gate_want) {
+                                                        T* __restrict__ Wmat, T* __restrict__ Tmat, long long sG, int r,
+                                                        int o, int nb, int below, int* __restrict__ info, int fresh,
+                                                        const int* gate, int gate_want) {
   typedef typename Mfma<T>::acc_t acc_t;
   typedef Quad<T> quad_t;
   __shared__ __attribute__((aligned(16))) T scol[2][4][NB];     // published block column of S: [column][row]
@@ -74,22 +77,66 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   // panel tiles; the rest: W tiles).  The operand tile of a product does not depend on this step's factor: it is
   // requested now, 16 elements per thread, and the next one while the previous product runs.
   const int nroles = 1 + below + o / NB;
-  T pre[16];
-  auto fetch = [&](int role) {
-    const bool panel = role <= below;
-    const int row0 = o + nb + (role - 1) * NB;
-    const int rows_ok = r - row0 < NB ? r - row0 : NB;
-    const T* src = panel ? G + (long long)b * sG + (long long)row0 * r + o
-                         : Lmat + (long long)b * sG + (long long)o * r + (role - 1 - below) * NB;
+  // A 64 x 64 tile in registers: thread t holds the four elements (row (t >> 4) + 16 q, columns 4 (t & 15) .. + 3),
+  // q = 0 .. 3 (named vectors, not an array: an array that one loop iteration writes and the next one reads ends up
+  // in scratch memory).
+  typedef T tv4_t __attribute__((ext_vector_type(4)));
+  tv4_t pa0, pa1, pa2, pa3, pb0, pb1, pb2, pb3;
+  const int trow = tid >> 4, tcol = (tid & 15) * 4;
+  // rows < rows_ok, columns < cols_ok of the tile at src (row pitch r); the rest reads as zero
+  auto load_quad = [&](const T* src, int q, int rows_ok, int cols_ok) __attribute__((always_inline)) {
+    const int row = trow + 16 * q;
+    tv4_t v = {T(0), T(0), T(0), T(0)};
+    if (row < rows_ok) {
+      const T* p = src + (long long)row * r + tcol;
+      if (tcol + 4 <= cols_ok) {
+        v = *reinterpret_cast<const tv4_t*>(p);
+      } else {
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int e = tid + 256 * t, hi = e >> 6, lo = e & 63;
-      const bool in = panel ? (hi < rows_ok && lo < nb) : hi < nb;
-      pre[t] = in ? src[(long long)hi * r + lo] : T(0);
+        for (int i = 0; i < 4; ++i) v[i] = tcol + i < cols_ok ? p[i] : T(0);
+      }
+    }
+    return v;
+  };
+#define DA_LOAD_TILE(v0, v1, v2, v3, src, rows_ok, cols_ok)                                  \
+  do {                                                                                       \
+    v0 = load_quad((src), 0, (rows_ok), (cols_ok)); v1 = load_quad((src), 1, (rows_ok), (cols_ok)); \
+    v2 = load_quad((src), 2, (rows_ok), (cols_ok)); v3 = load_quad((src), 3, (rows_ok), (cols_ok)); \
+  } while (0)
+  // quad -> LDS tile, k-major with pitch LP: transposed (element (row, col) at [col][row]) or as it is
+  auto store_quad = [&](const tv4_t v, int q, T* dst, bool transposed) __attribute__((always_inline)) {
+    const int row = trow + 16 * q;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (transposed) dst[(tcol + i) * LP + row] = v[i];
+      else dst[row * LP + tcol + i] = v[i];
     }
   };
+#define DA_STORE_TILE(v0, v1, v2, v3, dst, transposed)                                       \
+  do {                                                                                       \
+    store_quad(v0, 0, (dst), (transposed)); store_quad(v1, 1, (dst), (transposed));          \
+    store_quad(v2, 2, (dst), (transposed)); store_quad(v3, 3, (dst), (transposed));          \
+  } while (0)
+  // operand tiles of one term of T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]  (j = o / 64): L[j, k] and T[k, c]
+  auto fetch_t = [&](int c, int k) __attribute__((always_inline)) {
+    if (!INV) return;
+    DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)o * r + (long long)k * NB, nb, NB);
+    DA_LOAD_TILE(pb0, pb1, pb2, pb3, Tmat + (long long)b * sG + (long long)k * NB * r + (long long)c * NB, NB, NB);
+  };
+  auto fetch = [&](int role) __attribute__((always_inline)) {
+    const bool panel = role <= below;
+    if (INV && !panel) {
+      fetch_t(role - 1 - below, role - 1 - below);
+      return;
+    }
+    const int row0 = o + nb + (role - 1) * NB;
+    if (panel) DA_LOAD_TILE(pa0, pa1, pa2, pa3, G + (long long)b * sG + (long long)row0 * r + o, r - row0 < NB ? r - row0 : NB, nb);
+    else DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)o * r + (role - 1 - below) * NB, nb, NB);
+  };
   int role = blockIdx.x == 0 ? (int)gridDim.x : (int)blockIdx.x;   // this workgroup's first product
-  if (role < nroles) fetch(role);
+  // (the two tiles of a T role would stay in registers through the whole factor loop: those are requested after it)
+  const bool early = role < nroles && !(INV && role > below);
+  if (early) fetch(role);
   if (tid < 2 * NB) {
     // columns right of the diagonal tile of a row block are never published: they read as zero
     quad_t z;
@@ -202,7 +249,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   // ---- the 64 x 64 x 64 products that depend on the factor: C[m][n] = sum_k opa[k][m] * opb[k][n]
   if (blockIdx.x == 0) {
     T* l = Lmat + (long long)b * sG + (long long)o * r + o;
-    T* w = Wmat + (long long)b * sG + (long long)o * r + o;
+    T* w = (INV ? Tmat : Wmat) + (long long)b * sG + (long long)o * r + o;
     for (int e = tid; e < NB * NB; e += 256) {
       const int i = e >> 6, j = e & 63;
       if (i < nb && j < nb) {
@@ -214,15 +261,84 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
     if (tid == 0 && (fresh || (bad != 0 && info[b] == 0))) info[b] = bad;
   }
   const int wm = wave >> 1, wn = wave & 1;
+  // acc += opa^T opb over one 64-deep tile pair (k-major tiles of pitch LP)
+  auto mma_tile = [&](const T* opa, const T* opb, acc_t (&acc)[2][2]) __attribute__((always_inline)) {
+#pragma unroll 4
+    for (int ks = 0; ks < NB / 4; ++ks) {
+      const int k = ks * 4 + (lane >> 4);
+      T af[2], bfv[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = opa[k * LP + wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bfv[j] = opb[k * LP + wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
+    }
+  };
+  if (role < nroles && !early) fetch(role);
   while (role < nroles) {
     const bool panel = role <= below;
-    __syncthreads();   // `op` may still be read (role 0's copy, the previous product's MFMAs)
+    if (INV && !panel) {
+      // Row block j of T = L^-1, column block c:  T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]
+      const int c = role - 1 - below, jb = o / NB;
+      acc_t acc[2][2];
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int e = tid + 256 * t;
-      // panel: opa[k][m] = A[row0 + m][o + k] (element e = (m, k));  W: opb[k][n] = L[o + k][col0 + n] (e = (k, n))
-      op[panel ? (e & 63) * LP + (e >> 6) : (e >> 6) * LP + (e & 63)] = pre[t];
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+      const int next = role + (int)gridDim.x;
+      // the tile pairs alternate between two LDS buffers: pair k + 1 is requested before the product of pair k and
+      // written after it (the registers live within one iteration)
+      auto put = [&](int buf) __attribute__((always_inline)) {
+        T* pa = op + buf * (2 * NB * LP);
+        DA_STORE_TILE(pa0, pa1, pa2, pa3, pa, true);              // opa[kk][m] = L[o + m][64 k + kk]
+        DA_STORE_TILE(pb0, pb1, pb2, pb3, pa + NB * LP, false);  // opb[kk][n] = T[64 k + kk][64 c + n]
+      };
+      __syncthreads();   // the buffers may still be read (role 0's copy, a previous product)
+      put(0);
+      for (int k = c; k < jb; ++k) {
+        const int buf = (k - c) & 1;
+        if (k + 1 < jb) fetch_t(c, k + 1);
+        __syncthreads();                                     // pair k is in place; the other buffer is free
+        mma_tile(op + buf * (2 * NB * LP), op + buf * (2 * NB * LP) + NB * LP, acc);
+        if (k + 1 < jb) put(buf ^ 1);
+      }
+      if (next < nroles) fetch(next);
+      T* const op2 = op + NB * LP;   // (buffer 0's second tile: free after the barrier below)
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            op2[(wm * 32 + i * 16 + Mfma<T>::row(v, lane)) * LP + wn * 32 + j * 16 + (lane & 15)] = acc[i][j][v];
+      __syncthreads();
+      acc_t res[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) res[i][j] = acc_t{0, 0, 0, 0};
+      mma_tile(dT, op2, res);
+      T* dst = Tmat + (long long)b * sG + (long long)o * r + (long long)c * NB;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int m = wm * 32 + i * 16 + Mfma<T>::row(v, lane);
+            const int n = wn * 32 + j * 16 + (lane & 15);
+            if (m < nb) dst[(long long)m * r + n] = -res[i][j][v];
+          }
+      role = next;
+      continue;
     }
+    __syncthreads();   // `op` may still be read (role 0's copy, the previous product's MFMAs)
+    // panel: opa[k][m] = A[row0 + m][o + k];  W: opb[k][n] = L[o + k][col0 + n]
+    DA_STORE_TILE(pa0, pa1, pa2, pa3, op, panel);
     const int next = role + (int)gridDim.x;
     if (next < nroles) fetch(next);   // in flight during this role's product
     __syncthreads();
@@ -237,20 +353,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
-#pragma unroll 4
-    for (int ks = 0; ks < NB / 4; ++ks) {
-      const int k = ks * 4 + (lane >> 4);
-      T af[2], bfv[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) af[i] = opa[k * LP + wm * 32 + i * 16 + (lane & 15)];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) bfv[j] = opb[k * LP + wn * 32 + j * 16 + (lane & 15)];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
-    }
+    mma_tile(opa, opb, acc);
     T* dst = (panel ? Lmat : Wmat) + (long long)b * sG + (long long)row0 * r + col0;
     const T sign = panel ? T(1) : T(-1);
 #pragma unroll
@@ -267,14 +370,17 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   }
 }
 
-template <typename T>
-int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, int* info, int batch, DaGate gate,
-              bool fresh, hipStream_t s) {
+#undef DA_LOAD_TILE
+#undef DA_STORE_TILE
+
+template <typename T, bool INV>
+int chol_step(const T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int nb, int* info, int batch,
+              DaGate gate, bool fresh, hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   const int rest = r - o - nb;
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
   const int below = (rest + NB - 1) / NB;
-  const int smem = 2 * NB * LP * (int)sizeof(T);
+  const int smem = (INV ? 5 : 2) * NB * LP * (int)sizeof(T);
   // workgroups per matrix: as many as fit one per CU over the batch (the factorisation every workgroup repeats is
   // bound by fp64 instruction issue, which two workgroups on a CU would share: 384 instead of 256 in flight cost
   // 3 % of the orthonormaliser on a 48-matrix bucket), never more than there are roles
@@ -284,11 +390,11 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
   if (per > nroles) per = nroles;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
-    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(chol_step_kernel<T>),
+    DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(chol_step_kernel<T, INV>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  hipLaunchKernelGGL(chol_step_kernel<T>, dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, sG, r, o, nb, below, info,
+  hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r, o, nb, below, info,
                      fresh ? 1 : 0, gate.flags, gate.want);
   return da_launch_status();
 }
@@ -297,10 +403,14 @@ int chol_step(const T* G, T* Lmat, T* Wmat, long long sG, int r, int o, int nb, 
 
 int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
                  int batch, DaGate gate, hipStream_t s) {
-  return chol_step<double>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, false, s);
+  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, s);
 }
 int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s) {
   // the fp32 pass keeps its status in a word of its own, which its first block column initialises
-  return chol_step<float>(G, Lmat, Wmat, sG, r, o, nb, info, batch, gate, o == 0, s);
+  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, s);
+}
+int da_chol_step_f32_inv(const float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
+                         int batch, DaGate gate, hipStream_t s) {
+  return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, s);
 }

@@ -784,16 +784,17 @@ __global__ __launch_bounds__(256) void eye_kernel(float* __restrict__ T, long lo
 }
 
 // Tcat[k][0 .. r) = bf16(T[k][:]), Tcat[k][r .. 2r) = bf16(T[k][:] - that): T to 16 bits as two bf16 factors
-// `stacked`: [T_hi; T_lo] (2r x r) instead of [T_hi | T_lo] (r x 2r)
+// `stacked`: [T_hi; T_lo] (2r x r) instead of [T_hi | T_lo] (r x 2r).  `lower`: the source holds L^-1 (lower
+// triangular, blocks of 64 above the diagonal never written) and T = R^-1 is its transpose.
 __global__ __launch_bounds__(256) void split_factor_kernel(const float* __restrict__ T, bf16_t* __restrict__ Tcat,
-                                                           long long rr, int r, int stacked) {
+                                                           long long rr, int r, int stacked, int lower) {
   const long long b = blockIdx.y;
   const int k = blockIdx.x;
   const float* t = T + b * rr + (long long)k * r;
   bf16_t* o = Tcat + b * 2 * rr + (long long)k * (stacked ? r : 2 * r);
   const long long lo = stacked ? rr : r;
   for (int j = threadIdx.x; j < r; j += 256) {
-    const float v = t[j];
+    const float v = !lower ? t[j] : ((j >> 6) >= (k >> 6) ? T[b * rr + (long long)j * r + k] : 0.f);
     const bf16_t h = f2bf(v);
     o[j] = h;
     o[lo + j] = f2bf(v - bf2f(h));
@@ -843,9 +844,12 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   float* part = reinterpret_cast<float*>(w.part);
   int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, s);
   if (rc) return rc;
+  // (the steps write the rows of L^-1 themselves: no W, no recurrence on the identity afterwards)
+  static const bool inv_rows = [] { const char* e = getenv("DION_AMD_ORTH_NO_INV"); return !(e && atoi(e)); }();
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-    rc = da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s);
+    rc = inv_rows ? da_chol_step_f32_inv(G, L, T, rr, r, o, nb, w.info32, batch, all, s)
+                  : da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s);
     if (rc) return rc;
     if (rest <= 0) break;
     Gemm32Desc u{};
@@ -858,10 +862,12 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
     rc = da_gemm_f32s(u, s);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(eye_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, rr, r);
-  rc = da_launch_status();
-  if (rc) return rc;
-  for (int j = 0; j < nblk; ++j) {
+  if (!inv_rows) {
+    hipLaunchKernelGGL(eye_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, rr, r);
+    rc = da_launch_status();
+    if (rc) return rc;
+  }
+  for (int j = 0; j < nblk && !inv_rows; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB;
     Gemm32Desc a{};
     a.batch = batch;
@@ -878,7 +884,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   // products go side by side into an fp32 matrix and a pass of its own adds and splits them.
   const bool stacked = r % 64 == 0 && rows % 128 == 0 && (Lo - w.Ph) % 8 == 0;
   hipLaunchKernelGGL(split_factor_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, T, Tcat, rr, r,
-                     stacked ? 1 : 0);
+                     stacked ? 1 : 0, inv_rows ? 1 : 0);
   rc = da_launch_status();
   if (rc) return rc;
   if (stacked) {

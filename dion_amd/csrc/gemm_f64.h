@@ -79,6 +79,11 @@ int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int 
                  int batch, DaGate gate, hipStream_t s);
 int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s);
+// The same step, but instead of the row block of W it writes row block j of T = L^-1 itself into Tmat (lower
+// triangular, row-major): T[j, j] = D_j and T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c] for c < j, from the
+// rows of T that the earlier steps left.  After the last step Tmat holds L^-1 (blocks above the diagonal untouched).
+int da_chol_step_f32_inv(const float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
+                         int batch, DaGate gate, hipStream_t s);
 
 #define DA_CHOL_NB 64
 
