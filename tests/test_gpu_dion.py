@@ -41,6 +41,29 @@ def test_orthonormalize(dev, rows, r, dtype):
     assert (torch.diagonal(Rm) > 0).all()
 
 
+@pytest.mark.parametrize("rows,r,batch", [(1536, 200, 3), (1024, 72, 2), (2048, 192, 4), (3072, 520, 1)])
+def test_orthonormalize_bf16_ragged_ranks(dev, rows, r, batch):
+    """bf16 factors with `rows >= 4 r` take the fp32 pass on the bf16 matrix cores; ranks that are not multiples
+    of 64 leave a ragged last block column in the blocked Cholesky and in the rows of the inverse factor.  The
+    result must be orthonormal to bf16 rounding and span what Householder QR of the same matrix spans."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(11)
+    P = torch.randn(batch, rows, r).bfloat16()
+    Q, info = orthonormalize(P.to(dev), return_info=True)
+    assert Q.dtype == torch.bfloat16 and (info == 0).all()
+    Qd = Q.double().cpu()
+    eye = torch.eye(r, dtype=torch.float64)
+    for b in range(batch):
+        orth = (Qd[b].T @ Qd[b] - eye).norm().item()
+        Qh, _ = torch.linalg.qr(P[b].double())
+        # projector onto the span, compared with Householder's (column signs and bf16 rounding aside)
+        span = ((Qd[b] @ (Qd[b].T @ Qh)) - Qh).norm().item() / Qh.norm().item()
+        diff = rel_fro(_sign_align(Qd[b], Qh), Qh)
+        print(f"{rows}x{r} matrix {b}: ||QtQ-I|| = {orth:.2e}, span defect {span:.2e}, vs Householder {diff:.2e}")
+        assert orth <= 3e-2 * (r / 200) ** 0.5 and span <= 5e-3 and diff <= 5e-3
+
+
 @pytest.mark.parametrize("log_cond,passes,tol", [(4, 1, 5e-6), (6, 2, 5e-5), (7, 2, 2e-4), (7.5, 3, 5e-5)])
 def test_orthonormalize_conditioning(dev, log_cond, passes, tol):
     """Genuinely ill-conditioned factors (singular values graded over `log_cond` decades between random
