@@ -548,37 +548,80 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   int rc = gram<T>(P0, G, part, batch, rows, r, r_live, nullptr, gate, s);
   if (rc) return rc;
-  // blocked lower Cholesky G = L L^T (right-looking), building W alongside
+  // Two-level blocking: 64-column steps inside panels of `pw` steps.  A step's rank-64 update reaches only the
+  // rest of its panel's columns; what lies right of the panel gets one rank-(64 pw) update when the panel is done
+  // (the trailing matrix is then read and written once per panel instead of once per step).
+  static const int pw_env = [] {
+    const char* e = getenv("DION_AMD_CHOL_PANEL");
+    const int v = e ? atoi(e) : 0;
+    return v > 0 ? v : 4;
+  }();
+  const int pw = pw_env;
+  // blocked lower Cholesky G = L L^T, building W alongside
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
     rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s);
     if (rc) return rc;
     if (rest <= 0) break;
-    // A22 -= L21 L21^T, lower triangle only (nothing reads the upper one)
+    const int p0 = j / pw * pw * NB;                       // first column of the panel
+    const int pe = p0 + pw * NB < r ? p0 + pw * NB : r;    // one past its last column
     RealGemmDesc<T> u{};
     u.batch = batch;
-    u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;
-    u.B = u.A; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
-    u.C = G + (long long)(o + nb) * r + (o + nb); u.sC = rr; u.ldc = r;
-    u.E = u.C; u.sE = rr; u.lde = r;
-    u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
+    u.sA = rr; u.lda = r; u.a_kstrided = 0;
+    u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+    u.sC = rr; u.ldc = r; u.sE = rr; u.lde = r;
+    u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
     u.gate = gate.flags; u.gate_want = gate.want;
-    rc = gemm_real(u, s);
-    if (rc) return rc;
+    if (o + nb < pe) {
+      // rest of the panel's columns, all rows from the diagonal down:  A[:, panel] -= L[:, j] L[panel, j]^T
+      u.A = L + (long long)(o + nb) * r + o;
+      u.B = u.A;
+      u.C = G + (long long)(o + nb) * r + (o + nb);
+      u.E = u.C;
+      u.M = rest; u.N = pe - (o + nb); u.K = nb;
+      rc = gemm_real(u, s);
+      if (rc) return rc;
+    } else {
+      // panel done:  A22 -= L[:, panel] L[:, panel]^T, lower triangle only (nothing reads the upper one)
+      u.A = L + (long long)pe * r + p0;
+      u.B = u.A;
+      u.C = G + (long long)pe * r + pe;
+      u.E = u.C;
+      u.M = r - pe; u.N = r - pe; u.K = pe - p0;
+      rc = gemm_real(u, s);
+      if (rc) return rc;
+    }
   }
-  // P0 <- P0 R^-1 with R = L^T, in place, block column by block column:
-  //   P0[:, j] <- P0[:, 0 .. j] W[j, 0 .. j]^T
+  // P0 <- P0 R^-1 with R = L^T, in place, by the same panels: first the solved columns left of the panel are
+  // taken out of it in one product,
+  //   P0[:, panel] -= P0[:, 0 .. p0] L[panel, 0 .. p0]^T
+  // then block column by block column inside it
+  //   P0[:, j] <- P0[:, p0 .. j] W[j, p0 .. j]^T
   // (each workgroup owns 64 rows and the one 64-column output tile, and has read all it needs of
   // those rows before it stores)
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB;
+    const int p0 = j / pw * pw * NB;
+    const int pe = p0 + pw * NB < r ? p0 + pw * NB : r;
+    if (o == p0 && p0 > 0) {
+      RealGemmDesc<T> u{};
+      u.batch = batch;
+      u.A = P0; u.sA = pr; u.lda = r; u.a_kstrided = 0;
+      u.B = L + (long long)p0 * r; u.sB = rr; u.ldb = r; u.b_kstrided = 0;
+      u.C = P0 + p0; u.sC = pr; u.ldc = r;
+      u.E = u.C; u.sE = pr; u.lde = r;
+      u.M = rows; u.N = pe - p0; u.K = p0; u.alpha = -1.0; u.beta = 1.0;
+      u.gate = gate.flags; u.gate_want = gate.want;
+      rc = gemm_real(u, s);
+      if (rc) return rc;
+    }
     RealGemmDesc<T> a{};
     a.batch = batch;
-    a.A = P0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
-    a.B = W + (long long)o * r; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
+    a.A = P0 + p0; a.sA = pr; a.lda = r; a.a_kstrided = 0;
+    a.B = W + (long long)o * r + p0; a.sB = rr; a.ldb = r; a.b_kstrided = 0;
     a.C = P0 + o; a.sC = pr; a.ldc = r;
     a.E = nullptr;
-    a.M = rows; a.N = nb; a.K = o + nb; a.alpha = 1.0; a.beta = 0.0;
+    a.M = rows; a.N = nb; a.K = o + nb - p0; a.alpha = 1.0; a.beta = 0.0;
     a.gate = gate.flags; a.gate_want = gate.want;
     rc = gemm_real(a, s);
     if (rc) return rc;
@@ -712,40 +755,93 @@ int zero_cols(void* out, int dtype, const int* bad, const int* info, int batch, 
 
 // ---- the fp32 pass on the bf16 matrix cores (bf16 P: its products with bf16 factors are exact in fp32) ----
 
-// Row i of G[b] = sum of `n_hh` slabs + sum of `n_hl` slabs and their transposes (the cross terms h^T l + l^T h of
-// a matrix held as h + l), in slab order; padded diagonal and row defects as in gram_finish_kernel.
+// G[b] = sum of `n_hh` slabs + sum of `n_hl` slabs and their transposes (the cross terms h^T l + l^T h of a matrix
+// held as h + l), in slab order; padded diagonal and row defects as in gram_finish_kernel.  One workgroup per 16 rows:
+// it walks the 64-column blocks of its rows, thread t owning row t / 16 and 4 consecutive columns; the transposed
+// term comes from the mirrored 64 x 16 tile, read along its rows like the others and turned in LDS.
 __global__ __launch_bounds__(256) void gram16_finish_kernel(const float* __restrict__ part, int n_hh, int n_hl,
                                                             long long slab, float* __restrict__ G, long long rr, int r,
-                                                            int r_live, float* __restrict__ rowdef) {
-  const int b = blockIdx.y, i = blockIdx.x;
-  float* g = G + b * rr + (long long)i * r;
+                                                            int r_live, float* __restrict__ rowdef, const int* gate,
+                                                            int want) {
+  __shared__ float tr[64][17];
+  const int b = blockIdx.y, ib = blockIdx.x;
+  if (!orth_gate_open(gate, want, b)) return;
+  const int ri = threadIdx.x >> 4, c0 = (threadIdx.x & 15) * 4;
+  const int mr = threadIdx.x >> 2, mc0 = (threadIdx.x & 3) * 4;
+  const int i = ib * 16 + ri;
+  const float* pb = part + b * rr;
+  const bool vec = (r & 3) == 0;
   float acc = 0.f;
-  for (int j = threadIdx.x; j < r; j += 256) {
-    float v = 0.f;
-    for (int q = 0; q < n_hh; ++q) v += part[q * slab + b * rr + (long long)i * r + j];
-    for (int q = n_hh; q < n_hh + n_hl; ++q)
-      v += part[q * slab + b * rr + (long long)i * r + j] + part[q * slab + b * rr + (long long)j * r + i];
-    if (i >= r_live && j == i) v = 1.f;
-    g[j] = v;
-    const float e = v - (i == j ? 1.f : 0.f);
-    acc += e * e;
+  for (int jb = 0; jb * 64 < r; ++jb) {
+    const int j0 = jb * 64 + c0;
+    float v[4] = {0.f, 0.f, 0.f, 0.f}, m[4] = {0.f, 0.f, 0.f, 0.f};
+    if (i < r) {
+      for (int q = 0; q < n_hh + n_hl; ++q) {
+        const float* src = pb + q * slab + (long long)i * r + j0;
+        if (vec && j0 + 3 < r) {
+          const float4 x = *reinterpret_cast<const float4*>(src);
+          v[0] += x.x, v[1] += x.y, v[2] += x.z, v[3] += x.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (j0 + e < r) v[e] += src[e];
+        }
+      }
+    }
+    if (n_hl > 0) {
+      // mirrored tile (rows of column block jb, columns of this row block), summed over the cross-term slabs
+      const int mj = jb * 64 + mr, mi0 = ib * 16 + mc0;
+      if (mj < r) {
+        for (int q = n_hh; q < n_hh + n_hl; ++q) {
+          const float* src = pb + q * slab + (long long)mj * r + mi0;
+          if (vec && mi0 + 3 < r) {
+            const float4 x = *reinterpret_cast<const float4*>(src);
+            m[0] += x.x, m[1] += x.y, m[2] += x.z, m[3] += x.w;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (mi0 + e < r) m[e] += src[e];
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 4; ++e) tr[mr][mc0 + e] = m[e];
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += tr[c0 + e][ri];
+    }
+    if (i < r) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int j = j0 + e;
+        if (j < r) {
+          if (i >= r_live && j == i) v[e] = 1.f;
+          const float d = v[e] - (i == j ? 1.f : 0.f);
+          acc += d * d;
+        }
+      }
+      float* dst = G + b * rr + (long long)i * r + j0;
+      if (vec && j0 + 3 < r) {
+        *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j0 + e < r) dst[e] = v[e];
+      }
+    }
   }
   if (rowdef) {
-    __shared__ float red[256];
-    red[threadIdx.x] = acc;
-    __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-      if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
-      __syncthreads();
-    }
-    if (threadIdx.x == 0) rowdef[(long long)b * r + i] = red[0];
+    // the sixteen threads of a row sit in one wavefront
+    for (int o = 1; o < 16; o <<= 1) acc += __shfl_xor(acc, o);
+    if ((threadIdx.x & 15) == 0 && i < r) rowdef[(long long)b * r + i] = acc;
   }
 }
 
 // G = H^T H (+ H^T Lo + Lo^T H when Lo is given), fp32, from bf16 operands: up to four products (K slices x
 // {H^T H, H^T Lo}) run as the groups of one launch and leave fp32 slabs that the finish kernel adds in order.
 int gram16(const bf16_t* H, const bf16_t* Lo, float* G, float* part, int batch, int rows, int r, int r_live,
-           float* rowdef, hipStream_t s) {
+           float* rowdef, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   const int kinds = Lo ? 2 : 1;
   const long long tiles = (long long)batch * ((r + 255) / 256) * ((r + 255) / 256);
@@ -767,12 +863,13 @@ int gram16(const bf16_t* H, const bf16_t* Lo, float* G, float* part, int batch, 
       d.C = part + (long long)n * rr * batch; d.sC = rr; d.ldc = r; d.c_dtype = DA_F32;
       d.M = r; d.N = r; d.K = kn;
       d.epilogue = DA_EPI_STORE; d.s1 = 1.f; d.faithful = 0;
+      d.gate = gate.flags; d.gate_want = gate.want;
       ++n;
     }
   int rc = da_gemm_bf16_grouped(g, n, s);
   if (rc) return rc;
-  hipLaunchKernelGGL(gram16_finish_kernel, dim3((unsigned)r, (unsigned)batch), dim3(256), 0, s, part, nsl, Lo ? nsl : 0,
-                     rr * batch, G, rr, r, r_live, rowdef);
+  hipLaunchKernelGGL(gram16_finish_kernel, dim3((unsigned)((r + 15) / 16), (unsigned)batch), dim3(256), 0, s, part, nsl, Lo ? nsl : 0,
+                     rr * batch, G, rr, r, r_live, rowdef, gate.flags, gate.want);
   return da_launch_status();
 }
 
@@ -842,7 +939,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   float* C2 = reinterpret_cast<float*>(w.P0);         // rows x 2r fp32 = the room of the fp64 copy
   bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
   float* part = reinterpret_cast<float*>(w.part);
-  int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, s);
+  int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, all, s);
   if (rc) return rc;
   // (the steps write the rows of L^-1 themselves: no W, no recurrence on the identity afterwards)
   static const bool inv_rows = [] { const char* e = getenv("DION_AMD_ORTH_NO_INV"); return !(e && atoi(e)); }();
@@ -897,7 +994,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
     c.epilogue = DA_EPI_STORE; c.s1 = 1.f; c.faithful = 0;
     rc = da_gemm_bf16(c, s);
     if (rc || !second_gram) return rc;
-    return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, s);
+    return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, all, s);
   }
   GemmDesc c{};
   c.batch = batch;
@@ -915,7 +1012,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
                      w.Ph, Lo, pr, r);
   rc = da_launch_status();
   if (rc || !second_gram) return rc;
-  return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, s);
+  return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, all, s);
 }
 
 // bf16 copy of the matrices whose gate is open
@@ -1035,14 +1132,21 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   if (rc) return rc;
   if (passes == 1) return da_cvt_from_f64(w.P0, out, dtype, pr, batch, gate, s);
   float* Gf = reinterpret_cast<float*>(w.G);
-  // one conversion pass to fp32 costs less than reading fp64 twice in the polishing products
   const bool last_low = passes == 2 && low;
-  rc = da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate, s);
+  // A bf16 result after one polishing pass needs the fp64 pass's result to 16 bits only, as h + l (bf16 each): the
+  // Gram matrix that measures its defect then runs on the bf16 matrix cores (h^T h + h^T l + l^T h), and the
+  // correction product reads h.  Otherwise: one conversion pass to fp32 costs less than reading fp64 twice in the
+  // polishing products.
+  const bool hl = last_low && dtype == DA_BF16 && !no16;
+  bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
+  rc = hl ? da_cvt_f64_to_hl(w.P0, w.Ph, Lo, pr, batch, gate, s)
+          : da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate, s);
   if (rc) return rc;
   const float* cur = w.Pf;
   for (int pass = 1; pass < passes; ++pass) {
     const bool last = pass + 1 == passes;
-    rc = gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s);
+    rc = hl ? gram16(w.Ph, Lo, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s)
+            : gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s);
     if (rc) return rc;
     const int* bad = nullptr;
     if (pass == 1) {

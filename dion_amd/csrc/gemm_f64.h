@@ -14,7 +14,7 @@ struct RealGemmDesc {
   int lda, ldb, ldc, lde;
   int M, N, K, batch;
   int a_kstrided, b_kstrided, symmetric;
-  int lower_only;  // 1 (M == N): only tiles on or below the diagonal are computed and stored
+  int lower_only;  // 1 (M >= N): only tiles on or below the diagonal (row tile >= column tile) are computed and stored
   double alpha, beta;
   int split_k;   // > 1: K is cut into that many slices (no E term); slice s writes its partial product to
                  // C + s * split_stride and the caller adds the slices in a fixed order (da_auto_split tells it
@@ -64,6 +64,8 @@ int da_cvt_to_f32(const void* src, int src_dtype, float* dst, long long per, int
 int da_cvt_from_f64(const double* src, void* dst, int dst_dtype, long long per, int batch, DaGate gate, hipStream_t s);
 // dst (f32) <- src (f64 / f32; dst may be null for an f32 source); `low`, if not null, receives the same values in bf16
 int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
+// h, l (bf16) <- src (f64): h = src rounded to bf16, l = bf16(src - h), i.e. src to 16 bits as h + l
+int da_cvt_f64_to_hl(const double* src, bf16_t* h, bf16_t* l, long long per, int batch, DaGate gate, hipStream_t s);
 int da_cvt_f32_to_bf16(const float* src, bf16_t* low, long long per, int batch, DaGate gate, hipStream_t s);
 // dst (bf16 / f32) <- src (f32)
 int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, int batch, DaGate gate, hipStream_t s);

@@ -73,7 +73,8 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (d.M + BTt - 1) / BTt, tiles_n = (d.N + BTt - 1) / BTt;
   const bool tri = SYM || d.lower_only;
-  const int per_batch = tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  // SYM: M == N; lower_only: M >= N, column tile c holds the tiles_m - c row tiles from the diagonal down
+  const int per_batch = tri ? tiles_n * tiles_m - tiles_n * (tiles_n - 1) / 2 : tiles_m * tiles_n;
   const int split = blockIdx.y;  // split-K slice
   const int b = blockIdx.x / per_batch;
   if (d.gate && (d.gate[b] != 0) != (d.gate_want != 0)) return;
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(RealGemmDesc<T> d) {
 template <typename T, int BTt>
 long long blocks_of(const RealGemmDesc<T>& d) {
   const long long tiles_m = (d.M + BTt - 1) / BTt, tiles_n = (d.N + BTt - 1) / BTt;
-  return ((d.symmetric || d.lower_only) ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n) * d.batch;
+  return ((d.symmetric || d.lower_only) ? tiles_n * tiles_m - tiles_n * (tiles_n - 1) / 2 : tiles_m * tiles_n) * d.batch;
 }
 
 template <typename T, bool A_KS, bool B_KS, bool SYM, int BTt>
@@ -302,6 +303,20 @@ __global__ __launch_bounds__(256) void cvt_f32_low_kernel(const R* __restrict__ 
   }
 }
 
+// fp64 -> h + l (bf16 each): h = the value rounded to bf16, l = what is left of it, rounded to bf16
+__global__ __launch_bounds__(256) void cvt_hl_kernel(const double* __restrict__ src, bf16_t* __restrict__ h,
+                                                     bf16_t* __restrict__ l, long long per, const int* gate, int want) {
+  const long long b = blockIdx.y;
+  if (!gate_open(gate, want, (int)b)) return;
+  src += b * per;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < per; i += (long long)gridDim.x * 256) {
+    const float v = (float)src[i];
+    const bf16_t hi = f2bf(v);
+    h[b * per + i] = hi;
+    l[b * per + i] = f2bf(v - bf2f(hi));
+  }
+}
+
 inline dim3 cvt_grid(long long per, int batch) {
   long long b = (per + 255) / 256;
   const long long cap = 8192 / batch > 0 ? 8192 / batch : 1;
@@ -312,7 +327,7 @@ inline dim3 cvt_grid(long long per, int batch) {
 template <typename T>
 int gemm_real(const RealGemmDesc<T>& d, hipStream_t s) {
   if (!d.A || !d.B || !d.C || d.M <= 0 || d.N <= 0 || d.K < 0 || d.batch <= 0) return DA_ERR_ARG;
-  if (d.lower_only && (d.M != d.N || d.symmetric)) return DA_ERR_ARG;
+  if (d.lower_only && (d.M < d.N || d.symmetric)) return DA_ERR_ARG;
   if (d.c_store != DA_STORE_NATIVE && d.c_store != DA_STORE_BF16 && d.c_store != DA_STORE_F32) return DA_ERR_DTYPE;
   if (d.c_store != DA_STORE_NATIVE && (d.E || d.split_k > 1 || d.symmetric)) return DA_ERR_ARG;
   if (d.k_tri && (d.symmetric || d.lower_only || d.split_k > 1)) return DA_ERR_ARG;
@@ -367,6 +382,11 @@ int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, i
     hipLaunchKernelGGL((cvt_down_kernel<float, float>), cvt_grid(per, batch), dim3(256), 0, s, src, static_cast<float*>(dst), per, g.flags, g.want);
   else
     return DA_ERR_DTYPE;
+  return da_launch_status();
+}
+int da_cvt_f64_to_hl(const double* src, bf16_t* h, bf16_t* l, long long per, int batch, DaGate g, hipStream_t s) {
+  if (per <= 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  hipLaunchKernelGGL(cvt_hl_kernel, cvt_grid(per, batch), dim3(256), 0, s, src, h, l, per, g.flags, g.want);
   return da_launch_status();
 }
 int da_cvt_f64_to_f32(const double* src, float* dst, bf16_t* low, long long per, int batch, DaGate g, hipStream_t s) {
