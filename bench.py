@@ -385,6 +385,14 @@ def tile_trace(dev):
         run(f"X' = aX + BX, {b} x {m}x{n}", lambda: gemm(B, X, b_kstrided=True, E=X, s0=3.0, s1=1.0, out=Y, faithful=True),
             b * (m // 256) * (n // 256))
         del X, B, Y
+    # A = X X^T (upper tiles) on b x (768 x 3072): 6 b tiles of 48 stages each, one per CU while 6 b <= 256 -- the
+    # same tile program on 48 ... 252 busy CUs
+    from dion_amd.newton_schulz import ns_line_1
+    for b in (8, 24, 32, 40, 42):
+        X = (torch.randn(b, 768, 3072, device=dev) * 0.03).to(bf)
+        A = torch.empty(b, 768, 768, device=dev, dtype=bf)
+        run(f"A = X X^T, {b} x 768x3072 ({6 * b} tiles)", lambda: ns_line_1(X, out=A), 6 * b)
+        del X, A
 
 
 def main():
