@@ -741,8 +741,10 @@ int correction_f32(const float* in, void* out, int out_store, const float* G, fl
 int zero_cols(void* out, int dtype, const int* bad, const int* info, int batch, int rows, int r, DaGate gate,
               hipStream_t s) {
   const long long n = (long long)rows * r;
+  // (a rare pass: a few workgroups per matrix, so that the launch costs little when no column was dropped)
   long long blocks = (n + 255) / 256;
-  if (blocks > 1024) blocks = 1024;
+  const long long cap = 2048 / batch > 8 ? 2048 / batch : 8;
+  if (blocks > cap) blocks = cap;
   const dim3 grid((unsigned)blocks, (unsigned)batch);
   if (dtype == DA_BF16)
     hipLaunchKernelGGL(zero_cols_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(out), bad, rows, r, info,
