@@ -214,14 +214,21 @@ __global__ __launch_bounds__(256) void colsum_kernel(const TM* __restrict__ R, d
   }
 }
 
-// sums[b][c] = part[0][b][c] + part[1][b][c] + ... in that order
+// sums[b][c] = sum over the slices of part[k][b][c], in a fixed order: 64 columns per workgroup, the slices cut into
+// four contiguous runs (one per wavefront, each added in slice order), the four run sums added in run order
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const double* __restrict__ part, double* __restrict__ sums,
                                                             int slices, long long per_slice) {
-  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (i >= per_slice) return;
+  __shared__ double run[4][64];
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const long long i = (long long)blockIdx.x * 64 + lane;
+  const int per_run = (slices + 3) / 4;
+  const int k0 = q * per_run, k1 = k0 + per_run < slices ? k0 + per_run : slices;
   double s = 0.0;
-  for (int k = 0; k < slices; ++k) s += part[k * per_slice + i];
-  sums[i] = s;
+  if (i < per_slice)
+    for (int k = k0; k < k1; ++k) s += part[k * per_slice + i];
+  run[q][lane] = s;
+  __syncthreads();
+  if (q == 0 && i < per_slice) sums[i] = ((run[0][lane] + run[1][lane]) + run[2][lane]) + run[3][lane];
 }
 
 template <typename TM, typename TQ>
@@ -356,7 +363,7 @@ int da_colnorm(const void* R, void* qn, int m_dtype, const DaPtrTable& q, int q_
     hipLaunchKernelGGL(colsum_kernel<float>, g1, dim3(256), 0, s, static_cast<const float*>(R), part, rows, r, rps);
   else
     return DA_ERR_DTYPE;
-  hipLaunchKernelGGL(colsum_finish_kernel, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, s, part, sums, slices, ns);
+  hipLaunchKernelGGL(colsum_finish_kernel, dim3((unsigned)((ns + 63) / 64)), dim3(256), 0, s, part, sums, slices, ns);
   const long long n = (long long)rows * r;
   dim3 g2(ew_blocks(n), batch);
   if (m_dtype == DA_BF16 && q_dtype == DA_BF16)
