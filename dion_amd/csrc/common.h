@@ -107,6 +107,11 @@ struct GemmDesc {
   // over is rounded to bf16 as well and stored c2_off elements after C -- the result as two bf16 matrices.
   int a_kwrap;
   long long c2_off;
+  // bf16 kernel, optional.  k_slices > 1: the sum over k is cut into that many slices of k_slice elements (a multiple
+  // of 64; the last one may be shorter) that run as tiles of their own; slice s stores its partial product as
+  // matrices s * batch ... s * batch + batch - 1 of C, which therefore holds k_slices * batch matrices sC apart,
+  // and the caller adds them in a fixed order.  Plain fp32 store only (no E, no tables, no second output).
+  int k_slices, k_slice;
 };
 
 // Epilogues.  With `faithful` set the rounding points of the reference's separate

@@ -388,6 +388,23 @@ namespace {
 // Slices of K of the Gram products of `batch` rows x r matrices (1: unsliced).
 int gram_slices(int batch, int rows, int r) { return da_auto_split(da_gram_blocks(r, batch), rows); }
 
+// The same for the Gram products on the bf16 matrix cores (`kinds` products in the launch): slices until about 256
+// tiles of 256 x 256 exist, but each slice is another fp32 slab for the finishing pass to read, so no more of them
+// than keep the slabs (r x r each) small beside the operand (rows x r): rows / 4r; each at least 512 rows deep and a
+// multiple of the stage depth.  `ks` receives the rows per slice.
+int gram16_slices(int batch, int rows, int r, int kinds, int* ks) {
+  const long long tiles = (long long)kinds * batch * ((r + 255) / 256) * ((r + 255) / 256);
+  long long nsl = (256 + tiles - 1) / tiles;
+  const int by_slab = rows / (4 * r) > 0 ? rows / (4 * r) : 1;
+  if (nsl > by_slab) nsl = by_slab;
+  const int by_rows = rows / 512 > 0 ? rows / 512 : 1;
+  if (nsl > by_rows) nsl = by_rows;
+  if (nsl > 64) nsl = 64;
+  const int per = (int)(((rows + nsl - 1) / nsl + 63) / 64 * 64);
+  if (ks) *ks = per;
+  return (rows + per - 1) / per;
+}
+
 size_t orth_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Workspace of one call, carved in this order.
@@ -400,6 +417,7 @@ struct OrthWs {
   double* W;       // inverse-factor blocks
   double* part;    // K-slice outputs of a sliced Gram product
   float* rowdef;   // r per matrix: squared defect of each row of the polishing pass's Gram matrix
+  float* rowdef_part;   // ... as partial sums per 64-column block
   int* need;       // per matrix: 1 = the fp32 pass was not enough, the fp64 pass runs
   int* info32;     // per matrix: status of the fp32 factorisation
   int* bad;        // r per matrix: 1 = the column is not usable (noise-level pivot), it is zeroed
@@ -415,9 +433,12 @@ struct OrthWs {
     G = reinterpret_cast<double*>(take(rr * 8));
     L = reinterpret_cast<double*>(take(rr * 8));
     W = reinterpret_cast<double*>(take(rr * 8));
-    // K-slice outputs: `sp` slices of the fp64 / fp32 Gram kernels, or up to four fp32 slabs of the bf16 one
-    part = reinterpret_cast<double*>(take(rr * 8 * (sp > 2 ? sp : 2)));
+    // K-slice outputs: `sp` slices of the fp64 / fp32 Gram kernels, or two fp32 slabs per slice of the bf16 one
+    const size_t slabs16 = (size_t)2 * gram16_slices(batch, rows, r, 1, nullptr);   // (one product has the most slices)
+    const size_t part_a = rr * 8 * (sp > 2 ? sp : 2), part_b = rr * 4 * slabs16;
+    part = reinterpret_cast<double*>(take(part_a > part_b ? part_a : part_b));
     rowdef = reinterpret_cast<float*>(take((size_t)r * batch * 4));
+    rowdef_part = reinterpret_cast<float*>(take((size_t)((r + 63) / 64) * r * batch * 4));
     need = reinterpret_cast<int*>(take((size_t)batch * 4));
     info32 = reinterpret_cast<int*>(take((size_t)batch * 4));
     bad = reinterpret_cast<int*>(take((size_t)r * batch * 4));
@@ -771,20 +792,24 @@ int zero_cols(void* out, int dtype, const int* bad, const int* info, int batch, 
 __global__ __launch_bounds__(256) void gram16_finish_kernel(const float* __restrict__ part, int n_hh, int n_hl,
                                                             long long slab, float* __restrict__ G, long long rr, int r,
                                                             int r_live, float* __restrict__ rowdef, const int* gate,
-                                                            int want) {
+                                                            int want, int jb_per_z) {
   __shared__ float tr[64][17];
   const int b = blockIdx.y, ib = blockIdx.x;
   if (!orth_gate_open(gate, want, b)) return;
+  // gridDim.z > 1: this workgroup covers jb_per_z column blocks and leaves its rows' defects as partial sums,
+  // gridDim.y * r floats per z, for rowdef_sum_kernel
+  const int jb_first = blockIdx.z * jb_per_z;
   const int ri = threadIdx.x >> 4, c0 = (threadIdx.x & 15) * 4;
   const int mr = threadIdx.x >> 2, mc0 = (threadIdx.x & 3) * 4;
   const int i = ib * 16 + ri;
   const float* pb = part + b * rr;
   const bool vec = (r & 3) == 0;
   float acc = 0.f;
-  for (int jb = 0; jb * 64 < r; ++jb) {
+  for (int jb = jb_first; jb < jb_first + jb_per_z && jb * 64 < r; ++jb) {
     const int j0 = jb * 64 + c0;
     float v[4] = {0.f, 0.f, 0.f, 0.f}, m[4] = {0.f, 0.f, 0.f, 0.f};
     if (i < r) {
+#pragma unroll 4
       for (int q = 0; q < n_hh + n_hl; ++q) {
         const float* src = pb + q * slab + (long long)i * r + j0;
         if (vec && j0 + 3 < r) {
@@ -801,6 +826,7 @@ __global__ __launch_bounds__(256) void gram16_finish_kernel(const float* __restr
       // mirrored tile (rows of column block jb, columns of this row block), summed over the cross-term slabs
       const int mj = jb * 64 + mr, mi0 = ib * 16 + mc0;
       if (mj < r) {
+#pragma unroll 4
         for (int q = n_hh; q < n_hh + n_hl; ++q) {
           const float* src = pb + q * slab + (long long)mj * r + mi0;
           if (vec && mi0 + 3 < r) {
@@ -843,42 +869,57 @@ __global__ __launch_bounds__(256) void gram16_finish_kernel(const float* __restr
   if (rowdef) {
     // the sixteen threads of a row sit in one wavefront
     for (int o = 1; o < 16; o <<= 1) acc += __shfl_xor(acc, o);
-    if ((threadIdx.x & 15) == 0 && i < r) rowdef[(long long)b * r + i] = acc;
+    if ((threadIdx.x & 15) == 0 && i < r) rowdef[((long long)blockIdx.z * gridDim.y + b) * r + i] = acc;
   }
 }
 
-// G = H^T H (+ H^T Lo + Lo^T H when Lo is given), fp32, from bf16 operands: up to four products (K slices x
-// {H^T H, H^T Lo}) run as the groups of one launch and leave fp32 slabs that the finish kernel adds in order.
+// rowdef[e] = part[0][e] + part[1][e] + ... in that order (`n` floats per part)
+__global__ __launch_bounds__(256) void rowdef_sum_kernel(const float* __restrict__ part, int parts, long long n,
+                                                         float* __restrict__ rowdef) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  float s = 0.f;
+  for (int z = 0; z < parts; ++z) s += part[z * n + e];
+  rowdef[e] = s;
+}
+
+// G = H^T H (+ H^T Lo + Lo^T H when Lo is given), fp32, from bf16 operands: the two products run as the groups of
+// one launch, each cut into K slices that are tiles of their own (so that a tall, narrow H still fills the GPU),
+// and leave fp32 slabs that the finish kernel adds in order.
 int gram16(const bf16_t* H, const bf16_t* Lo, float* G, float* part, int batch, int rows, int r, int r_live,
-           float* rowdef, DaGate gate, hipStream_t s) {
+           float* rowdef, float* rowdef_part, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   const int kinds = Lo ? 2 : 1;
-  const long long tiles = (long long)batch * ((r + 255) / 256) * ((r + 255) / 256);
-  int nsl = (int)((256 + tiles - 1) / tiles);
-  if (nsl > DA_MAX_GROUPS / kinds) nsl = DA_MAX_GROUPS / kinds;
-  if (nsl > rows / 256) nsl = rows / 256 > 0 ? rows / 256 : 1;
-  const int ks = ((rows + nsl - 1) / nsl + 63) / 64 * 64;   // rows per slice, a multiple of the stage depth
-  nsl = (rows + ks - 1) / ks;
-  GemmDesc g[DA_MAX_GROUPS];
-  int n = 0;
-  for (int kind = 0; kind < kinds; ++kind)
-    for (int q = 0; q < nsl; ++q) {
-      const int k0 = q * ks, kn = rows - k0 < ks ? rows - k0 : ks;
-      GemmDesc& d = g[n];
-      d = GemmDesc{};
-      d.batch = batch;
-      d.A = H + (long long)k0 * r; d.sA = pr; d.lda = r; d.a_kstrided = 1;
-      d.B = (kind == 0 ? H : Lo) + (long long)k0 * r; d.sB = pr; d.ldb = r; d.b_kstrided = 1;
-      d.C = part + (long long)n * rr * batch; d.sC = rr; d.ldc = r; d.c_dtype = DA_F32;
-      d.M = r; d.N = r; d.K = kn;
-      d.epilogue = DA_EPI_STORE; d.s1 = 1.f; d.faithful = 0;
-      d.gate = gate.flags; d.gate_want = gate.want;
-      ++n;
-    }
+  int ks = 0;
+  const int nsl = gram16_slices(batch, rows, r, kinds, &ks);
+  GemmDesc g[2];
+  const int n = kinds;
+  for (int kind = 0; kind < kinds; ++kind) {
+    GemmDesc& d = g[kind];
+    d = GemmDesc{};
+    d.batch = batch;
+    d.A = H; d.sA = pr; d.lda = r; d.a_kstrided = 1;
+    d.B = kind == 0 ? H : Lo; d.sB = pr; d.ldb = r; d.b_kstrided = 1;
+    // the slices' partial products: slabs kind * nsl ... kind * nsl + nsl - 1 of `batch` matrices each
+    d.C = part + (long long)kind * nsl * rr * batch; d.sC = rr; d.ldc = r; d.c_dtype = DA_F32;
+    d.M = r; d.N = r; d.K = rows;
+    d.k_slices = nsl; d.k_slice = ks;
+    d.epilogue = DA_EPI_STORE; d.s1 = 1.f; d.faithful = 0;
+    d.gate = gate.flags; d.gate_want = gate.want;
+  }
   int rc = da_gemm_bf16_grouped(g, n, s);
   if (rc) return rc;
-  hipLaunchKernelGGL(gram16_finish_kernel, dim3((unsigned)((r + 15) / 16), (unsigned)batch), dim3(256), 0, s, part, nsl, Lo ? nsl : 0,
-                     rr * batch, G, rr, r, r_live, rowdef, gate.flags, gate.want);
+  // few row blocks (a narrow factor, a small batch): one workgroup per column block as well, so that the slabs are
+  // read by enough workgroups; the rows' defects then take a second, tiny launch
+  const int njb = (r + 63) / 64, row_wgs = (r + 15) / 16 * batch;
+  const int nz = row_wgs < 256 ? njb : 1;
+  hipLaunchKernelGGL(gram16_finish_kernel, dim3((unsigned)((r + 15) / 16), (unsigned)batch, (unsigned)nz), dim3(256), 0, s,
+                     part, nsl, Lo ? nsl : 0, rr * batch, G, rr, r, r_live, rowdef && nz > 1 ? rowdef_part : rowdef,
+                     gate.flags, gate.want, nz > 1 ? 1 : njb);
+  rc = da_launch_status();
+  if (rc || !rowdef || nz == 1) return rc;
+  const long long nd = (long long)batch * r;
+  hipLaunchKernelGGL(rowdef_sum_kernel, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, s, rowdef_part, nz, nd, rowdef);
   return da_launch_status();
 }
 
@@ -948,7 +989,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   float* C2 = reinterpret_cast<float*>(w.P0);         // rows x 2r fp32 = the room of the fp64 copy
   bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
   float* part = reinterpret_cast<float*>(w.part);
-  int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, all, s);
+  int rc = gram16(P, nullptr, G, part, batch, rows, r, r_live, nullptr, nullptr, all, s);
   if (rc) return rc;
   // (the steps write the rows of L^-1 themselves: no W, no recurrence on the identity afterwards)
   static const bool inv_rows = [] { const char* e = getenv("DION_AMD_ORTH_NO_INV"); return !(e && atoi(e)); }();
@@ -1003,7 +1044,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
     c.epilogue = DA_EPI_STORE; c.s1 = 1.f; c.faithful = 0;
     rc = da_gemm_bf16(c, s);
     if (rc || !second_gram) return rc;
-    return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, all, s);
+    return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, w.rowdef_part, all, s);
   }
   GemmDesc c{};
   c.batch = batch;
@@ -1021,7 +1062,7 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
                      w.Ph, Lo, pr, r);
   rc = da_launch_status();
   if (rc || !second_gram) return rc;
-  return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, all, s);
+  return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, w.rowdef_part, all, s);
 }
 
 // bf16 copy of the matrices whose gate is open
@@ -1154,7 +1195,7 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   const float* cur = w.Pf;
   for (int pass = 1; pass < passes; ++pass) {
     const bool last = pass + 1 == passes;
-    rc = hl ? gram16(w.Ph, Lo, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s)
+    rc = hl ? gram16(w.Ph, Lo, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, w.rowdef_part, gate, s)
             : gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s);
     if (rc) return rc;
     const int* bad = nullptr;

@@ -378,11 +378,22 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const int wave = wave_uniform(tid >> 6);
   const int wm = wave / C::WGN, wn = wave % C::WGN;
   const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0);
-  const int b = tile.b, ti = tile.ti, tj = tile.tj;
+  const int ti = tile.ti, tj = tile.tj;
+  // with K slices the tile index counts (slice, matrix) pairs: the slice's partial product is matrix tile.b of C
+  int b = tile.b, dK = d.K;
+  long long k0 = 0;
+  if (d.k_slices > 1) {
+    const int slice = tile.b / d.batch;
+    b = tile.b - slice * d.batch;
+    k0 = (long long)slice * d.k_slice;
+    dK = d.K - (int)k0 < d.k_slice ? d.K - (int)k0 : d.k_slice;
+  }
   if (d.gate && (d.gate[b] != 0) != (d.gate_want != 0)) return;   // (before any barrier: the whole workgroup leaves)
   const int m0 = ti * BT, n0 = tj * BT;
-  const bf16_t* A = d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) + d.a_off : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA;
-  const bf16_t* B = d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB;
+  const bf16_t* A = (d.Atab ? static_cast<const bf16_t*>(d.Atab[b]) + d.a_off : static_cast<const bf16_t*>(d.A) + (long long)b * d.sA) +
+                    k0 * (A_KS ? d.lda : 1);
+  const bf16_t* B = (d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB) +
+                    k0 * (B_KS ? d.ldb : 1);
 
   f32x16_t acc[TMI][TNJ];
 #pragma unroll
@@ -395,7 +406,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   StageAddr<C, A_KS> sa(A, d.lda, m0, tid, d.M);
   StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
   const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
-  const int KT = (d.K + BK - 1) / BK;
+  const int KT = (dK + BK - 1) / BK;
   bf16x8_t fa[TMI], fb[TNJ];
 
 #define DA_FREAD(st, ks)                                                                           \
@@ -482,15 +493,15 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
       const int r_ = sa.row + i * A_RSTEP;                                                         \
-      const bool ok = A_KS ? ((kt) * BK + r_ < d.K && m0 + sa.col < d.M)                           \
-                           : (m0 + r_ < d.M && (kt) * BK + sa.col < d.K);                          \
+      const bool ok = A_KS ? ((kt) * BK + r_ < dK && m0 + sa.col < d.M)                            \
+                           : (m0 + r_ < d.M && (kt) * BK + sa.col < dK);                           \
       const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
       ra[i] = ok ? *reinterpret_cast<const u32x4_t*>(sa.g + i * sa.gstep) : z_;                    \
     }                                                                                              \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
       const int r_ = sb.row + i * B_RSTEP;                                                         \
-      const bool ok = B_KS ? ((kt) * BK + r_ < d.K && n0 + sb.col < d.N)                           \
-                           : (n0 + r_ < d.N && (kt) * BK + sb.col < d.K);                          \
+      const bool ok = B_KS ? ((kt) * BK + r_ < dK && n0 + sb.col < d.N)                            \
+                           : (n0 + r_ < d.N && (kt) * BK + sb.col < dK);                           \
       const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
       rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;                    \
     }                                                                                              \
@@ -528,7 +539,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
 #undef DA_FREAD2
 #undef DA_MMA2
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
-  epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, b, ti, tj, m0, n0, wave, lane, wm, wn);
+  epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, tile.b, ti, tj, m0, n0, wave, lane, wm, wn);
   if (trace) {
     __syncthreads();
     if (tid == 0) {
@@ -578,7 +589,7 @@ bool edge_loop_ok(const GemmDesc* d, int n, int bt) {
 template <typename C>
 long long tiles_of(const GemmDesc& d) {
   const long long tm = (d.M + C::BT - 1) / C::BT, tn = (d.N + C::BT - 1) / C::BT;
-  return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch;
+  return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch * (d.k_slices > 1 ? d.k_slices : 1);
 }
 
 template <typename C, bool A_KS, bool B_KS, bool SYM>
@@ -645,6 +656,10 @@ int check_desc(const GemmDesc& d) {
   if (d.a_kwrap && (d.a_kwrap < 0 || d.a_kstrided || d.a_kwrap % BK || d.K % d.a_kwrap)) return DA_ERR_ARG;
   if (d.c2_off && (d.c_dtype != DA_BF16 || d.epilogue != DA_EPI_STORE || d.faithful || d.symmetric || (d.c2_off & 7)))
     return DA_ERR_ARG;
+  if (d.k_slices < 0 || (d.k_slices > 1 && (d.k_slice <= 0 || d.k_slice % BK || (long long)(d.k_slices - 1) * d.k_slice >= d.K ||
+                                            (long long)d.k_slices * d.k_slice < d.K || d.c_dtype != DA_F32 ||
+                                            d.epilogue != DA_EPI_STORE || d.Ctab || d.a_kwrap || d.c2_off || d.symmetric)))
+    return DA_ERR_ARG;
   return DA_OK;
 }
 
@@ -656,7 +671,7 @@ template <typename C>
 double launch_cost(const GemmDesc* d, int n, int slots, double unit) {
   double level = 0.0, longest = 0.0;
   for (int g = 0; g < n; ++g) {
-    const double kt = (double)((d[g].K + BK - 1) / BK);
+    const double kt = (double)(((d[g].k_slices > 1 ? d[g].k_slice : d[g].K) + BK - 1) / BK);
     const double rounds = (double)tiles_of<C>(d[g]) / slots;
     if (g + 1 < n) {
       level += rounds * kt;
