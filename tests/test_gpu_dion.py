@@ -41,11 +41,14 @@ def test_orthonormalize(dev, rows, r, dtype):
     assert (torch.diagonal(Rm) > 0).all()
 
 
-@pytest.mark.parametrize("rows,r,batch", [(1536, 200, 3), (1024, 72, 2), (2048, 192, 4), (3072, 520, 1)])
+@pytest.mark.parametrize("rows,r,batch", [(1536, 200, 3), (1024, 72, 2), (2048, 192, 4), (3072, 520, 1),
+                                          (16384, 256, 1), (12296, 136, 2)])
 def test_orthonormalize_bf16_ragged_ranks(dev, rows, r, batch):
     """bf16 factors with `rows >= 4 r` take the fp32 pass on the bf16 matrix cores; ranks that are not multiples
     of 64 leave a ragged last block column in the blocked Cholesky and in the rows of the inverse factor.  The
-    result must be orthonormal to bf16 rounding and span what Householder QR of the same matrix spans."""
+    result must be orthonormal to bf16 rounding and span what Householder QR of the same matrix spans.
+    The last two cases are tall and narrow: their Gram products run as 16 and 22 K slices (the last one ragged) and
+    the finishing pass splits the column blocks across workgroups."""
     from dion_amd.newton_schulz import orthonormalize
 
     torch.manual_seed(11)
