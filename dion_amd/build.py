@@ -33,7 +33,9 @@ FLAGS = [
 PER_FILE_FLAGS = {
     "gemm_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "gemm_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
-    "cholesky.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    # (cholesky.hip also: without the second option the compiler merges the stores of two branches into different
+    # named register tiles into one store through a selected pointer, and both tiles then live in scratch memory)
+    "cholesky.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1", "-mllvm", "-simplifycfg-sink-common=false"],
 }
 
 

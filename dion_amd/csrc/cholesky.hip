@@ -11,6 +11,11 @@
 // A second form of the kernel (INV) writes, instead of W's row block, row block j of T = L^-1 itself:
 //   T[j, j] = D_j,   T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c],   c < j,
 // for the callers that need the inverse factor as a matrix.
+// Deferred trailing update (o_prev >= 0): the rank-64 update of the previous step, A[i, c] -= L[i, p] L[c, p]^T
+// (p = the previous block column), has not been applied to the matrix.  This launch applies it where it needs it
+// -- every workgroup to the diagonal block before factoring it, a panel role to its tile -- and further workgroups
+// (workgroup index >= per) do nothing but apply it to the tiles right of this block column (up to column c_end), which
+// the later steps read: the separate update launch between two steps is gone.
 // No host synchronisation: a failed pivot is recorded in a device-side info word, mirroring
 // torch.linalg.cholesky_ex's `info`.
 #include "gemm_f64.h"
@@ -43,10 +48,10 @@ __device__ __forceinline__ bool usable_pivot(float p) { return __builtin_amdgcn_
 template <typename T> struct Quad { T v[4]; };
 
 template <typename T, bool INV>
-__global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G, T* __restrict__ Lmat,
+__global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __restrict__ Lmat,
                                                         T* __restrict__ Wmat, T* __restrict__ Tmat, long long sG, int r,
                                                         int o, int nb, int below, int* __restrict__ info, int fresh,
-                                                        const int* gate, int gate_want) {
+                                                        const int* gate, int gate_want, int o_prev, int c_end, int per) {
   typedef typename Mfma<T>::acc_t acc_t;
   typedef Quad<T> quad_t;
   __shared__ __attribute__((aligned(16))) T scol[2][4][NB];     // published block column of S: [column][row]
@@ -55,24 +60,19 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   __shared__ __attribute__((aligned(16))) quad_t xops[2][NB];   // X, [column] -> 4 rows
   extern __shared__ __attribute__((aligned(16))) unsigned char opnd_raw[];   // two k-major 64 x 64 operand tiles
   T* const opnd = reinterpret_cast<T*>(opnd_raw);
-  const int b = blockIdx.y, tid = threadIdx.x;
+  // grid (matrix, workgroup of the matrix): the matrices' workgroups 0 are dispatched first, the update-only
+  // workgroups of a deferred trailing update last -- they must not keep the serial part waiting for a CU
+  const int b = blockIdx.x, wg = blockIdx.y, tid = threadIdx.x;
   if (gate && (gate[b] != 0) != (gate_want != 0)) return;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lc = lane & 15, lg = lane >> 4;
   // D_j transposed (dT[k][x] = D[x][k], zero outside the nb x nb lower triangle) and, for role 0, L_jj (in `op`)
   T* const dT = opnd;
   T* const op = opnd + NB * LP;
+  // deferred mode: L[j, p] k-major (ljT[k][n] = L[o + n][o_prev + k]), behind the role buffers
+  T* const ljT = opnd + (INV ? 5 : 2) * NB * LP;
+  const bool defer = o_prev >= 0;
   const T* g = G + (long long)b * sG + (long long)o * r + o;
-  acc_t S[4], Y[4];
-#pragma unroll
-  for (int tj = 0; tj < 4; ++tj)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int i = wave * 16 + Mfma<T>::row(v, lane), j = tj * 16 + lc;
-      // identity padding beyond nb keeps the padded part inert
-      S[tj][v] = (tj <= wave && i < nb && j < nb) ? g[(long long)i * r + j] : (i == j ? T(1) : T(0));
-      Y[tj][v] = (i == j) ? T(1) : T(0);
-    }
   // The workgroups of one matrix share its roles round-robin (role 0: L_jj, D_j and the status word; 1 .. below:
   // panel tiles; the rest: W tiles).  The operand tile of a product does not depend on this step's factor: it is
   // requested now, 16 elements per thread, and the next one while the previous product runs.
@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   // q = 0 .. 3 (named vectors, not an array: an array that one loop iteration writes and the next one reads ends up
   // in scratch memory).
   typedef T tv4_t __attribute__((ext_vector_type(4)));
-  tv4_t pa0, pa1, pa2, pa3, pb0, pb1, pb2, pb3;
+  const tv4_t tz = {T(0), T(0), T(0), T(0)};
+  tv4_t pa0 = tz, pa1 = tz, pa2 = tz, pa3 = tz, pb0 = tz, pb1 = tz, pb2 = tz, pb3 = tz;
   const int trow = tid >> 4, tcol = (tid & 15) * 4;
   // rows < rows_ok, columns < cols_ok of the tile at src (row pitch r); the rest reads as zero
   auto load_quad = [&](const T* src, int q, int rows_ok, int cols_ok) __attribute__((always_inline)) {
@@ -117,6 +118,93 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
     store_quad(v0, 0, (dst), (transposed)); store_quad(v1, 1, (dst), (transposed));          \
     store_quad(v2, 2, (dst), (transposed)); store_quad(v3, 3, (dst), (transposed));          \
   } while (0)
+  const int wm = wave >> 1, wn = wave & 1;
+  // acc += opa^T opb over one 64-deep tile pair (k-major tiles of pitch LP)
+  auto mma_tile = [&](const T* opa, const T* opb, acc_t (&acc)[2][2]) __attribute__((always_inline)) {
+#pragma unroll 4
+    for (int ks = 0; ks < NB / 4; ++ks) {
+      const int k = ks * 4 + (lane >> 4);
+      T af[2], bfv[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = opa[k * LP + wm * 32 + i * 16 + (lane & 15)];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bfv[j] = opb[k * LP + wn * 32 + j * 16 + (lane & 15)];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
+    }
+  };
+  if (wg >= per) {
+    // ---- deferred trailing update only: tiles (ti, tc) of the lower triangle right of this block column, columns
+    // below c_end:  A[ti, tc] -= L[ti, p] L[tc, p]^T
+    const int jb = o / NB, nblk = (r + NB - 1) / NB, cblk = (c_end + NB - 1) / NB;
+    int u = wg - per;
+    const int stride = (int)gridDim.y - per;
+    int tc = jb + 1, left = nblk - tc;   // tiles of column block tc: row blocks tc .. nblk - 1
+    while (tc < cblk) {
+      if (u >= left) { u -= left; ++tc; --left; continue; }
+      const int ti = tc + u;
+      const int rows_ok = r - ti * NB < NB ? r - ti * NB : NB;
+      const int cols_ok = c_end - tc * NB < NB ? c_end - tc * NB : NB;
+      const int crow_ok = r - tc * NB < NB ? r - tc * NB : NB;
+      const T* lbase = Lmat + (long long)b * sG + o_prev;
+      tv4_t ua0, ua1, ua2, ua3, ub0, ub1, ub2, ub3;   // (of this iteration only)
+      DA_LOAD_TILE(ua0, ua1, ua2, ua3, lbase + (long long)ti * NB * r, rows_ok, NB);
+      DA_LOAD_TILE(ub0, ub1, ub2, ub3, lbase + (long long)tc * NB * r, crow_ok, NB);
+      __syncthreads();   // the previous tile's products are done with the buffers
+      DA_STORE_TILE(ua0, ua1, ua2, ua3, dT, true);   // opa[k][m] = L[ti, p][m][k]
+      DA_STORE_TILE(ub0, ub1, ub2, ub3, op, true);   // opb[k][n] = L[tc, p][n][k]
+      __syncthreads();
+      acc_t acc[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+      mma_tile(dT, op, acc);
+      T* dst = G + (long long)b * sG + (long long)ti * NB * r + (long long)tc * NB;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int m = wm * 32 + i * 16 + Mfma<T>::row(v, lane);
+            const int n = wn * 32 + j * 16 + (lane & 15);
+            if (m < rows_ok && n < cols_ok) dst[(long long)m * r + n] -= acc[i][j][v];
+          }
+      u += stride;
+    }
+    return;
+  }
+  if (defer) {
+    // L[j, p], k-major: the deferred update of the diagonal block below and of this workgroup's panel tiles
+    tv4_t lj0, lj1, lj2, lj3;
+    DA_LOAD_TILE(lj0, lj1, lj2, lj3, Lmat + (long long)b * sG + (long long)o * r + o_prev, nb, NB);
+    DA_STORE_TILE(lj0, lj1, lj2, lj3, ljT, true);
+  }
+  acc_t S[4], Y[4];
+#pragma unroll
+  for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int i = wave * 16 + Mfma<T>::row(v, lane), j = tj * 16 + lc;
+      // identity padding beyond nb keeps the padded part inert
+      S[tj][v] = (tj <= wave && i < nb && j < nb) ? g[(long long)i * r + j] : (i == j ? T(1) : T(0));
+      Y[tj][v] = (i == j) ? T(1) : T(0);
+    }
+  if (defer) {
+    __syncthreads();   // ljT is in place
+    // S -= L[j, p] L[j, p]^T on the wavefront's tile row (rows >= nb of ljT are zero: the padding stays inert)
+#pragma unroll 4
+    for (int ks = 0; ks < NB / 4; ++ks) {
+      const T* lk = ljT + (ks * 4 + lg) * LP;
+      const T aop = -lk[wave * 16 + lc];
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj)
+        if (tj <= wave) S[tj] = Mfma<T>::mma(aop, lk[tj * 16 + lc], S[tj]);
+    }
+  }
   // operand tiles of one term of T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]  (j = o / 64): L[j, k] and T[k, c]
   auto fetch_t = [&](int c, int k) __attribute__((always_inline)) {
     if (!INV) return;
@@ -130,10 +218,13 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
       return;
     }
     const int row0 = o + nb + (role - 1) * NB;
-    if (panel) DA_LOAD_TILE(pa0, pa1, pa2, pa3, G + (long long)b * sG + (long long)row0 * r + o, r - row0 < NB ? r - row0 : NB, nb);
-    else DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)o * r + (role - 1 - below) * NB, nb, NB);
+    if (panel) {
+      DA_LOAD_TILE(pa0, pa1, pa2, pa3, G + (long long)b * sG + (long long)row0 * r + o, r - row0 < NB ? r - row0 : NB, nb);
+      // (deferred update: L[i, p] as well)
+      if (defer) DA_LOAD_TILE(pb0, pb1, pb2, pb3, Lmat + (long long)b * sG + (long long)row0 * r + o_prev, r - row0 < NB ? r - row0 : NB, NB);
+    } else DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)o * r + (role - 1 - below) * NB, nb, NB);
   };
-  int role = blockIdx.x == 0 ? (int)gridDim.x : (int)blockIdx.x;   // this workgroup's first product
+  int role = wg == 0 ? per : wg;   // this workgroup's first product (`per` workgroups share the roles)
   // (the two tiles of a T role would stay in registers through the whole factor loop: those are requested after it)
   const bool early = role < nroles && !(INV && role > below);
   if (early) fetch(role);
@@ -227,7 +318,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
     if (wave == (cb & 3)) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) dT[lane * LP + k0 + k] = lane < nb ? xo.v[k] : T(0);
-      if (blockIdx.x == 0) {
+      if (wg == 0) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) op[lane * LP + k0 + k] = lfin.v[k];
       }
@@ -247,7 +338,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
   }
 
   // ---- the 64 x 64 x 64 products that depend on the factor: C[m][n] = sum_k opa[k][m] * opb[k][n]
-  if (blockIdx.x == 0) {
+  if (wg == 0) {
     T* l = Lmat + (long long)b * sG + (long long)o * r + o;
     T* w = (INV ? Tmat : Wmat) + (long long)b * sG + (long long)o * r + o;
     for (int e = tid; e < NB * NB; e += 256) {
@@ -260,23 +351,6 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
     // (`fresh`: the first block column of a factorisation starts the matrix's status word)
     if (tid == 0 && (fresh || (bad != 0 && info[b] == 0))) info[b] = bad;
   }
-  const int wm = wave >> 1, wn = wave & 1;
-  // acc += opa^T opb over one 64-deep tile pair (k-major tiles of pitch LP)
-  auto mma_tile = [&](const T* opa, const T* opb, acc_t (&acc)[2][2]) __attribute__((always_inline)) {
-#pragma unroll 4
-    for (int ks = 0; ks < NB / 4; ++ks) {
-      const int k = ks * 4 + (lane >> 4);
-      T af[2], bfv[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) af[i] = opa[k * LP + wm * 32 + i * 16 + (lane & 15)];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) bfv[j] = opb[k * LP + wn * 32 + j * 16 + (lane & 15)];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
-    }
-  };
   if (role < nroles && !early) fetch(role);
   while (role < nroles) {
     const bool panel = role <= below;
@@ -288,7 +362,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
-      const int next = role + (int)gridDim.x;
+      const int next = role + per;
       // the tile pairs alternate between two LDS buffers: pair k + 1 is requested before the product of pair k and
       // written after it (the registers live within one iteration)
       auto put = [&](int buf) __attribute__((always_inline)) {
@@ -336,10 +410,38 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
       role = next;
       continue;
     }
+    if (defer && panel) {
+      // the deferred update of this tile first:  A[i, j] -= L[i, p] L[j, p]^T
+      __syncthreads();                                 // `op` may still be read
+      DA_STORE_TILE(pb0, pb1, pb2, pb3, op, true);     // opa[k][m] = L[i, p][m][k]
+      __syncthreads();
+      acc_t du[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) du[i][j] = acc_t{0, 0, 0, 0};
+      mma_tile(op, ljT, du);
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            op[(wm * 32 + i * 16 + Mfma<T>::row(v, lane)) * LP + wn * 32 + j * 16 + (lane & 15)] = du[i][j][v];
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pa0[i] -= op[(trow + 0) * LP + tcol + i];
+        pa1[i] -= op[(trow + 16) * LP + tcol + i];
+        pa2[i] -= op[(trow + 32) * LP + tcol + i];
+        pa3[i] -= op[(trow + 48) * LP + tcol + i];
+      }
+    }
     __syncthreads();   // `op` may still be read (role 0's copy, the previous product's MFMAs)
     // panel: opa[k][m] = A[row0 + m][o + k];  W: opb[k][n] = L[o + k][col0 + n]
     DA_STORE_TILE(pa0, pa1, pa2, pa3, op, panel);
-    const int next = role + (int)gridDim.x;
+    const int next = role + per;
     if (next < nroles) fetch(next);   // in flight during this role's product
     __syncthreads();
     const int row0 = panel ? o + nb + (role - 1) * NB : o;
@@ -374,13 +476,14 @@ __global__ __launch_bounds__(256) void chol_step_kernel(const T* __restrict__ G,
 #undef DA_STORE_TILE
 
 template <typename T, bool INV>
-int chol_step(const T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int nb, int* info, int batch,
-              DaGate gate, bool fresh, hipStream_t s) {
+int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int nb, int* info, int batch,
+              DaGate gate, bool fresh, int o_prev, int c_end, hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  if (o_prev >= 0 && (o_prev != o - NB || c_end < o + nb || c_end > r)) return DA_ERR_ARG;
   const int rest = r - o - nb;
   if (rest > 0 && nb != NB) return DA_ERR_ARG;
   const int below = (rest + NB - 1) / NB;
-  const int smem = (INV ? 5 : 2) * NB * LP * (int)sizeof(T);
+  const int smem = ((INV ? 5 : 2) + 1) * NB * LP * (int)sizeof(T);   // (+ the tile of the deferred update)
   // workgroups per matrix: as many as fit one per CU over the batch (the factorisation every workgroup repeats is
   // bound by fp64 instruction issue, which two workgroups on a CU would share: 384 instead of 256 in flight cost
   // 3 % of the orthonormaliser on a 48-matrix bucket), never more than there are roles
@@ -394,23 +497,33 @@ int chol_step(const T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(per, batch), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r, o, nb, below, info,
-                     fresh ? 1 : 0, gate.flags, gate.want);
+  // update-only workgroups of a deferred trailing update: one per tile right of this block column (columns below
+  // c_end, lower triangle), at most 1024 over the batch
+  int extra = 0;
+  if (o_prev >= 0) {
+    const int jb = o / NB, nblk = (r + NB - 1) / NB, cblk = (c_end + NB - 1) / NB;
+    long long tiles = 0;
+    for (int tc = jb + 1; tc < cblk; ++tc) tiles += nblk - tc;
+    const long long cap = 1024 / batch > 1 ? 1024 / batch : 1;
+    extra = (int)(tiles < cap ? tiles : cap);
+  }
+  hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(batch, per + extra), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r, o, nb,
+                     below, info, fresh ? 1 : 0, gate.flags, gate.want, o_prev, c_end, per);
   return da_launch_status();
 }
 
 }  // namespace
 
-int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, DaGate gate, hipStream_t s) {
-  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, s);
+int da_chol_step(double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
+                 int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
+  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, o_prev, c_end, s);
 }
-int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
-                     int batch, DaGate gate, hipStream_t s) {
+int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
+                     int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
   // the fp32 pass keeps its status in a word of its own, which its first block column initialises
-  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, s);
+  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, s);
 }
-int da_chol_step_f32_inv(const float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
-                         int batch, DaGate gate, hipStream_t s) {
-  return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, s);
+int da_chol_step_f32_inv(float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
+                         int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
+  return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, s);
 }

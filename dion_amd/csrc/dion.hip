@@ -537,10 +537,14 @@ __global__ __launch_bounds__(256) void zero_cols_kernel(T* __restrict__ out, con
 
 inline int gemm_real(const Gemm64Desc& d, hipStream_t s) { return da_gemm_f64(d, s); }
 inline int gemm_real(const Gemm32Desc& d, hipStream_t s) { return da_gemm_f32s(d, s); }
-inline int chol_step_real(const double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info, int batch,
-                          DaGate g, hipStream_t s) { return da_chol_step(G, L, W, sG, r, o, nb, info, batch, g, s); }
-inline int chol_step_real(const float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info, int batch,
-                          DaGate g, hipStream_t s) { return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, g, s); }
+inline int chol_step_real(double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info, int batch,
+                          DaGate g, hipStream_t s, int o_prev, int c_end) {
+  return da_chol_step(G, L, W, sG, r, o, nb, info, batch, g, s, o_prev, c_end);
+}
+inline int chol_step_real(float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info, int batch,
+                          DaGate g, hipStream_t s, int o_prev, int c_end) {
+  return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, g, s, o_prev, c_end);
+}
 
 // G = P^T P (K-sliced if that fills the GPU; the slices are added in a fixed order), padded diagonal, and
 // optionally the rows' squared defects.
@@ -567,6 +571,9 @@ int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, floa
   return rc;
 }
 
+// Most 64 x 64 tiles (over the batch) a trailing update may have to ride along in the next step's launch.
+constexpr long long DA_CHOL_DEFER_TILES = 256;
+
 // One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
 template <typename T>
 int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, int r_live, int* info, DaGate gate,
@@ -585,14 +592,18 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
     return v > 0 ? v : 4;
   }();
   const int pw = pw_env;
+  // (the rank-64 updates inside a panel ride along in the next step's launch instead of taking one of their own)
+  static const bool defer = [] { const char* e = getenv("DION_AMD_CHOL_NO_DEFER"); return !(e && atoi(e)); }();
+  bool pending = false;   // the previous step left its update to the next launch
   // blocked lower Cholesky G = L L^T, building W alongside
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-    rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s);
-    if (rc) return rc;
-    if (rest <= 0) break;
     const int p0 = j / pw * pw * NB;                       // first column of the panel
     const int pe = p0 + pw * NB < r ? p0 + pw * NB : r;    // one past its last column
+    rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s, pending ? o - NB : -1, pe);
+    pending = false;
+    if (rc) return rc;
+    if (rest <= 0) break;
     RealGemmDesc<T> u{};
     u.batch = batch;
     u.sA = rr; u.lda = r; u.a_kstrided = 0;
@@ -601,6 +612,11 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
     u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
     u.gate = gate.flags; u.gate_want = gate.want;
     if (o + nb < pe) {
+      // A small update rides along in the next step's launch, which applies it where it needs it and has
+      // workgroups to spare for the rest (one 64 x 64 tile each); a large one is better off as a product of its own.
+      long long tiles = 0;
+      for (int tc = j + 1; tc * NB < pe; ++tc) tiles += nblk - tc;
+      if (defer && tiles * batch <= DA_CHOL_DEFER_TILES) { pending = true; continue; }
       // rest of the panel's columns, all rows from the diagonal down:  A[:, panel] -= L[:, j] L[panel, j]^T
       u.A = L + (long long)(o + nb) * r + o;
       u.B = u.A;
@@ -993,12 +1009,20 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   if (rc) return rc;
   // (the steps write the rows of L^-1 themselves: no W, no recurrence on the identity afterwards)
   static const bool inv_rows = [] { const char* e = getenv("DION_AMD_ORTH_NO_INV"); return !(e && atoi(e)); }();
+  // (every step's trailing update rides along in the next step's launch)
+  static const bool defer = [] { const char* e = getenv("DION_AMD_CHOL_NO_DEFER"); return !(e && atoi(e)); }();
+  bool pending = false;
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
-    rc = inv_rows ? da_chol_step_f32_inv(G, L, T, rr, r, o, nb, w.info32, batch, all, s)
-                  : da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s);
+    const int o_prev = pending ? o - NB : -1;
+    rc = inv_rows ? da_chol_step_f32_inv(G, L, T, rr, r, o, nb, w.info32, batch, all, s, o_prev, r)
+                  : da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s, o_prev, r);
+    pending = false;
     if (rc) return rc;
     if (rest <= 0) break;
+    // (small updates only: see cholqr_pass)
+    const long long below = nblk - j - 1;
+    if (defer && below * (below + 1) / 2 * batch <= DA_CHOL_DEFER_TILES) { pending = true; continue; }
     Gemm32Desc u{};
     u.batch = batch;
     u.A = L + (long long)(o + nb) * r + o; u.sA = rr; u.lda = r; u.a_kstrided = 0;

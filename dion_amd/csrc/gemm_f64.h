@@ -77,15 +77,19 @@ int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, i
 // diagonal, -D_j L[j, c] left of it).  A non-positive or non-finite pivot zeroes that column (of
 // L_jj and of D_j) and records (o + column + 1) in info[b] if it is the matrix's first failure.
 // `gate`: as in RealGemmDesc.
-int da_chol_step(const double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, DaGate gate, hipStream_t s);
-int da_chol_step_f32(const float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
-                     int batch, DaGate gate, hipStream_t s);
+// o_prev >= 0 (= o - 64): the trailing update of the previous step, A[i, c] -= L[i, p] L[c, p]^T with p the
+// block column at o_prev, has NOT been applied to G; this launch applies it to its own block column before
+// use and, with additional workgroups, to the columns o + nb .. c_end - 1 of the lower triangle (in G),
+// so that no separate update launch runs between two steps.  Columns >= c_end are left to the caller.
+int da_chol_step(double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
+                 int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
+int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
+                     int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
 // The same step, but instead of the row block of W it writes row block j of T = L^-1 itself into Tmat (lower
 // triangular, row-major): T[j, j] = D_j and T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c] for c < j, from the
 // rows of T that the earlier steps left.  After the last step Tmat holds L^-1 (blocks above the diagonal untouched).
-int da_chol_step_f32_inv(const float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
-                         int batch, DaGate gate, hipStream_t s);
+int da_chol_step_f32_inv(float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
+                         int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
 
 #define DA_CHOL_NB 64
 
