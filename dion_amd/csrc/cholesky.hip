@@ -51,7 +51,8 @@ template <typename T, bool INV>
 __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __restrict__ Lmat,
                                                         T* __restrict__ Wmat, T* __restrict__ Tmat, long long sG, int r,
                                                         int o, int nb, int below, int* __restrict__ info, int fresh,
-                                                        const int* gate, int gate_want, int o_prev, int c_end, int per) {
+                                                        const int* gate, int gate_want, int o_prev, int c_end, int per, int t_row, int n_t,
+                                                        int t_inline) {
   typedef typename Mfma<T>::acc_t acc_t;
   typedef Quad<T> quad_t;
   __shared__ __attribute__((aligned(16))) T scol[2][4][NB];     // published block column of S: [column][row]
@@ -76,7 +77,9 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
   // The workgroups of one matrix share its roles round-robin (role 0: L_jj, D_j and the status word; 1 .. below:
   // panel tiles; the rest: W tiles).  The operand tile of a product does not depend on this step's factor: it is
   // requested now, 16 elements per thread, and the next one while the previous product runs.
-  const int nroles = 1 + below + o / NB;
+  const int nroles = 1 + below + ((!INV || t_inline) ? o / NB : 0);
+  // row block of T that the T roles work on: this step's, or an earlier one in the workgroups that only do that
+  int t_o = o, t_nb = nb;
   // A 64 x 64 tile in registers: thread t holds the four elements (row (t >> 4) + 16 q, columns 4 (t & 15) .. + 3),
   // q = 0 .. 3 (named vectors, not an array: an array that one loop iteration writes and the next one reads ends up
   // in scratch memory).
@@ -135,12 +138,86 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
         for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::mma(af[i], bfv[j], acc[i][j]);
     }
   };
+  // operand tiles of one term of T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]  (j = o / 64): L[j, k] and T[k, c]
+  auto fetch_t = [&](int c, int k) __attribute__((always_inline)) {
+    if (!INV) return;
+    DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)t_o * r + (long long)k * NB, t_nb, NB);
+    DA_LOAD_TILE(pb0, pb1, pb2, pb3, Tmat + (long long)b * sG + (long long)k * NB * r + (long long)c * NB, NB, NB);
+  };
+  // Row block jb (rows t_o ..) of T = L^-1, column block c:  T[jb, c] = -D sum_{k = c .. jb-1} L[jb, k] T[k, c]  with
+  // D (transposed, in dT) the inverse of the row's diagonal block.  `have_first`: the first tile pair is already in
+  // the registers; next_role >= 0: that role's operand is requested before the last product.
+  auto t_tile = [&](int c, int jb, bool have_first, int next_role, auto fetch_next) __attribute__((always_inline)) {
+      acc_t acc[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+      // the tile pairs alternate between two LDS buffers: pair k + 1 is requested before the product of pair k and
+      // written after it (the registers live within one iteration)
+      auto put = [&](int buf) __attribute__((always_inline)) {
+        T* pa = op + buf * (2 * NB * LP);
+        DA_STORE_TILE(pa0, pa1, pa2, pa3, pa, true);              // opa[kk][m] = L[t_o + m][64 k + kk]
+        DA_STORE_TILE(pb0, pb1, pb2, pb3, pa + NB * LP, false);  // opb[kk][n] = T[64 k + kk][64 c + n]
+      };
+      if (!have_first) fetch_t(c, c);
+      __syncthreads();   // the buffers may still be read (role 0's copy, a previous product)
+      put(0);
+      for (int k = c; k < jb; ++k) {
+        const int buf = (k - c) & 1;
+        if (k + 1 < jb) fetch_t(c, k + 1);
+        __syncthreads();                                     // pair k is in place; the other buffer is free
+        mma_tile(op + buf * (2 * NB * LP), op + buf * (2 * NB * LP) + NB * LP, acc);
+        if (k + 1 < jb) put(buf ^ 1);
+      }
+      if (next_role >= 0) fetch_next(next_role);
+      T* const op2 = op + NB * LP;   // (buffer 0's second tile: free after the barrier below)
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            op2[(wm * 32 + i * 16 + Mfma<T>::row(v, lane)) * LP + wn * 32 + j * 16 + (lane & 15)] = acc[i][j][v];
+      __syncthreads();
+      acc_t res[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) res[i][j] = acc_t{0, 0, 0, 0};
+      mma_tile(dT, op2, res);
+      T* dst = Tmat + (long long)b * sG + (long long)t_o * r + (long long)c * NB;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int m = wm * 32 + i * 16 + Mfma<T>::row(v, lane);
+            const int n = wn * 32 + j * 16 + (lane & 15);
+            if (m < t_nb) dst[(long long)m * r + n] = -res[i][j][v];
+          }
+  };
+  if (INV && wg >= per && wg < per + n_t) {
+    // ---- rows of T only: block row t_row (a row whose diagonal block an earlier launch inverted), column blocks
+    // wg - per, + n_t, ...; its inverse diagonal block comes from Tmat
+    t_o = t_row * NB;
+    t_nb = r - t_o < NB ? r - t_o : NB;
+    {
+      tv4_t d0, d1, d2, d3;
+      DA_LOAD_TILE(d0, d1, d2, d3, Tmat + (long long)b * sG + (long long)t_o * r + t_o, t_nb, t_nb);
+      DA_STORE_TILE(d0, d1, d2, d3, dT, true);   // dT[k][x] = D[x][k]
+    }
+    for (int c = wg - per; c < t_row; c += n_t) t_tile(c, t_row, false, -1, [](int) {});
+    return;
+  }
   if (wg >= per) {
     // ---- deferred trailing update only: tiles (ti, tc) of the lower triangle right of this block column, columns
     // below c_end:  A[ti, tc] -= L[ti, p] L[tc, p]^T
     const int jb = o / NB, nblk = (r + NB - 1) / NB, cblk = (c_end + NB - 1) / NB;
-    int u = wg - per;
-    const int stride = (int)gridDim.y - per;
+    int u = wg - per - n_t;
+    const int stride = (int)gridDim.y - per - n_t;
     int tc = jb + 1, left = nblk - tc;   // tiles of column block tc: row blocks tc .. nblk - 1
     while (tc < cblk) {
       if (u >= left) { u -= left; ++tc; --left; continue; }
@@ -205,12 +282,6 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
         if (tj <= wave) S[tj] = Mfma<T>::mma(aop, lk[tj * 16 + lc], S[tj]);
     }
   }
-  // operand tiles of one term of T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]  (j = o / 64): L[j, k] and T[k, c]
-  auto fetch_t = [&](int c, int k) __attribute__((always_inline)) {
-    if (!INV) return;
-    DA_LOAD_TILE(pa0, pa1, pa2, pa3, Lmat + (long long)b * sG + (long long)o * r + (long long)k * NB, nb, NB);
-    DA_LOAD_TILE(pb0, pb1, pb2, pb3, Tmat + (long long)b * sG + (long long)k * NB * r + (long long)c * NB, NB, NB);
-  };
   auto fetch = [&](int role) __attribute__((always_inline)) {
     const bool panel = role <= below;
     if (INV && !panel) {
@@ -355,58 +426,8 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
   while (role < nroles) {
     const bool panel = role <= below;
     if (INV && !panel) {
-      // Row block j of T = L^-1, column block c:  T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c]
-      const int c = role - 1 - below, jb = o / NB;
-      acc_t acc[2][2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
       const int next = role + per;
-      // the tile pairs alternate between two LDS buffers: pair k + 1 is requested before the product of pair k and
-      // written after it (the registers live within one iteration)
-      auto put = [&](int buf) __attribute__((always_inline)) {
-        T* pa = op + buf * (2 * NB * LP);
-        DA_STORE_TILE(pa0, pa1, pa2, pa3, pa, true);              // opa[kk][m] = L[o + m][64 k + kk]
-        DA_STORE_TILE(pb0, pb1, pb2, pb3, pa + NB * LP, false);  // opb[kk][n] = T[64 k + kk][64 c + n]
-      };
-      __syncthreads();   // the buffers may still be read (role 0's copy, a previous product)
-      put(0);
-      for (int k = c; k < jb; ++k) {
-        const int buf = (k - c) & 1;
-        if (k + 1 < jb) fetch_t(c, k + 1);
-        __syncthreads();                                     // pair k is in place; the other buffer is free
-        mma_tile(op + buf * (2 * NB * LP), op + buf * (2 * NB * LP) + NB * LP, acc);
-        if (k + 1 < jb) put(buf ^ 1);
-      }
-      if (next < nroles) fetch(next);
-      T* const op2 = op + NB * LP;   // (buffer 0's second tile: free after the barrier below)
-      __syncthreads();
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int v = 0; v < 4; ++v)
-            op2[(wm * 32 + i * 16 + Mfma<T>::row(v, lane)) * LP + wn * 32 + j * 16 + (lane & 15)] = acc[i][j][v];
-      __syncthreads();
-      acc_t res[2][2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) res[i][j] = acc_t{0, 0, 0, 0};
-      mma_tile(dT, op2, res);
-      T* dst = Tmat + (long long)b * sG + (long long)o * r + (long long)c * NB;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const int m = wm * 32 + i * 16 + Mfma<T>::row(v, lane);
-            const int n = wn * 32 + j * 16 + (lane & 15);
-            if (m < nb) dst[(long long)m * r + n] = -res[i][j][v];
-          }
+      t_tile(role - 1 - below, o / NB, true, next < nroles ? next : -1, fetch);
       role = next;
       continue;
     }
@@ -477,7 +498,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
 
 template <typename T, bool INV>
 int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int nb, int* info, int batch,
-              DaGate gate, bool fresh, int o_prev, int c_end, hipStream_t s) {
+              DaGate gate, bool fresh, int o_prev, int c_end, int t_row, int t_inline, hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   if (o_prev >= 0 && (o_prev != o - NB || c_end < o + nb || c_end > r)) return DA_ERR_ARG;
   const int rest = r - o - nb;
@@ -487,7 +508,8 @@ int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int n
   // workgroups per matrix: as many as fit one per CU over the batch (the factorisation every workgroup repeats is
   // bound by fp64 instruction issue, which two workgroups on a CU would share: 384 instead of 256 in flight cost
   // 3 % of the orthonormaliser on a 48-matrix bucket), never more than there are roles
-  const int nroles = 1 + below + o / NB;
+  const int nroles = 1 + below + ((!INV || t_inline) ? o / NB : 0);
+  if (t_row >= 0 && (!INV || t_row < 1 || t_row * NB >= o)) return DA_ERR_ARG;   // an earlier row with tiles left of its diagonal
   int per = 256 / batch;
   if (per < 1) per = 1;
   if (per > nroles) per = nroles;
@@ -507,8 +529,14 @@ int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int n
     const long long cap = 1024 / batch > 1 ? 1024 / batch : 1;
     extra = (int)(tiles < cap ? tiles : cap);
   }
-  hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(batch, per + extra), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r, o, nb,
-                     below, info, fresh ? 1 : 0, gate.flags, gate.want, o_prev, c_end, per);
+  // workgroups for the row of T that lags behind: one per tile of the row, at most 512 over the batch
+  int n_t = 0;
+  if (t_row >= 1) {
+    const int cap = 512 / batch > 1 ? 512 / batch : 1;
+    n_t = t_row < cap ? t_row : cap;
+  }
+  hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(batch, per + n_t + extra), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r,
+                     o, nb, below, info, fresh ? 1 : 0, gate.flags, gate.want, o_prev, c_end, per, t_row, n_t, t_inline);
   return da_launch_status();
 }
 
@@ -516,14 +544,26 @@ int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int n
 
 int da_chol_step(double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
                  int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
-  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, o_prev, c_end, s);
+  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, o_prev, c_end, -1, 1, s);
 }
 int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
   // the fp32 pass keeps its status in a word of its own, which its first block column initialises
-  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, s);
+  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, -1, 1, s);
 }
 int da_chol_step_f32_inv(float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
-                         int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
-  return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, s);
+                         int batch, DaGate gate, hipStream_t s, int o_prev, int c_end, int t_row, int t_inline) {
+  return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, t_row,
+                                t_inline, s);
+}
+int da_chol_trow_f32(float* Lmat, float* Tmat, long long sG, int r, int t_row, int batch, DaGate gate, hipStream_t s) {
+  if (t_row < 1 || t_row * NB >= r || batch <= 0 || batch > 65535) return DA_ERR_ARG;
+  const int smem = 6 * NB * LP * (int)sizeof(float);
+  const int cap = 512 / batch > 1 ? 512 / batch : 1;
+  const int n_t = t_row < cap ? t_row : cap;
+  // (the attribute is set by the first factorisation step, which always precedes this launch)
+  hipLaunchKernelGGL((chol_step_kernel<float, true>), dim3(batch, n_t), dim3(256), smem, s, static_cast<float*>(nullptr), Lmat,
+                     static_cast<float*>(nullptr), Tmat, sG, r, t_row * NB, r - t_row * NB < NB ? r - t_row * NB : NB, 0,
+                     static_cast<int*>(nullptr), 0, gate.flags, gate.want, -1, 0, 0, t_row, n_t, 0);
+  return da_launch_status();
 }

@@ -1011,11 +1011,15 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   static const bool inv_rows = [] { const char* e = getenv("DION_AMD_ORTH_NO_INV"); return !(e && atoi(e)); }();
   // (every step's trailing update rides along in the next step's launch)
   static const bool defer = [] { const char* e = getenv("DION_AMD_CHOL_NO_DEFER"); return !(e && atoi(e)); }();
+  static const bool lag_on = [] { const char* e = getenv("DION_AMD_CHOL_NO_TLAG"); return !(e && atoi(e)); }();
+  const bool lag = inv_rows && lag_on && nblk >= 4;   // (short chains: the extra launch at the end costs what the lag saves)
   bool pending = false;
   for (int j = 0; j < nblk; ++j) {
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
     const int o_prev = pending ? o - NB : -1;
-    rc = inv_rows ? da_chol_step_f32_inv(G, L, T, rr, r, o, nb, w.info32, batch, all, s, o_prev, r)
+    // (the rows of L^-1 lag one step behind: row j - 1 is formed by workgroups of step j's launch that do nothing else)
+    rc = inv_rows ? da_chol_step_f32_inv(G, L, T, rr, r, o, nb, w.info32, batch, all, s, o_prev, r,
+                                         lag && j >= 2 ? j - 1 : -1, lag ? 0 : 1)
                   : da_chol_step_f32(G, L, W, rr, r, o, nb, w.info32, batch, all, s, o_prev, r);
     pending = false;
     if (rc) return rc;
@@ -1031,6 +1035,10 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
     u.E = u.C; u.sE = rr; u.lde = r;
     u.M = rest; u.N = rest; u.K = nb; u.alpha = -1.0; u.beta = 1.0; u.lower_only = 1;
     rc = da_gemm_f32s(u, s);
+    if (rc) return rc;
+  }
+  if (lag) {
+    rc = da_chol_trow_f32(L, T, rr, r, nblk - 1, batch, all, s);
     if (rc) return rc;
   }
   if (!inv_rows) {

@@ -88,8 +88,14 @@ int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, in
 // The same step, but instead of the row block of W it writes row block j of T = L^-1 itself into Tmat (lower
 // triangular, row-major): T[j, j] = D_j and T[j, c] = -D_j sum_{k = c .. j-1} L[j, k] T[k, c] for c < j, from the
 // rows of T that the earlier steps left.  After the last step Tmat holds L^-1 (blocks above the diagonal untouched).
+// t_inline = 0: the step leaves the tiles of its row of T left of the diagonal to a later launch (it writes D_j only);
+// t_row >= 1: additional workgroups of this launch form those tiles of block row t_row (t_row < j: its D and all rows
+// above it are complete), so that the rows of T lag one step behind the factorisation instead of lengthening it.
+// da_chol_trow_f32 is that work alone, for the row that is still missing after the last step.
 int da_chol_step_f32_inv(float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
-                         int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
+                         int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0, int t_row = -1,
+                         int t_inline = 1);
+int da_chol_trow_f32(float* Lmat, float* Tmat, long long sG, int r, int t_row, int batch, DaGate gate, hipStream_t s);
 
 #define DA_CHOL_NB 64
 
