@@ -591,7 +591,10 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
     const int v = e ? atoi(e) : 0;
     return v > 0 ? v : 4;
   }();
-  const int pw = pw_env;
+  // As the pass for flagged matrices only (gated), most launches find nothing to do and what counts is their number:
+  // one level, every trailing update deferred into the next step's launch.
+  const bool fallback = gate.flags != nullptr;
+  const int pw = fallback ? nblk : pw_env;
   // (the rank-64 updates inside a panel ride along in the next step's launch instead of taking one of their own)
   static const bool defer = [] { const char* e = getenv("DION_AMD_CHOL_NO_DEFER"); return !(e && atoi(e)); }();
   bool pending = false;   // the previous step left its update to the next launch
@@ -616,7 +619,7 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
       // workgroups to spare for the rest (one 64 x 64 tile each); a large one is better off as a product of its own.
       long long tiles = 0;
       for (int tc = j + 1; tc * NB < pe; ++tc) tiles += nblk - tc;
-      if (defer && tiles * batch <= DA_CHOL_DEFER_TILES) { pending = true; continue; }
+      if (defer && (fallback || tiles * batch <= DA_CHOL_DEFER_TILES)) { pending = true; continue; }
       // rest of the panel's columns, all rows from the diagonal down:  A[:, panel] -= L[:, j] L[panel, j]^T
       u.A = L + (long long)(o + nb) * r + o;
       u.B = u.A;
