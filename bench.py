@@ -462,7 +462,7 @@ def main():
             if name == args.workload:
                 continue
             w = WORKLOADS[name]
-            big = "llama" in name
+            big = name in ("muon_llama8b", "dion_llama70b_mlp")   # hundreds of ms and tens of GB per step
             r = measure(w, dev, 3 if big else 10, 1 if big else 2)
             s = summarize(name, w, r)
             s["roofline"] = roofline_of(r, w["kind"], name)
