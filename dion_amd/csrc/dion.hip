@@ -572,7 +572,7 @@ int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, floa
 }
 
 // Most 64 x 64 tiles (over the batch) a trailing update may have to ride along in the next step's launch.
-constexpr long long DA_CHOL_DEFER_TILES = 256;
+const long long DA_CHOL_DEFER_TILES = [] { const char* e = getenv("DION_AMD_CHOL_DEFER_TILES"); const long long v = e ? atoll(e) : 0; return v > 0 ? v : 256; }();
 
 // One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
 template <typename T>
