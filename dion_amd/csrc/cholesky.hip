@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
                                                         T* __restrict__ Wmat, T* __restrict__ Tmat, long long sG, int r,
                                                         int o, int nb, int below, int* __restrict__ info, int fresh,
                                                         const int* gate, int gate_want, int o_prev, int c_end, int per, int t_row, int n_t,
-                                                        int t_inline) {
+                                                        int t_inline, T* __restrict__ pstat) {
   typedef typename Mfma<T>::acc_t acc_t;
   typedef Quad<T> quad_t;
   __shared__ __attribute__((aligned(16))) T scol[2][4][NB];     // published block column of S: [column][row]
@@ -331,6 +331,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
 
   constexpr int NEWTON = sizeof(T) == 8 ? 2 : 0;   // the hardware estimate is good to 1 ulp in fp32, ~2^-27 in fp64
   int bad = 0;                                     // first failed pivot (every lane computes the same)
+  T pmin = T(3e38), pmax = T(0);                   // smallest and largest usable pivot of this block column
   for (int cb = 0; cb < NB / 4; ++cb) {
     const int buf = cb & 1, k0 = cb * 4;
     quad_t sv;                             // lane = row: S[lane][k0 ..]
@@ -357,6 +358,10 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
       for (int it = 0; it < NEWTON; ++it) rs = rs * (T(1.5) - T(0.5) * p * rs * rs);
       di[c] = ok ? rs : T(0);
       bad = (!ok && bad == 0 && k0 + c < nb) ? o + k0 + c + 1 : bad;
+      if (ok && k0 + c < nb) {
+        pmin = p < pmin ? p : pmin;
+        pmax = p > pmax ? p : pmax;
+      }
 #pragma unroll
       for (int i = c + 1; i < 4; ++i) a[i][c] *= di[c];
 #pragma unroll
@@ -421,6 +426,16 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
     }
     // (`fresh`: the first block column of a factorisation starts the matrix's status word)
     if (tid == 0 && (fresh || (bad != 0 && info[b] == 0))) info[b] = bad;
+    // pivot range of the matrix so far (the squares of R's diagonal: their ratio bounds cond(R)^2 from below)
+    if (tid == 0 && pstat) {
+      T mn = pmin, mx = pmax;
+      if (o > 0) {
+        mn = pstat[2 * b] < mn ? pstat[2 * b] : mn;
+        mx = pstat[2 * b + 1] > mx ? pstat[2 * b + 1] : mx;
+      }
+      pstat[2 * b] = mn;
+      pstat[2 * b + 1] = mx;
+    }
   }
   if (role < nroles && !early) fetch(role);
   while (role < nroles) {
@@ -498,7 +513,7 @@ __global__ __launch_bounds__(256) void chol_step_kernel(T* __restrict__ G, T* __
 
 template <typename T, bool INV>
 int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int nb, int* info, int batch,
-              DaGate gate, bool fresh, int o_prev, int c_end, int t_row, int t_inline, hipStream_t s) {
+              DaGate gate, bool fresh, int o_prev, int c_end, int t_row, int t_inline, T* pstat, hipStream_t s) {
   if (nb <= 0 || nb > NB || o < 0 || o + nb > r || (o % NB) != 0 || batch <= 0 || batch > 65535) return DA_ERR_ARG;
   if (o_prev >= 0 && (o_prev != o - NB || c_end < o + nb || c_end > r)) return DA_ERR_ARG;
   const int rest = r - o - nb;
@@ -536,25 +551,25 @@ int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int n
     n_t = t_row < cap ? t_row : cap;
   }
   hipLaunchKernelGGL((chol_step_kernel<T, INV>), dim3(batch, per + n_t + extra), dim3(256), smem, s, G, Lmat, Wmat, Tmat, sG, r,
-                     o, nb, below, info, fresh ? 1 : 0, gate.flags, gate.want, o_prev, c_end, per, t_row, n_t, t_inline);
+                     o, nb, below, info, fresh ? 1 : 0, gate.flags, gate.want, o_prev, c_end, per, t_row, n_t, t_inline, pstat);
   return da_launch_status();
 }
 
 }  // namespace
 
 int da_chol_step(double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
-  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, o_prev, c_end, -1, 1, s);
+                 int batch, DaGate gate, hipStream_t s, int o_prev, int c_end, double* pstat) {
+  return chol_step<double, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, false, o_prev, c_end, -1, 1, pstat, s);
 }
 int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s, int o_prev, int c_end) {
   // the fp32 pass keeps its status in a word of its own, which its first block column initialises
-  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, -1, 1, s);
+  return chol_step<float, false>(G, Lmat, Wmat, nullptr, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, -1, 1, nullptr, s);
 }
 int da_chol_step_f32_inv(float* G, float* Lmat, float* Tmat, long long sG, int r, int o, int nb, int* info,
                          int batch, DaGate gate, hipStream_t s, int o_prev, int c_end, int t_row, int t_inline) {
   return chol_step<float, true>(G, Lmat, nullptr, Tmat, sG, r, o, nb, info, batch, gate, o == 0, o_prev, c_end, t_row,
-                                t_inline, s);
+                                t_inline, nullptr, s);
 }
 int da_chol_trow_f32(float* Lmat, float* Tmat, long long sG, int r, int t_row, int batch, DaGate gate, hipStream_t s) {
   if (t_row < 1 || t_row * NB >= r || batch <= 0 || batch > 65535) return DA_ERR_ARG;
@@ -564,6 +579,6 @@ int da_chol_trow_f32(float* Lmat, float* Tmat, long long sG, int r, int t_row, i
   // (the attribute is set by the first factorisation step, which always precedes this launch)
   hipLaunchKernelGGL((chol_step_kernel<float, true>), dim3(batch, n_t), dim3(256), smem, s, static_cast<float*>(nullptr), Lmat,
                      static_cast<float*>(nullptr), Tmat, sG, r, t_row * NB, r - t_row * NB < NB ? r - t_row * NB : NB, 0,
-                     static_cast<int*>(nullptr), 0, gate.flags, gate.want, -1, 0, 0, t_row, n_t, 0);
+                     static_cast<int*>(nullptr), 0, gate.flags, gate.want, -1, 0, 0, t_row, n_t, 0, static_cast<float*>(nullptr));
   return da_launch_status();
 }

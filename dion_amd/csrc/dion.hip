@@ -421,6 +421,9 @@ struct OrthWs {
   int* need;       // per matrix: 1 = the fp32 pass was not enough, the fp64 pass runs
   int* info32;     // per matrix: status of the fp32 factorisation
   int* bad;        // r per matrix: 1 = the column is not usable (noise-level pivot), it is zeroed
+  double* pstat;   // 2 per matrix: smallest and largest pivot of the fp64 factorisation
+  int* polish;     // per matrix: 1 = the fp64 pass's result goes through the polishing pass
+  int* direct;     // per matrix: 1 = it is the result as it is
   size_t bytes;
   OrthWs(void* ws, int batch, int rows, int r) {
     const size_t pr = (size_t)rows * r * batch, rr = (size_t)r * r * batch;
@@ -442,6 +445,9 @@ struct OrthWs {
     need = reinterpret_cast<int*>(take((size_t)batch * 4));
     info32 = reinterpret_cast<int*>(take((size_t)batch * 4));
     bad = reinterpret_cast<int*>(take((size_t)r * batch * 4));
+    pstat = reinterpret_cast<double*>(take((size_t)batch * 16));
+    polish = reinterpret_cast<int*>(take((size_t)batch * 4));
+    direct = reinterpret_cast<int*>(take((size_t)batch * 4));
     bytes = (size_t)(p - static_cast<char*>(ws));
   }
 };
@@ -538,11 +544,11 @@ __global__ __launch_bounds__(256) void zero_cols_kernel(T* __restrict__ out, con
 inline int gemm_real(const Gemm64Desc& d, hipStream_t s) { return da_gemm_f64(d, s); }
 inline int gemm_real(const Gemm32Desc& d, hipStream_t s) { return da_gemm_f32s(d, s); }
 inline int chol_step_real(double* G, double* L, double* W, long long sG, int r, int o, int nb, int* info, int batch,
-                          DaGate g, hipStream_t s, int o_prev, int c_end) {
-  return da_chol_step(G, L, W, sG, r, o, nb, info, batch, g, s, o_prev, c_end);
+                          DaGate g, hipStream_t s, int o_prev, int c_end, double* pstat) {
+  return da_chol_step(G, L, W, sG, r, o, nb, info, batch, g, s, o_prev, c_end, pstat);
 }
 inline int chol_step_real(float* G, float* L, float* W, long long sG, int r, int o, int nb, int* info, int batch,
-                          DaGate g, hipStream_t s, int o_prev, int c_end) {
+                          DaGate g, hipStream_t s, int o_prev, int c_end, float*) {
   return da_chol_step_f32(G, L, W, sG, r, o, nb, info, batch, g, s, o_prev, c_end);
 }
 
@@ -577,7 +583,7 @@ const long long DA_CHOL_DEFER_TILES = [] { const char* e = getenv("DION_AMD_CHOL
 // One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
 template <typename T>
 int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, int r_live, int* info, DaGate gate,
-                hipStream_t s) {
+                hipStream_t s, T* pstat = nullptr) {
   const int NB = DA_CHOL_NB;
   const int nblk = (r + NB - 1) / NB;
   const long long pr = (long long)rows * r, rr = (long long)r * r;
@@ -603,7 +609,7 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
     const int o = j * NB, nb = r - o < NB ? r - o : NB, rest = r - o - nb;
     const int p0 = j / pw * pw * NB;                       // first column of the panel
     const int pe = p0 + pw * NB < r ? p0 + pw * NB : r;    // one past its last column
-    rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s, pending ? o - NB : -1, pe);
+    rc = chol_step_real(G, L, W, rr, r, o, nb, info, batch, gate, s, pending ? o - NB : -1, pe, pstat);
     pending = false;
     if (rc) return rc;
     if (rest <= 0) break;
@@ -1100,6 +1106,22 @@ int fast16_pass(const bf16_t* P, const OrthWs& w, int batch, int rows, int r, in
   return gram16(w.Ph, Lo, G, part, batch, rows, r, r_live, w.rowdef, w.rowdef_part, all, s);
 }
 
+// After the fp64 factorisation: which of the matrices it ran for need the polishing pass.  The pivots are the
+// squares of R's diagonal, so pmax / pmin <= cond(R)^2 = cond(P)^2; with pmin >= ratio * pmax and no failed pivot the
+// defect the fp64 pass leaves, eps64 * cond(P)^2, is far below what the result's dtype resolves even if cond(P) is
+// a hundred times the estimate, and the result is converted as it is.
+__global__ void decide_polish_kernel(const double* __restrict__ pstat, const int* __restrict__ info,
+                                     const int* gate, int want, int* __restrict__ polish, int* __restrict__ direct,
+                                     int batch, double ratio) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  const bool open = orth_gate_open(gate, want, b);
+  const double mn = pstat[2 * b], mx = pstat[2 * b + 1];
+  const bool healthy = info[b] == 0 && mn >= ratio * mx && mx > 0.0;   // (false for NaN)
+  polish[b] = open && !healthy ? 1 : 0;
+  direct[b] = open && healthy ? 1 : 0;
+}
+
 // bf16 copy of the matrices whose gate is open
 __global__ __launch_bounds__(256) void copy_bf16_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst,
                                                         long long per, const int* gate, int want) {
@@ -1119,6 +1141,10 @@ __global__ void decide_cqr_kernel(const int* __restrict__ info32, int* __restric
 // Defect ||P^T P - I||_F up to which the closed-form polishing pass is trusted after the fp32 pass: it leaves
 // about 3 E^2, i.e. 1e-5.
 constexpr float FAST_TOL = 2e-3f;
+// Smallest pivot, relative to the largest, with which the fp64 pass's result needs no polishing pass: the pivot range
+// then puts cond(P) at 3e3 or more below, eps64 * cond^2 at 1e-9 -- and at 1e-5 if the estimate is a hundred times
+// too low.
+constexpr double POLISH_PIVOT_RATIO = 1e-7;
 
 }  // namespace
 
@@ -1213,9 +1239,22 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   const DaGate gate = fast ? DaGate{w.need, 1} : all;
   rc = da_cvt_to_f64(P, dtype, w.P0, pr, batch, gate, s);
   if (rc) return rc;
-  rc = cholqr_pass<double>(w.P0, w.G, w.L, w.W, w.part, batch, rows, r, r_live, info, gate, s);
+  rc = cholqr_pass<double>(w.P0, w.G, w.L, w.W, w.part, batch, rows, r, r_live, info, gate, s, w.pstat);
   if (rc) return rc;
   if (passes == 1) return da_cvt_from_f64(w.P0, out, dtype, pr, batch, gate, s);
+  // One polishing pass (the optimizer's case) is for factors whose conditioning leaves a visible defect even in fp64
+  // and for noise-level pivots: the pivot range tells on the device which matrices those are; the others are done.
+  static const bool always_polish = getenv("DION_AMD_ORTH_ALWAYS_POLISH") != nullptr;
+  const DaGate whole = gate;   // every matrix of the fp64 pass
+  if (passes == 2 && !always_polish) {
+    hipLaunchKernelGGL(decide_polish_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, w.pstat, info, gate.flags,
+                       gate.want, w.polish, w.direct, batch, POLISH_PIVOT_RATIO);
+    rc = da_launch_status();
+    if (rc) return rc;
+    rc = da_cvt_from_f64(w.P0, out, dtype, pr, batch, DaGate{w.direct, 1}, s);
+    if (rc) return rc;
+  }
+  const DaGate gate2 = passes == 2 && !always_polish ? DaGate{w.polish, 1} : whole;
   float* Gf = reinterpret_cast<float*>(w.G);
   const bool last_low = passes == 2 && low;
   // A bf16 result after one polishing pass needs the fp64 pass's result to 16 bits only, as h + l (bf16 each): the
@@ -1224,34 +1263,34 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   // polishing products.
   const bool hl = last_low && dtype == DA_BF16 && !no16;
   bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
-  rc = hl ? da_cvt_f64_to_hl(w.P0, w.Ph, Lo, pr, batch, gate, s)
-          : da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate, s);
+  rc = hl ? da_cvt_f64_to_hl(w.P0, w.Ph, Lo, pr, batch, gate2, s)
+          : da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate2, s);
   if (rc) return rc;
   const float* cur = w.Pf;
   for (int pass = 1; pass < passes; ++pass) {
     const bool last = pass + 1 == passes;
-    rc = hl ? gram16(w.Ph, Lo, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, w.rowdef_part, gate, s)
-            : gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate, s);
+    rc = hl ? gram16(w.Ph, Lo, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, w.rowdef_part, gate2, s)
+            : gram<float>(cur, Gf, reinterpret_cast<float*>(w.part), batch, rows, r, r_live, w.rowdef, gate2, s);
     if (rc) return rc;
     const int* bad = nullptr;
     if (pass == 1) {
       hipLaunchKernelGGL(decide_cols_kernel, dim3((unsigned)batch), dim3(256), 0, s, w.rowdef, w.bad, info, r,
-                         gate.flags, gate.want);
+                         gate2.flags, gate2.want);
       rc = da_launch_status();
       if (rc) return rc;
       bad = w.bad;
     }
     if (last && last_low) {
-      rc = correction_bf16(cur, w.Ph, out, dtype, Gf, reinterpret_cast<bf16_t*>(w.L), bad, batch, rows, r, gate,
+      rc = correction_bf16(cur, w.Ph, out, dtype, Gf, reinterpret_cast<bf16_t*>(w.L), bad, batch, rows, r, gate2,
                            FastVerdict{nullptr, nullptr, nullptr, 0.f}, s);
     } else {
       // intermediate iterates alternate between the fp32 buffer and (as fp32) the no longer needed P0
       float* other = cur == w.Pf ? reinterpret_cast<float*>(w.P0) : w.Pf;
       rc = correction_f32(cur, last ? out : static_cast<void*>(other), last ? da_store_of(dtype) : DA_STORE_NATIVE, Gf,
-                          reinterpret_cast<float*>(w.L), bad, batch, rows, r, gate, s);
+                          reinterpret_cast<float*>(w.L), bad, batch, rows, r, gate2, s);
       cur = other;
     }
     if (rc) return rc;
   }
-  return zero_cols(out, dtype, w.bad, info, batch, rows, r, gate, s);
+  return zero_cols(out, dtype, w.bad, info, batch, rows, r, gate2, s);
 }

@@ -81,8 +81,10 @@ int da_cvt_from_f32(const float* src, void* dst, int dst_dtype, long long per, i
 // block column at o_prev, has NOT been applied to G; this launch applies it to its own block column before
 // use and, with additional workgroups, to the columns o + nb .. c_end - 1 of the lower triangle (in G),
 // so that no separate update launch runs between two steps.  Columns >= c_end are left to the caller.
+// pstat (fp64 form, may be null): two words per matrix, the smallest and the largest pivot met so far (step o == 0
+// starts them): the squares of R's diagonal, whose ratio bounds cond(R)^2 from below.
 int da_chol_step(double* G, double* Lmat, double* Wmat, long long sG, int r, int o, int nb, int* info,
-                 int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
+                 int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0, double* pstat = nullptr);
 int da_chol_step_f32(float* G, float* Lmat, float* Wmat, long long sG, int r, int o, int nb, int* info,
                      int batch, DaGate gate, hipStream_t s, int o_prev = -1, int c_end = 0);
 // The same step, but instead of the row block of W it writes row block j of T = L^-1 itself into Tmat (lower
