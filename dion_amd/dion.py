@@ -12,7 +12,9 @@ error-feedback and weight updates fused into GEMM epilogues, and the column norm
 that yields the next Q.
 """
 import math
+import os
 from collections import defaultdict
+from concurrent.futures import ThreadPoolExecutor
 from dataclasses import dataclass
 from typing import Any, Dict, Optional, Tuple
 
@@ -31,6 +33,13 @@ class DionMixedPrecisionConfig:
     momentum_dtype: Optional[torch.dtype] = None
     Q_dtype: Optional[torch.dtype] = None
     variance_dtype: Optional[torch.dtype] = None
+
+
+
+def _enqueue_dion_step(lib, device, args):
+    """One bucket's library call, made by a worker thread (ctypes releases the interpreter lock for its duration)."""
+    torch.cuda.set_device(device)
+    return lib.dion_amd_dion_step_qr(*args)
 
 
 class Dion(Optimizer):
@@ -126,6 +135,7 @@ class Dion(Optimizer):
         self._workspaces = [_lib.Workspace() for _ in range(self._max_concurrent_tasks)]
         self._streams = {}
         self._info = {}
+        self._pool = None   # worker threads that enqueue the buckets of a wave side by side
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -252,61 +262,90 @@ class Dion(Optimizer):
             if info is None or info.numel() != len(plist):
                 self._info[key] = torch.zeros(len(plist), dtype=torch.int32, device=device)
         slots = min(len(buckets), self._max_concurrent_tasks)
+        # A bucket's step is one library call that enqueues a few hundred launches on the bucket's stream.  With
+        # several buckets the calls of a wave (one bucket per stream) are made by worker threads side by side: at a
+        # low rank the step is otherwise bound by the time one thread needs to enqueue it, not by the GPU.
+        threaded = (slots > 1 and not os.environ.get("DION_AMD_DION_SERIAL")
+                    and not torch.cuda.is_current_stream_capturing())
+        if threaded and getattr(self, "_pool", None) is None:
+            self._pool = ThreadPoolExecutor(max_workers=self._max_concurrent_tasks, thread_name_prefix="dion_amd")
         forked = {}
-        for index, ((shape, dtype, gdtype, device), plist) in enumerate(buckets.items()):
-            slot = index % slots
-            main = torch.cuda.current_stream(device)
-            if slots == 1:
-                stream = main
-            else:
-                pool = self._streams.setdefault(device, [])
-                while len(pool) < slots:
-                    pool.append(torch.cuda.Stream(device=device))
-                stream = pool[slot]
-                if (device, slot) not in forked:
-                    stream.wait_stream(main)   # gradients and earlier updates were produced on `main`
-                    forked[(device, slot)] = (main, stream)
-            states = [self._get_or_initialize_state(p, group) for p in plist]
-            m, n = shape
-            Ms = [s["momentum"] for s in states]
-            Qs = [s["Q"] for s in states]
-            r = Qs[0].size(1)
-            for t in (*plist, *Ms, *Qs):
-                if not t.is_contiguous():
-                    raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
-            scaled_lr = ((m / n) ** 0.5) * lr
-            mcode = _lib.dtype_code(Ms[0].dtype)
-            info = self._info[(shape, dtype, gdtype, device)]
-            with torch.cuda.device(device), torch.cuda.stream(stream):
-                # contiguous gradient copies and the workspace belong to this stream
-                Xs = plist
-                Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
-                crops = []
-                if m % 8 or n % 8:
-                    # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
-                    m, n = _lib.padded_dims(m, n)
-                    Xw, Gw, Mw = (_lib.zero_padded(t, m, n) for t in (plist, Gs, Ms))
-                    Qw = _lib.zero_padded(Qs, min(m, n), r)
-                    crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
-                    Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
-                ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
-                # Cholesky QR only after the warm-up, when the factors are well conditioned
-                # (reference dion/dion_reference.py:296-299)
-                qr_method = self._qr_method
-                if qr_method == "cqr" and group["step"] <= self._cqr_warmup_steps:
-                    qr_method = "rcqr"
-                rc = lib.dion_amd_dion_step_qr(
-                    _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
-                    len(plist), m, n, r,
-                    _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
-                    ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
-                    _lib.QR_METHODS[qr_method],
-                    info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
-                )
-                _lib.check(rc, "dion_amd_dion_step_qr")
-                for dst, padded in crops:
-                    _lib.crop_back(dst, padded)
-                del Xs, Gs, Ms, Qs, crops
+        items = list(buckets.items())
+        for wave0 in range(0, len(items), slots):
+            pending = []
+            for index in range(wave0, min(wave0 + slots, len(items))):
+                (shape, dtype, gdtype, device), plist = items[index]
+                slot = index % slots
+                main = torch.cuda.current_stream(device)
+                if slots == 1:
+                    stream = main
+                else:
+                    pool = self._streams.setdefault(device, [])
+                    while len(pool) < slots:
+                        pool.append(torch.cuda.Stream(device=device))
+                    stream = pool[slot]
+                    if (device, slot) not in forked:
+                        stream.wait_stream(main)   # gradients and earlier updates were produced on `main`
+                        forked[(device, slot)] = (main, stream)
+                states = [self._get_or_initialize_state(p, group) for p in plist]
+                m, n = shape
+                Ms = [s["momentum"] for s in states]
+                Qs = [s["Q"] for s in states]
+                r = Qs[0].size(1)
+                for t in (*plist, *Ms, *Qs):
+                    if not t.is_contiguous():
+                        raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
+                scaled_lr = ((m / n) ** 0.5) * lr
+                mcode = _lib.dtype_code(Ms[0].dtype)
+                info = self._info[(shape, dtype, gdtype, device)]
+                with torch.cuda.device(device), torch.cuda.stream(stream):
+                    # contiguous gradient copies and the workspace belong to this stream
+                    Xs = plist
+                    Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
+                    crops = []
+                    if m % 8 or n % 8:
+                        # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
+                        m, n = _lib.padded_dims(m, n)
+                        Xw, Gw, Mw = (_lib.zero_padded(t, m, n) for t in (plist, Gs, Ms))
+                        Qw = _lib.zero_padded(Qs, min(m, n), r)
+                        crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
+                        Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
+                    ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
+                    # Cholesky QR only after the warm-up, when the factors are well conditioned
+                    # (reference dion/dion_reference.py:296-299)
+                    qr_method = self._qr_method
+                    if qr_method == "cqr" and group["step"] <= self._cqr_warmup_steps:
+                        qr_method = "rcqr"
+                    args = (
+                        _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
+                        len(plist), m, n, r,
+                        _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
+                        ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
+                        _lib.QR_METHODS[qr_method],
+                        info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
+                    )
+                    if threaded:
+                        # (the tensors behind the pointers stay referenced until the call has returned)
+                        pending.append((self._pool.submit(_enqueue_dion_step, lib, device, args), device, stream, crops,
+                                        (Xs, Gs, Ms, Qs, ws)))
+                        continue
+                    rc = lib.dion_amd_dion_step_qr(*args)
+                    _lib.check(rc, "dion_amd_dion_step_qr")
+                    for dst, padded in crops:
+                        _lib.crop_back(dst, padded)
+                    del Xs, Gs, Ms, Qs, crops
+            failure = None
+            for future, device, stream, crops, keep in pending:
+                rc = future.result()   # every call of the wave has returned before anything is raised
+                if rc != 0 and failure is None:
+                    failure = rc
+                if rc == 0 and crops:
+                    with torch.cuda.device(device), torch.cuda.stream(stream):
+                        for dst, padded in crops:
+                            _lib.crop_back(dst, padded)
+            del pending
+            if failure is not None:
+                _lib.check(failure, "dion_amd_dion_step_qr")
         for main, stream in forked.values():
             main.wait_stream(stream)
 
