@@ -1244,7 +1244,10 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   if (passes == 1) return da_cvt_from_f64(w.P0, out, dtype, pr, batch, gate, s);
   // One polishing pass (the optimizer's case) is for factors whose conditioning leaves a visible defect even in fp64
   // and for noise-level pivots: the pivot range tells on the device which matrices those are; the others are done.
-  static const bool always_polish = getenv("DION_AMD_ORTH_ALWAYS_POLISH") != nullptr;
+  // (not as the fall-back of an fp32 pass: those matrices were flagged for their conditioning, and the launches that
+  // find nothing to do should be few)
+  static const bool always_polish_env = getenv("DION_AMD_ORTH_ALWAYS_POLISH") != nullptr;
+  const bool always_polish = always_polish_env || fast;
   const DaGate whole = gate;   // every matrix of the fp64 pass
   if (passes == 2 && !always_polish) {
     hipLaunchKernelGGL(decide_polish_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, w.pstat, info, gate.flags,
