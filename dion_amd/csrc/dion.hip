@@ -557,7 +557,8 @@ inline int chol_step_real(float* G, float* L, float* W, long long sG, int r, int
 template <typename T>
 int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, float* rowdef, DaGate gate, hipStream_t s) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
-  const int sp = gram_slices(batch, rows, r);
+  // (as the fall-back of flagged matrices: unsliced, so that no finishing launch is needed)
+  const int sp = gate.flags ? 1 : gram_slices(batch, rows, r);
   RealGemmDesc<T> g{};
   g.batch = batch;
   g.A = P; g.B = P; g.C = sp > 1 ? part : G; g.E = nullptr;
