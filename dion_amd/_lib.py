@@ -58,6 +58,7 @@ _SIGNATURES = {
                                 _vp, _vp, _sz, _vp]),
     "dion_amd_dion_step_qr": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i, _i,
                                    _vp, _vp, _sz, _vp]),
+    "dion_amd_set_option": (_i, [_c.c_char_p, _i]),
     "dion_amd_tile_trace_enable": (_i, [_i]),
     "dion_amd_tile_trace_read": (_i, [_vp, _i]),
     "dion_amd_profile_enable": (_i, [_i]),
@@ -179,6 +180,11 @@ class Workspace:
 
 
 QR_METHODS = {"rcqr": 0, "qr": 1, "cqr": 2}   # DION_AMD_QR_*
+
+
+def set_option(name, value):
+    """`dion_amd_set_option`: a run-time switch of the library (e.g. "fused_update": 1 / 0 / -1 = default)."""
+    check(load().dion_amd_set_option(name.encode(), int(value)), f"dion_amd_set_option({name!r})")
 
 PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
               "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt", "dion_ef_upd")

@@ -3,6 +3,7 @@
 #include "../../include/dion_amd.h"
 #include "common.h"
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include "elementwise.h"
 #include "prof.h"
@@ -177,6 +178,17 @@ int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype,
 }
 
 bool dtype_ok(int d) { return d == DA_BF16 || d == DA_F32; }
+
+// Run-time options (dion_amd_set_option).  -1: not set by the caller, the environment decides.
+std::atomic<int> g_opt_fused_update{-1};
+
+// Error feedback and weight update as one pass (the default) or as two AXPBY products.
+bool fused_update_enabled() {
+  const int v = g_opt_fused_update.load(std::memory_order_relaxed);
+  if (v >= 0) return v != 0;
+  static const bool env_off = getenv("DION_AMD_NO_FUSED") != nullptr;
+  return !env_off;
+}
 
 // Number of slices (1, 2 or 4) of the inner dimension `mp` for the product R = B^T P (np x r per matrix, `cb`
 // matrices), by the bf16 launcher's own estimate: workgroup rounds x 64-deep stages per tile, a 256 x 256 tile
@@ -353,6 +365,15 @@ int dion_amd_gemm(const void* A, long long a_stride, int lda, int a_kstrided, co
   g.a_kstrided = a_kstrided != 0; g.b_kstrided = b_kstrided != 0; g.symmetric = 0;
   g.epilogue = epilogue; g.s0 = s0; g.s1 = s1; g.faithful = faithful; g.c_dtype = c_dtype;
   return gemm_any(g, in_dtype, static_cast<hipStream_t>(stream));
+}
+
+int dion_amd_set_option(const char* name, int value) {
+  if (!name) return DA_ERR_ARG;
+  if (strcmp(name, "fused_update") == 0) {
+    g_opt_fused_update.store(value < 0 ? -1 : (value != 0), std::memory_order_relaxed);
+    return DA_OK;
+  }
+  return DA_ERR_ARG;
 }
 
 size_t dion_amd_muon_workspace_bytes(int batch, int m, int n) {
@@ -788,8 +809,7 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
       }
     }  // power iterations
     // ---- error feedback, column normalisation and weight update (reference dion/dion.py:851-872)
-    static const bool no_fused = getenv("DION_AMD_NO_FUSED") != nullptr;
-    if (faithful && !no_fused && da_dion_ef_update_applicable(mp, np, r, m_dtype)) {
+    if (faithful && fused_update_enabled() && da_dion_ef_update_applicable(mp, np, r, m_dtype)) {
       // Q_new first (it only needs R), then both rank-r updates in one pass over M and X
       {
         DaProfScope prof(DA_PROF_DION_ELEM, 0.0, s);

@@ -528,12 +528,13 @@ int chol_step(T* G, T* Lmat, T* Wmat, T* Tmat, long long sG, int r, int o, int n
   int per = 256 / batch;
   if (per < 1) per = 1;
   if (per > nroles) per = nroles;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
+  static DaOncePerDevice configured;
+  const int rc_cfg = configured.run([&]() -> int {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(chol_step_kernel<T, INV>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    configured = true;
-  }
+    return DA_OK;
+  });
+  if (rc_cfg) return rc_cfg;
   // update-only workgroups of a deferred trailing update: one per tile right of this block column (columns below
   // c_end, lower triangle), at most 1024 over the batch
   int extra = 0;

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <atomic>
 
 // ---- error codes of the C ABI (0 ok, <0 bad argument, >0 hipError_t) -------------
 #define DA_OK 0
@@ -58,18 +59,36 @@ static inline int da_launch_status() {
   return e == hipSuccess ? DA_OK : (int)e;
 }
 
-// Compute units of the current device (persistent kernels size their grids with it).
+// Compute units of the current device (persistent kernels size their grids with it).  Callers may be on several
+// host threads at once: the cache entries are atomics (racing first calls store the same value).
 static inline int da_cu_count() {
-  static int cache[64] = {0};
+  static std::atomic<int> cache[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cache[dev] == 0) {
-    int n = 0;
+  int n = cache[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cache[dev] = n;
+    cache[dev].store(n, std::memory_order_relaxed);
   }
-  return cache[dev];
+  return n;
 }
+
+// One-time set-up of a kernel (its dynamic shared memory limit) per device.  The set-up call is idempotent, so two
+// host threads that race on the first launch may both make it; the flag word itself is an atomic with one bit per
+// device, set only after the call succeeded.
+struct DaOncePerDevice {
+  std::atomic<unsigned long long> done{0};
+  template <typename F>
+  int run(F&& setup) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    const unsigned long long bit = 1ull << dev;
+    if (done.load(std::memory_order_acquire) & bit) return DA_OK;
+    const int rc = setup();
+    if (rc == DA_OK) done.fetch_or(bit, std::memory_order_release);
+    return rc;
+  }
+};
 
 // ---- GEMM descriptor shared by the bf16 / f32 / f64 kernels -------------------------
 // C[b] (M x N) = epilogue( sum_k Aop[b](i,k) * Bop[b](j,k) ).

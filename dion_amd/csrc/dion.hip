@@ -1173,7 +1173,10 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   const bool cqr = passes == 2 && method == DA_QR_CQR;
   const bool fast = cqr || (passes == 2 && method == DA_QR_AUTO && !force64 && rows >= 4 * r);
   static const bool no16 = getenv("DION_AMD_ORTH_NO_BF16") != nullptr;
-  const bool fast16 = fast && dtype == DA_BF16 && low && !no16;
+  // (the Gram products on the bf16 matrix cores sum over the rows in 16-byte chunks: rows a multiple of 8 as well;
+  // other factors keep the fp32 kernels, which take any number of rows)
+  const bool rows8 = (rows & 7) == 0;
+  const bool fast16 = fast && dtype == DA_BF16 && low && rows8 && !no16;
   const DaGate all{nullptr, 0};
   int rc;
   if (cqr) {
@@ -1265,7 +1268,7 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   // Gram matrix that measures its defect then runs on the bf16 matrix cores (h^T h + h^T l + l^T h), and the
   // correction product reads h.  Otherwise: one conversion pass to fp32 costs less than reading fp64 twice in the
   // polishing products.
-  const bool hl = last_low && dtype == DA_BF16 && !no16;
+  const bool hl = last_low && dtype == DA_BF16 && rows8 && !no16;
   bf16_t* Lo = reinterpret_cast<bf16_t*>(w.Pf);
   rc = hl ? da_cvt_f64_to_hl(w.P0, w.Ph, Lo, pr, batch, gate2, s)
           : da_cvt_f64_to_f32(w.P0, w.Pf, last_low ? w.Ph : nullptr, pr, batch, gate2, s);

@@ -285,25 +285,16 @@ __global__ __launch_bounds__(512) void dion_ef_update_kernel(FusedArgs a) {
   }
 }
 
-int cu_count() {
-  static int n = [] {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-    return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  }();
-  return n;
-}
-
 template <bool DUAL_A, bool XF32>
 int launch(const FusedArgs& a, hipStream_t s) {
   auto k = dion_ef_update_kernel<DUAL_A, XF32>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
+  static DaOncePerDevice configured;
+  const int rc_cfg = configured.run([&]() -> int {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM));
-    configured = true;
-  }
-  int grid = cu_count();
+    return DA_OK;
+  });
+  if (rc_cfg) return rc_cfg;
+  int grid = da_cu_count();
   if (grid > a.total) grid = a.total;
   hipLaunchKernelGGL(k, dim3((unsigned)grid), dim3(512), SMEM, s, a);
   return da_launch_status();

@@ -349,7 +349,7 @@ constexpr int DA_LOOP_CHECKED = 0, DA_LOOP_INTERIOR = 1, DA_LOOP_EDGE = 2;
 constexpr int DA_TRACE_TILES = 65536;
 constexpr int DA_TRACE_WORDS = 6;
 __device__ unsigned long long da_tile_trace[DA_TRACE_WORDS * DA_TRACE_TILES];
-bool g_tile_trace = false;
+std::atomic<bool> g_tile_trace{false};
 
 template <typename C, bool A_KS, bool B_KS, bool SYM, int MODE>
 __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
@@ -601,16 +601,17 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   auto kfull = gemm_bf16_kernel<C, A_KS, B_KS, SYM, DA_LOOP_INTERIOR>;
   auto kedge = gemm_bf16_kernel<C, A_KS, B_KS, SYM, (A_KS || B_KS) && !SYM ? DA_LOOP_EDGE : DA_LOOP_CHECKED>;
   auto kgen = gemm_bf16_kernel<C, A_KS, B_KS, SYM, DA_LOOP_CHECKED>;
-  static bool configured = false;  // benign race: the attribute calls are idempotent
-  if (!configured) {
+  static DaOncePerDevice configured;
+  const int rc_cfg = configured.run([&]() -> int {
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kfull), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kedge), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kgen), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    configured = true;
-  }
+    return DA_OK;
+  });
+  if (rc_cfg) return rc_cfg;
   GemmArgs args{};
   args.n = n;
-  args.trace = g_tile_trace ? 1 : 0;
+  args.trace = g_tile_trace.load(std::memory_order_relaxed) ? 1 : 0;
   const bool full = all_interior(d, n, BT);
   static const bool edge_on = [] { const char* e = getenv("DION_AMD_NO_EDGE_LOOP"); return !(e && atoi(e)); }();
   const bool edge = !full && edge_on && (A_KS || B_KS) && !SYM && edge_loop_ok(d, n, BT);
@@ -744,7 +745,7 @@ int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) { return da_gemm_bf16_gr
 
 // ---- measurement hook: time stamps of the tiles of the bf16 GEMM launches (see include/dion_amd.h)
 extern "C" int dion_amd_tile_trace_enable(int on) {
-  g_tile_trace = on != 0;
+  g_tile_trace.store(on != 0, std::memory_order_relaxed);
   return DA_OK;
 }
 extern "C" int dion_amd_tile_trace_read(void* dst, int tiles) {

@@ -2,16 +2,17 @@
 #include "../../include/dion_amd.h"
 #include <vector>
 #include <mutex>
+#include <atomic>
 
 namespace {
 struct Rec { hipEvent_t a, b; int kind; double work; };
 std::mutex g_mu;
-bool g_on = false;
+std::atomic<bool> g_on{false};   // read by every launch, from any host thread
 std::vector<Rec> g_recs;
 }  // namespace
 
 DaProfScope::DaProfScope(int kind, double work, hipStream_t stream) : slot(-1), s(stream) {
-  if (!g_on) return;
+  if (!g_on.load(std::memory_order_relaxed)) return;
   std::lock_guard<std::mutex> lk(g_mu);
   Rec r{};
   r.kind = kind; r.work = work;
@@ -31,7 +32,7 @@ extern "C" {
 
 int dion_amd_profile_enable(int on) {
   std::lock_guard<std::mutex> lk(g_mu);
-  g_on = on != 0;
+  g_on.store(on != 0, std::memory_order_relaxed);
   return 0;
 }
 

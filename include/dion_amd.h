@@ -327,6 +327,17 @@ int dion_amd_profile_reset(void);
  * summed work. */
 int dion_amd_profile_read(int kind, long long* launches, double* total_ms, double* total_work);
 
+/* Run-time options of the library (no counterpart in the reference; for tests and measurements that compare two
+ * roads through the same entry point within one process).  `name`:
+ *   "fused_update"  1: dion_amd_dion_step(_qr) applies error feedback and weight update in one pass over M and X
+ *                   where that kernel applies (bf16 momentum, dimensions multiples of 128, rank a multiple of 64);
+ *                   0: always as two products with the update in their epilogues (reference dion/dion.py:851-853
+ *                   and 865-872 as two calls); -1: the default (one pass unless DION_AMD_NO_FUSED is set in the
+ *                   environment).  Both roads give the same bits.
+ * The value applies to calls that start after this one returns, on every thread.  Unknown name:
+ * DION_AMD_ERR_ARG. */
+int dion_amd_set_option(const char* name, int value);
+
 /* Time line of a bf16 GEMM launch (no counterpart in the reference; used by the benchmark only).  While enabled,
  * every workgroup of a bf16 GEMM launch -- one output tile each -- records three readings of the GPU's 100 MHz
  * counter (start, end of its K loop, end of its epilogue) and the hardware id of the CU it ran on.  `read` waits

@@ -450,3 +450,24 @@ def test_orthonormalize_methods(dev):
     Q1 = Q[1].double().cpu()
     keep = [j for j in range(64) if j != 17]
     assert (Q1[:, keep].T @ Q1[:, keep] - torch.eye(63, dtype=torch.float64)).norm().item() <= ORTH_TOL
+
+
+@pytest.mark.parametrize("rows,r", [(100, 24), (1004, 64), (1001, 16)])
+@pytest.mark.parametrize("method", ["rcqr", "qr", "cqr"])
+def test_orthonormalize_bf16_with_rows_off_the_8_grid(dev, rows, r, method):
+    """A bf16 factor whose rank is a multiple of 8 but whose number of rows is not: the Gram products on the bf16
+    matrix cores sum over the rows in 16-byte chunks and do not apply; the fp32 kernels take such a factor (the entry
+    point only asks for rows >= r).  All three methods must return the thin-QR factor."""
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(13)
+    P = torch.randn(2, rows, r).bfloat16()
+    Q, info = orthonormalize(P.to(dev), qr_method=method, return_info=True)
+    assert Q.dtype == torch.bfloat16 and (info == 0).all()
+    for b in range(2):
+        Qd = Q[b].double().cpu()
+        orth = (Qd.T @ Qd - torch.eye(r, dtype=torch.float64)).norm().item()
+        Qh, _ = torch.linalg.qr(P[b].double())
+        diff = rel_fro(_sign_align(Qd, Qh), Qh)
+        print(f"{method} {rows}x{r} matrix {b}: ||QtQ-I|| = {orth:.2e}, vs Householder {diff:.2e}")
+        assert orth <= 3e-2 and diff <= 5e-3

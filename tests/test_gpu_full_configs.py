@@ -211,3 +211,77 @@ def test_dion_non_finite_gradient_follows_the_reference_guard(dev, bad):
     q_got = opt.state[params[0]]["Q"].cpu()
     assert torch.isfinite(q_got).all() and torch.isfinite(Qo[0]).all()
     assert torch.allclose(q_got, Qo[0], rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("rank_fraction", [0.25, 1.0])
+def test_config3_full_72_matrix_dion_step(dev, rank_fraction):
+    """All 72 GPT-small matrices (buckets of 48 / 12 / 12 on three streams, the calls of a wave enqueued by worker
+    threads: the default path of `Dion.step`) with bf16 weights and momentum and fp32 Q, 10 consecutive steps against
+    `oracle.dion_step` (reference dion/dion.py:742-875).
+
+    Two optimizers run side by side.  `free` follows its own trajectory (bar 1e-2 on M and X, the bf16 level).  `sync`
+    is put back on the oracle's state after every step, so that a step's *update* can be compared sharply: one step
+    moves X by less than 1 % of its norm, which the bar on X itself cannot see.  Measured on the updates:
+      error feedback  (M_new - B) = -(1 - mu) P R^T, B = M + G (bit exact)   relative error <= 4e-2
+      weight update   (X_new - X)                                             relative error <= 8e-2
+    (both are sums of bf16 roundings of single elements: the weight update is 1-2 ulps of a weight, and a different
+    summation order inside the products flips some of them)."""
+    from dion_amd import Dion, DionMixedPrecisionConfig
+    from oracle import dion_step as O
+
+    shapes = GPT_SMALL_LAYER * 12
+    bf = torch.bfloat16
+    g0 = torch.Generator().manual_seed(11)
+    X0 = [(torch.randn(s, generator=g0) * 0.02).to(bf) for s in shapes]
+    gq = torch.Generator().manual_seed(2)
+    Q0 = []
+    for (m, n) in shapes:
+        q = torch.randn((min(m, n), O.rank_of(m, n, rank_fraction)), generator=gq)
+        Q0.append(q / q.norm(dim=0, keepdim=True))
+    mp = DionMixedPrecisionConfig(momentum_dtype=bf, Q_dtype=torch.float32)
+    opts, plists = [], []
+    for _ in range(2):
+        params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+        opt = Dion(params, rank_fraction=rank_fraction, lr=0.01, mu=0.95, weight_decay=0.01, mixed_precision_config=mp)
+        for p, q in zip(params, Q0):
+            opt._get_or_initialize_state(p, opt.param_groups[0])["Q"].copy_(q.to(dev))
+        opts.append(opt)
+        plists.append(params)
+    (sync, free), (ps, pf) = opts, plists
+    Xo, Mo, Qo = [x.clone() for x in X0], [torch.zeros_like(x) for x in X0], [q.clone() for q in Q0]
+    gg = torch.Generator().manual_seed(3)
+    sk = torch.Generator().manual_seed(0)
+    worst = dict(ef=0.0, dx=0.0, M=0.0, X=0.0)
+    for step in range(10):
+        G = [(torch.randn(s, generator=gg) * 1e-3).to(bf) for s in shapes]
+        for params in plists:
+            for p, g in zip(params, G):
+                p.grad = g.to(dev)
+        Xprev = [x.clone() for x in Xo]
+        B = [m + g for m, g in zip(Mo, G)]                      # bf16 add, as torch._foreach_add_ (dion.py:794)
+        sync.step()
+        free.step()
+        O.dion_step(Xo, G, Mo, Qo, lr=0.01, mu=0.95, weight_decay=0.01, generator=sk)
+        torch.cuda.synchronize()
+        for opt in opts:
+            info = torch.cat([v for v in opt.cholesky_info().values()])
+            assert info.numel() == 72 and int(info.abs().sum().item()) == 0, f"step {step}: info {info.tolist()}"
+        for i in range(72):
+            st = sync.state[ps[i]]
+            ef_ref = Mo[i].double() - B[i].double()
+            ef_got = st["momentum"].cpu().double() - B[i].double()
+            dx_ref = Xo[i].double() - Xprev[i].double()
+            dx_got = ps[i].detach().cpu().double() - Xprev[i].double()
+            e_ef = ((ef_got - ef_ref).norm() / ef_ref.norm()).item()
+            e_dx = ((dx_got - dx_ref).norm() / dx_ref.norm()).item()
+            worst["ef"], worst["dx"] = max(worst["ef"], e_ef), max(worst["dx"], e_dx)
+            assert e_ef <= 4e-2 and e_dx <= 8e-2, (step, i, shapes[i], e_ef, e_dx)
+            assert (st["Q"].double().norm(dim=0) - 1).abs().max().item() < 1e-2
+            eM, eX = rel_fro(free.state[pf[i]]["momentum"], Mo[i]), rel_fro(pf[i].detach(), Xo[i])
+            worst["M"], worst["X"] = max(worst["M"], eM), max(worst["X"], eX)
+            assert eM <= 1e-2 and eX <= 1e-2, (step, i, shapes[i], eM, eX)
+            # back onto the oracle's state
+            ps[i].data.copy_(Xo[i])
+            st["momentum"].copy_(Mo[i])
+            st["Q"].copy_(Qo[i])
+        print(f"config 3, 72 matrices, rank fraction {rank_fraction}, step {step}: worst so far {worst}", flush=True)
