@@ -222,10 +222,10 @@ def test_config3_full_72_matrix_dion_step(dev, rank_fraction):
     Two optimizers run side by side.  `free` follows its own trajectory (bar 1e-2 on M and X, the bf16 level).  `sync`
     is put back on the oracle's state after every step, so that a step's *update* can be compared sharply: one step
     moves X by less than 1 % of its norm, which the bar on X itself cannot see.  Measured on the updates:
-      error feedback  (M_new - B) = -(1 - mu) P R^T, B = M + G (bit exact)   relative error <= 4e-2
-      weight update   (X_new - X)                                             relative error <= 8e-2
-    (both are sums of bf16 roundings of single elements: the weight update is 1-2 ulps of a weight, and a different
-    summation order inside the products flips some of them)."""
+      error feedback  (M_new - B) = -(1 - mu) P R^T, B = M + G (bit exact)   measured <= 1.0e-2, bar 2e-2
+      weight update   (X_new - X)         measured <= 2.6e-2 (r = 192) / 7.8e-2 (r = 768), bar 5e-2 / 1.2e-1
+    (both are differences of bf16 values: the weight update is 1-2 ulps of a weight, and a different summation order
+    inside the rank-r products flips the rounding of some of them; a wrong scale, sign or operand is an error of 1)."""
     from dion_amd import Dion, DionMixedPrecisionConfig
     from oracle import dion_step as O
 
@@ -275,7 +275,7 @@ def test_config3_full_72_matrix_dion_step(dev, rank_fraction):
             e_ef = ((ef_got - ef_ref).norm() / ef_ref.norm()).item()
             e_dx = ((dx_got - dx_ref).norm() / dx_ref.norm()).item()
             worst["ef"], worst["dx"] = max(worst["ef"], e_ef), max(worst["dx"], e_dx)
-            assert e_ef <= 4e-2 and e_dx <= 8e-2, (step, i, shapes[i], e_ef, e_dx)
+            assert e_ef <= 2e-2 and e_dx <= (5e-2 if rank_fraction < 1 else 1.2e-1), (step, i, shapes[i], e_ef, e_dx)
             assert (st["Q"].double().norm(dim=0) - 1).abs().max().item() < 1e-2
             eM, eX = rel_fro(free.state[pf[i]]["momentum"], Mo[i]), rel_fro(pf[i].detach(), Xo[i])
             worst["M"], worst["X"] = max(worst["M"], eM), max(worst["X"], eX)
