@@ -53,7 +53,7 @@ WORKLOADS = {
     "scalar_gpt_small": dict(kind="scalar", shapes=[(50304, 768)] * 2 + [(768,)] * 25, seed=6,
                              desc="Lion on the GPT-small embedding and norms, AdamW on lm_head (50304x768 each), bf16"),
 }
-GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")
+GEMM_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "ns_flow", "gemm", "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")
 
 
 def make_problem(shapes, seed, dtype, device="cpu"):
@@ -157,7 +157,7 @@ def summarize(name, wl, res):
                orthogonalisations_per_s=round(len(shapes) / (res["ms_per_step"] * 1e-3), 1))
     prof = res["prof"]
     if wl["kind"] == "muon":
-        ns_ms = sum(prof[k][1] for k in ("ns_syrk", "ns_poly", "ns_axpy") if k in prof) / res["steps"]
+        ns_ms = sum(prof[k][1] for k in ("ns_syrk", "ns_poly", "ns_axpy", "ns_flow") if k in prof) / res["steps"]
         f_sym = ns_flops(shapes, True)
         out.update(ns_gemm_ms_per_step=round(ns_ms, 4),
                    ns_executed_tflops=round(f_sym / (ns_ms * 1e-3) / 1e12, 1),
@@ -221,7 +221,7 @@ def roofline_of(res, kind, workload=None):
                     frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4),
                     traffic=MEASURED_TRAFFIC_BYTES.get((workload, "scalar_opt")), avg_launch_ms=round(ms / n, 5),
                     bytes_per_launch=work / n)
-    cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy") if kind == "muon"
+    cands = [k for k in (("ns_syrk", "ns_poly", "ns_axpy", "ns_flow") if kind == "muon"
                          else ("dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")) if k in prof]
     dom = max(cands, key=lambda k: prof[k][1])
     n, ms, work = prof[dom]

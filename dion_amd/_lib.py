@@ -61,6 +61,8 @@ _SIGNATURES = {
     "dion_amd_set_option": (_i, [_c.c_char_p, _i]),
     "dion_amd_tile_trace_enable": (_i, [_i]),
     "dion_amd_tile_trace_read": (_i, [_vp, _i]),
+    "dion_amd_ns_flow_trace_enable": (_i, [_i]),
+    "dion_amd_ns_flow_trace_read": (_i, [_vp, _i, _c.POINTER(_i)]),
     "dion_amd_profile_enable": (_i, [_i]),
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),
@@ -187,7 +189,7 @@ def set_option(name, value):
     check(load().dion_amd_set_option(name.encode(), int(value)), f"dion_amd_set_option({name!r})")
 
 PROF_KINDS = ("ns_syrk", "ns_poly", "ns_axpy", "stage", "normalize", "unstage", "gemm",
-              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt", "dion_ef_upd")
+              "dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_orth", "dion_elem", "scalar_opt", "dion_ef_upd", "ns_flow")
 
 
 def profile_read():

@@ -8,6 +8,7 @@
 #include "elementwise.h"
 #include "prof.h"
 #include "dion.h"
+#include "ns_flow.h"
 
 namespace {
 
@@ -23,7 +24,7 @@ struct NsLayout {
   int mw = 0, nw = 0, tiles = 0;
   int ldx = 0, lda = 0;   // row pitches of the mw x nw iterates and of the mw x mw Gram / polynomial
   size_t esz = 0;
-  size_t x_bytes = 0, a_bytes = 0, part_bytes = 0;  // per matrix
+  size_t x_bytes = 0, a_bytes = 0, part_bytes = 0, flow_bytes = 0;  // per matrix
   size_t per_matrix = 0;
   NsLayout() {}
   NsLayout(int m, int n, int dtype) {
@@ -37,7 +38,9 @@ struct NsLayout {
     x_bytes = (size_t)mw * ldx * esz;
     a_bytes = (size_t)mw * lda * esz;
     part_bytes = align_up((size_t)tiles * sizeof(float) + sizeof(float), 256);
-    per_matrix = 2 * x_bytes + 2 * a_bytes + part_bytes;
+    // control words of the persistent Newton-Schulz kernel: cb * flow_bytes >= da_ns_flow_ctl_bytes(cb) for cb >= 1
+    flow_bytes = DA_FLOW_CTR_STRIDE * sizeof(int) + 256;
+    per_matrix = 2 * x_bytes + 2 * a_bytes + part_bytes + flow_bytes;
   }
   int chunk(int batch, size_t ws_bytes) const {
     size_t c = ws_bytes / per_matrix;
@@ -57,6 +60,7 @@ struct NsLayout {
 struct NsBuffers {
   char *x0 = nullptr, *x1 = nullptr, *a = nullptr, *b = nullptr;
   float *partials = nullptr, *divisor = nullptr;
+  int* flow = nullptr;
   NsBuffers() {}
   NsBuffers(const NsLayout& L, void* ws, int cb) {
     char* p = static_cast<char*>(ws);
@@ -64,8 +68,9 @@ struct NsBuffers {
     x1 = p; p += L.x_bytes * cb;
     a = p; p += L.a_bytes * cb;
     b = p; p += L.a_bytes * cb;
-    partials = reinterpret_cast<float*>(p);
+    partials = reinterpret_cast<float*>(p); p += L.part_bytes * cb;
     divisor = partials + (size_t)L.tiles * cb;
+    flow = reinterpret_cast<int*>(p);
   }
 };
 
@@ -105,10 +110,41 @@ struct NsSet {
 
 // steps x { A = X X^T ; B = b A + c A A ; X' = a X + B X } on up to DA_MAX_GROUPS sets of wide
 // matrices at once (each of the three products is one grouped launch over all sets).
-// Returns in result[i] which of x0 / x1 of set i holds the final iterate.
+// Returns in result[i] which of x0 / x1 of set i holds the final iterate, and in *poison (if asked for) a device word
+// that is non-zero when the iterates are invalid (null: there is no such word).
 int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int steps, int faithful, hipStream_t s,
-               char** result) {
+               char** result, const int** poison = nullptr) {
   if (nsets < 1 || nsets > DA_MAX_GROUPS) return DA_ERR_ARG;
+  if (poison) *poison = nullptr;
+  if (dtype == DA_BF16 && steps >= 1) {
+    // many small matrices: all iterations of all sets as one persistent launch (ns_flow.hip); the sets are dealt to
+    // its queues most expensive first
+    DaNsFlowGroup fg[DA_MAX_GROUPS];
+    int order[DA_MAX_GROUPS];
+    for (int i = 0; i < nsets; ++i) order[i] = i;
+    auto cost = [&](int i) { const NsLayout& L = sets[i].L; return (double)L.mw * L.mw * (3.0 * L.nw + L.mw); };
+    for (int i = 1; i < nsets; ++i)
+      for (int j = i; j > 0 && cost(order[j - 1]) < cost(order[j]); --j) { const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t; }
+    for (int k = 0; k < nsets; ++k) {
+      const NsLayout& L = sets[order[k]].L;
+      const NsBuffers& W = sets[order[k]].W;
+      fg[k] = DaNsFlowGroup{W.x0, W.x1, W.a, W.b, (long long)(L.x_bytes / L.esz), (long long)(L.a_bytes / L.esz),
+                            L.mw, L.nw, L.ldx, L.lda, sets[order[k]].cb, W.flow};
+    }
+    if (da_ns_flow_applicable(fg, nsets, steps)) {
+      double flops = 0.0;
+      for (int i = 0; i < nsets; ++i) {
+        const NsLayout& L = sets[i].L;
+        flops += (double)steps * sets[i].cb * ((double)L.mw * (L.mw + 1.0) * (L.nw + L.mw) + 2.0 * L.mw * L.mw * L.nw);
+      }
+      DaProfScope prof(DA_PROF_NS_FLOW, flops, s);
+      const int rc = da_ns_flow(fg, nsets, coeffs, steps, faithful, s);
+      if (rc) return rc;
+      for (int i = 0; i < nsets; ++i) result[i] = (steps & 1) ? sets[i].W.x1 : sets[i].W.x0;
+      if (poison) *poison = da_ns_flow_status_word(fg);
+      return DA_OK;
+    }
+  }
   char *x[DA_MAX_GROUPS], *y[DA_MAX_GROUPS];
   for (int i = 0; i < nsets; ++i) { x[i] = sets[i].W.x0; y[i] = sets[i].W.x1; }
   for (int it = 0; it < steps; ++it) {
@@ -164,10 +200,10 @@ int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int
 }
 
 int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const float* coeffs, int steps,
-               int faithful, hipStream_t s, char** result) {
+               int faithful, hipStream_t s, char** result, const int** poison = nullptr) {
   NsSet one;
   one.L = L; one.W = W; one.cb = cb;
-  return ns_iterate(&one, 1, dtype, coeffs, steps, faithful, s, result);
+  return ns_iterate(&one, 1, dtype, coeffs, steps, faithful, s, result, poison);
 }
 
 int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
@@ -260,9 +296,11 @@ int ns_run(const void* G, int g_dtype, long long g_stride, int ldg, void* out, l
     rc = ns_normalize_chunk(L, W, cb, compute_dtype, eps, s);
     if (rc) return rc;
     char* res = nullptr;
-    rc = ns_iterate(L, W, cb, compute_dtype, coeffs, steps, faithful, s, &res);
+    const int* poison = nullptr;
+    rc = ns_iterate(L, W, cb, compute_dtype, coeffs, steps, faithful, s, &res, &poison);
     if (rc) return rc;
     DaUnstage us{};
+    us.poison = poison;
     for (int i = 0; i < cb; ++i) us.x.p[i] = static_cast<char*>(out) + (size_t)(b0 + i) * out_stride * L.esz;
     us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = ldo; us.ldw = L.ldx;
     us.x_dtype = compute_dtype; us.w_dtype = compute_dtype;
@@ -373,7 +411,24 @@ int dion_amd_set_option(const char* name, int value) {
     g_opt_fused_update.store(value < 0 ? -1 : (value != 0), std::memory_order_relaxed);
     return DA_OK;
   }
+  if (strcmp(name, "ns_flow") == 0) {
+    if (value < -1 || value > 2) return DA_ERR_ARG;
+    da_ns_flow_set_mode(value);
+    return DA_OK;
+  }
+  if (strcmp(name, "ns_flow_fail") == 0) {
+    da_ns_flow_set_fail(value != 0);
+    return DA_OK;
+  }
   return DA_ERR_ARG;
+}
+
+int dion_amd_ns_flow_trace_enable(int on) {
+  da_ns_flow_trace_enable(on);
+  return DA_OK;
+}
+int dion_amd_ns_flow_trace_read(void* host_dst, int max_tiles, int* tiles) {
+  return da_ns_flow_trace_read(host_dst, max_tiles, tiles);
 }
 
 size_t dion_amd_muon_workspace_bytes(int batch, int m, int n) {
@@ -419,9 +474,11 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
     rc = ns_normalize_chunk(L, W, cb, DA_BF16, eps, s);
     if (rc) return rc;
     char* res = nullptr;
-    rc = ns_iterate(L, W, cb, DA_BF16, coeffs, steps, faithful, s, &res);
+    const int* poison = nullptr;
+    rc = ns_iterate(L, W, cb, DA_BF16, coeffs, steps, faithful, s, &res, &poison);
     if (rc) return rc;
     DaUnstage us{};
+    us.poison = poison;
     for (int i = 0; i < cb; ++i) us.x.p[i] = X[b0 + i];
     us.wide = res; us.batch = cb; us.rows = m; us.cols = n; us.ld = n; us.ldw = L.ldx;
     us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
@@ -573,7 +630,8 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
       if (rc) return rc;
     }
     char* res[DA_MAX_GROUPS];
-    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res);
+    const int* poison = nullptr;
+    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res, &poison);
     if (rc) return rc;
     for (int i = 0; i < nr; ++i) {
       const dion_amd_muon_bucket& k = buckets[r0 + i];
@@ -586,6 +644,7 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
         us.batch = c; us.rows = k.m; us.cols = k.n; us.ld = k.n; us.ldw = L.ldx;
         us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
         us.decay = k.decay; us.step = k.adjusted_lr; us.muon = 1;
+        us.poison = poison;
         DaProfScope prof(DA_PROF_UNSTAGE, (double)k.m * k.n * (2 * xsz + 2) * c, s);
         rc = da_unstage(us, s);
         if (rc) return rc;

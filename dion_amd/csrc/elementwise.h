@@ -37,6 +37,9 @@ struct DaUnstage {
   // orientation) instead of the batch `wide`.
   int use_wtab;
   DaPtrTable wtab;
+  // Optional device word: if it is non-zero when the kernel runs, the working matrices are invalid (the launch that
+  // made them gave up) and every result element is written as NaN.
+  const int* poison;
 };
 
 int da_stage_tiles(int rows, int cols);

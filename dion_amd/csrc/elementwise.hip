@@ -325,11 +325,14 @@ struct UnstageArgs {
   int muon;           // 1: X <- X*decay - wide*step ; 0: X <- wide
   int use_wtab;       // 1: source b is wtab.p[b] (rows x cols contiguous); never with TALL
   DaPtrTable wtab;
+  const int* poison;  // optional device word: non-zero = the working matrices are invalid, the result becomes NaN
 };
 
 template <typename TX, typename TW, bool TALL>
 __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
   __shared__ float tile[TALL ? TS : 1][TS + 1];
+  const bool poisoned = a.poison != nullptr && *a.poison != 0;
+  const float nan = __builtin_nanf("");
   const int b = blockIdx.y;
   const int tiles_c = (a.cols + TS - 1) / TS;
   const int ti = blockIdx.x / tiles_c, tj = blockIdx.x % tiles_c;
@@ -352,6 +355,10 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
       if (ok[it]) {
         Vec8<TW>::load(W + (long long)i * a.ldw + j, u[it]);
         if (a.muon) Vec8<TX>::load_nt(X + (long long)i * a.ld + j, x[it]);
+        if (poisoned) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) u[it][e] = nan;
+        }
       }
     }
 #pragma unroll
@@ -404,6 +411,10 @@ __global__ __launch_bounds__(256) void unstage_kernel(UnstageArgs<TX, TW> a) {
     } else {
       Vec8<TW>::load(W + (long long)i * a.ldw + j, u);
     }
+    if (poisoned) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = nan;
+    }
     TX* xp = X + (long long)i * a.ld + j;
     if (a.muon) {
       float x[8];
@@ -443,7 +454,7 @@ int stage_dispatch_w(const DaStage& d, hipStream_t s) {
 
 template <typename TX, typename TW>
 int unstage_launch(const DaUnstage& d, hipStream_t s) {
-  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon, d.use_wtab, d.wtab};
+  UnstageArgs<TX, TW> a{d.x, static_cast<const TW*>(d.wide), d.rows, d.cols, d.ld, d.ldw, d.decay, d.step, d.muon, d.use_wtab, d.wtab, d.poison};
   const bool tall = d.rows > d.cols && !d.use_wtab;
   const int tiles = tall ? ((a.rows + TS - 1) / TS) * ((a.cols + TS - 1) / TS)
                          : ((a.rows + RT - 1) / RT) * ((a.cols + CT - 1) / CT);

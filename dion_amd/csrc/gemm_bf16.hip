@@ -30,6 +30,7 @@
 // also written transposed.
 #include "common.h"
 #include "mfma_tile.h"
+#include "gemm_bf16_tile.h"
 #include <cstdlib>
 
 namespace {
@@ -40,75 +41,6 @@ struct GemmArgs {
   int start[DA_MAX_GROUPS + 1];
   int n;
   int trace;   // 1: every workgroup records its time stamps (measurement hook)
-};
-
-template <int BT_, int WGM_, int WGN_>
-struct Cfg {
-  static constexpr int BT = BT_, WGM = WGM_, WGN = WGN_;
-  static constexpr int NT = 64 * WGM * WGN;        // threads
-  static constexpr int TMI = BT / (32 * WGM);      // accumulators per wavefront, row direction
-  static constexpr int TNJ = BT / (32 * WGN);      // ... column direction
-  static constexpr int NCH = BT * 8 / NT;          // 16-byte chunks per thread per operand stage
-  static constexpr int WROWS = BT / WGM, WCOLS = BT / WGN;
-};
-
-template <int BT, bool KS>
-struct Tile {
-  static constexpr int bytes = BT * BK * 2;   // either layout: 64 x BT bf16
-};
-
-// Per-thread addressing of the NCH 16-byte chunks a thread moves per operand stage.
-//   Register-staged path (bounds-checked): chunk i lies at global `g + i * gstep` (elements)
-//   and goes to LDS byte offset `l + i * lstep`.
-//   Direct-to-LDS path: wave-instruction i of wavefront w fills the 1024-byte LDS block
-//   (i * NW + w); lane p of it fetches the chunk whose *physical* position is p, i.e. the
-//   swizzle is applied to the global address, which is kept as a wave-uniform base pointer
-//   (`dbase`) plus a 32-bit byte offset (`doff + i * dstep`, per lane and loop invariant, plus
-//   the stage's offset, a scalar) so that the loads use SGPR-base addressing.
-template <typename C, bool KS>
-struct StageAddr {
-  const bf16_t* g;
-  const char* dbase;
-  unsigned doff, dstep;
-  long long gstep, tstep;   // per chunk and per stage, in elements
-  int l, lstep;
-  int row, col;             // first chunk's (row within tile, k offset) resp. (k row, row offset)
-  // `dim`: extent of the operand in the tile's row direction (M or N); the direct-to-LDS addresses of a
-  // k-strided operand keep their 16-byte chunks inside it (an edge tile then fetches a neighbouring chunk for the
-  // columns it does not own: finite values that the bounds-checked epilogue never stores).
-  __device__ __forceinline__ StageAddr(const bf16_t* base, int ld, int row0, int tid, int dim) {
-    constexpr int NW = C::NT / 64;
-    const int lane = tid & 63, wave = tid >> 6;
-    if (!KS) {
-      row = tid >> 3;
-      col = (tid & 7) * 8;
-      g = base + (long long)(row0 + row) * ld + col;
-      gstep = (long long)(C::NT / 8) * ld;
-      tstep = BK;
-      l = row * 128 + kc_swizzle(tid & 7, row) * 16;
-      lstep = (C::NT / 8) * 128;   // NT/8 is a multiple of 16: the swizzle term is the same for all chunks
-      const int drow = wave * 8 + (lane >> 3);             // block (0 * NW + wave), 8 rows per block
-      dbase = reinterpret_cast<const char*>(base + (long long)row0 * ld);
-      doff = (unsigned)(drow * ld + kc_swizzle(lane & 7, drow) * 8) * 2u;
-      dstep = (unsigned)(NW * 8 * ld) * 2u;                // NW * 8 is a multiple of 16
-    } else {
-      constexpr int CPR = C::BT / 8;                       // chunks per k-row
-      constexpr int RPB = 64 / CPR;                        // k-rows per 1024-byte block
-      row = tid / CPR;
-      col = (tid % CPR) * 8;
-      g = base + (long long)row * ld + row0 + col;
-      gstep = (long long)(C::NT / CPR) * ld;
-      tstep = (long long)BK * ld;
-      l = row * (C::BT * 2) + ks_swizzle(tid % CPR, row) * 16;
-      lstep = (C::NT / CPR) * (C::BT * 2);                 // NT / CPR = 16: swizzle term unchanged
-      const int drow = wave * RPB + lane / CPR;
-      dbase = reinterpret_cast<const char*>(base + row0);
-      int dcol = ks_swizzle(lane % CPR, drow) * 8;
-      if (row0 + dcol > dim - 8) dcol = dim - 8 - row0;
-      doff = (unsigned)(drow * ld + dcol) * 2u;
-      dstep = (unsigned)(NW * RPB * ld) * 2u;              // NW * RPB = 16
-    }
-  }
 };
 
 // Which output tile a workgroup owns.  Workgroups are dealt round-robin to the 8 XCDs (each
@@ -152,186 +84,6 @@ __device__ __forceinline__ TileId decode_tile(const GemmDesc& d, int bid, int nb
   return r;
 }
 
-// The accumulators go through LDS (the stage buffers are free by now), one 32-row band of the
-// wavefront's sub-tile at a time, so that C and E move as 16-byte row segments.  Each wavefront
-// stages through its own LDS region, so only wavefront-level ordering is needed inside.
-// Output dtype, epilogue form and rounding mode are compile-time here: evaluated per element at
-// run time they cost more than the MFMAs of a short-K product.
-template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL, bool S1_ONE>
-__device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
-                                              bool mirror, int m0, int n0, int wave, int lane, int wm, int wn) {
-  constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
-  constexpr int PITCH = W + 4;       // floats; 16-byte aligned rows, conflict-free float4 writes
-  constexpr int CPR = W / 8;         // 8-column chunks per row
-  constexpr int RPP = 64 / CPR;      // rows per pass of the wavefront
-  constexpr int NPASS = 32 / RPP;
-  constexpr int CSZ = CF32 ? 4 : 2;
-  constexpr int NV = CF32 ? 2 : 1;   // 16-byte vectors per 8 elements
-  float* stg = reinterpret_cast<float*>(lds) + wave * (32 * PITCH);
-  // the descriptor lives in the kernel-argument segment: fields read inside the band loop would be fetched
-  // again after every store (scalar load + a full wait in the middle of the band), so they are copied first
-  const float s0 = d.s0, s1 = d.s1;
-  const long long c2 = (!HAS_E && !FAITHFUL && !SYM && !CF32) ? d.c2_off * 2 : 0;   // bytes to the second output
-  const int dM = d.M, dN = d.N;
-  const long long ldc = d.ldc, lde = d.lde;
-  const int wm0 = m0 + wm * C::WROWS, wn0 = n0 + wn * W;
-  char* const Cbase = d.Ctab ? static_cast<char*>(d.Ctab[b]) : static_cast<char*>(d.C) + (long long)b * d.sC * CSZ;
-  const char* const Ebase = !HAS_E ? nullptr
-                            : d.Etab ? static_cast<const char*>(d.Etab[b])
-                                     : static_cast<const char*>(d.E) + (long long)b * d.sE * CSZ;
-  const int lr = lane / CPR, c8 = (lane % CPR) * 8;
-  const bool col_ok = FULL || wn0 + c8 < dN;
-  // E is requested up to three bands ahead (registers that the K loop's fragments no longer need), so that a
-  // tile's epilogue pays one memory latency and not one per band; an fp32 E (twice the registers) one band ahead.
-  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (C::TMI < 3 ? C::TMI : 3);
-  u32x4_t ev[DEPTH][NPASS][NV];
-  auto load_e = [&](int band, u32x4_t (&dst)[NPASS][NV]) {
-#pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
-      const int m = wm0 + band * 32 + pass * RPP + lr;
-      const u32x4_t z = {0u, 0u, 0u, 0u};
-#pragma unroll
-      for (int h = 0; h < NV; ++h) dst[pass][h] = z;
-      if (col_ok && (FULL || m < dM)) {
-        const char* Ep = Ebase + ((long long)m * lde + wn0 + c8) * CSZ;
-#pragma unroll
-        for (int h = 0; h < NV; ++h) dst[pass][h] = ldg16(Ep + 16 * h);
-      }
-    }
-  };
-  if (HAS_E) {
-#pragma unroll
-    for (int q = 0; q < DEPTH; ++q) load_e(q, ev[q]);
-  }
-#pragma unroll
-  for (int i = 0; i < C::TMI; ++i) {
-    {
-      float* row = stg + (lane & 31) * PITCH + (lane >> 5) * 4;
-#pragma unroll
-      for (int j = 0; j < C::TNJ; ++j)
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq)
-          *reinterpret_cast<float4*>(row + j * 32 + vq * 8) =
-              make_float4(acc[i][j][vq * 4], acc[i][j][vq * 4 + 1], acc[i][j][vq * 4 + 2], acc[i][j][vq * 4 + 3]);
-    }
-    wave_sync_lds();
-    const int band_m = wm0 + i * 32;
-    u32x4_t ec[NPASS][NV];
-    if (HAS_E) {
-#pragma unroll
-      for (int pass = 0; pass < NPASS; ++pass)
-#pragma unroll
-        for (int h = 0; h < NV; ++h) ec[pass][h] = ev[i % DEPTH][pass][h];
-      if (i + DEPTH < C::TMI) load_e(i + DEPTH, ev[i % DEPTH]);
-    }
-#pragma unroll
-    for (int pass = 0; pass < NPASS; ++pass) {
-      const int r = pass * RPP + lr;
-      const int m = band_m + r;
-      if (col_ok && (FULL || m < dM)) {
-        float* sp = stg + r * PITCH + c8;
-        const float4 a0 = *reinterpret_cast<const float4*>(sp);
-        const float4 a1 = *reinterpret_cast<const float4*>(sp + 4);
-        float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        float e[8];
-        char* Cp = Cbase + ((long long)m * ldc + wn0 + c8) * CSZ;
-        if (CF32) {
-#pragma unroll
-          for (int q = 0; q < 8; ++q) {
-            const unsigned w = HAS_E ? ec[pass][q >> 2][q & 3] : 0u;  // (bit_cast of a vector element lvalue reads element 0)
-            e[q] = __builtin_bit_cast(float, w);
-          }
-#pragma unroll
-          for (int q = 0; q < 8; ++q) v[q] = epi_value<HAS_E, FAITHFUL, true>(s0, s1, v[q], e[q]);
-          const u32x4_t o0 = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
-                              __builtin_bit_cast(unsigned, v[2]), __builtin_bit_cast(unsigned, v[3])};
-          const u32x4_t o1 = {__builtin_bit_cast(unsigned, v[4]), __builtin_bit_cast(unsigned, v[5]),
-                              __builtin_bit_cast(unsigned, v[6]), __builtin_bit_cast(unsigned, v[7])};
-          stg16(Cp, o0);
-          stg16(Cp + 16, o1);
-        } else {
-          u32x4_t pk;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const unsigned w = HAS_E ? ec[pass][0][q] : 0u;   // (copied out: see the note on bit_cast above)
-            const unsigned o = epi_pair<HAS_E, FAITHFUL, S1_ONE>(s0, s1, v[2 * q], v[2 * q + 1], w);
-            pk[q] = o;
-            if (SYM) {
-              v[2 * q] = lo_f(o);
-              v[2 * q + 1] = hi_f(o);
-            }
-          }
-          stg16(Cp, pk);
-          if (!HAS_E && !FAITHFUL && !SYM && c2) {
-            // what the stored bf16 leaves of s1 * acc, as a second bf16 matrix
-            u32x4_t lo;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) lo[q] = cvt_pk_bf16(s1 * v[2 * q] - lo_f(pk[q]), s1 * v[2 * q + 1] - hi_f(pk[q]));
-            stg16(Cp + c2, lo);
-          }
-        }
-        if (SYM && mirror) {  // keep the final values for the transposed store
-          *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
-          *reinterpret_cast<float4*>(sp + 4) = make_float4(v[4], v[5], v[6], v[7]);
-        }
-      }
-    }
-    if (SYM && mirror) {
-      wave_sync_lds();
-      // C^T: row n of the mirrored tile holds 32 consecutive m of this band
-#pragma unroll
-      for (int pass = 0; pass < (W / 64) * 4; ++pass) {
-        const int nl = (pass >> 2) * 64 + lane;
-        const int mg = (pass & 3) * 8;
-        const int n = wn0 + nl, m = band_m + mg;
-        if (FULL || (n < dN && m < dM)) {  // M is a multiple of 8 for symmetric outputs
-          float v[8];
-#pragma unroll
-          for (int q = 0; q < 8; ++q) v[q] = stg[(mg + q) * PITCH + nl];
-          char* Cp = Cbase + ((long long)n * ldc + m) * CSZ;
-          if (CF32) {
-            const u32x4_t o0 = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
-                                __builtin_bit_cast(unsigned, v[2]), __builtin_bit_cast(unsigned, v[3])};
-            const u32x4_t o1 = {__builtin_bit_cast(unsigned, v[4]), __builtin_bit_cast(unsigned, v[5]),
-                                __builtin_bit_cast(unsigned, v[6]), __builtin_bit_cast(unsigned, v[7])};
-            stg16(Cp, o0);
-            stg16(Cp + 16, o1);
-          } else {
-            u32x4_t pk;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) pk[q] = cvt_pk_bf16(v[2 * q], v[2 * q + 1]);
-            stg16(Cp, pk);
-          }
-        }
-      }
-    }
-    wave_sync_lds();
-  }
-}
-
-template <typename C, bool SYM, bool FULL>
-__device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
-                                         int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
-  const bool mirror = SYM && (ti != tj);
-  const bool cf32 = d.c_dtype == DA_F32, has_e = d.epilogue == DA_EPI_AXPBY, fa = d.faithful != 0;
-  const bool one = d.s1 == 1.f;   // rounding-faithful bf16 output: the exact multiplication by 1 is left out
-#define DA_EPI(CF, HE, FA, S1) \
-  epilogue_impl<C, SYM, FULL, CF, HE, FA, S1>(acc, d, lds, b, mirror, m0, n0, wave, lane, wm, wn)
-  if (!cf32) {
-    if (has_e) {
-      if (fa) { if (one) DA_EPI(false, true, true, true); else DA_EPI(false, true, true, false); }
-      else DA_EPI(false, true, false, false);
-    } else {
-      if (fa) { if (one) DA_EPI(false, false, true, true); else DA_EPI(false, false, true, false); }
-      else DA_EPI(false, false, false, false);
-    }
-  } else {
-    if (has_e) { if (fa) DA_EPI(true, true, true, false); else DA_EPI(true, true, false, false); }
-    else       { if (fa) DA_EPI(true, false, true, false); else DA_EPI(true, false, false, false); }
-  }
-#undef DA_EPI
-}
-
 // ---------------------------------------------------------------------------------------
 // One kernel, two K loops, three modes.
 //   DA_LOOP_INTERIOR: every tile is interior (M, N multiples of BT, K a multiple of 64).  Stages are
@@ -345,7 +97,6 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
 // ---------------------------------------------------------------------------------------
 // Measurement hook: per workgroup (tile) of the last traced launch, the 100 MHz counter at the start, after the
 // K loop and at the end, the hardware id of the CU it ran on, and the shader-clock counter at the start and the end.
-constexpr int DA_LOOP_CHECKED = 0, DA_LOOP_INTERIOR = 1, DA_LOOP_EDGE = 2;
 constexpr int DA_TRACE_TILES = 65536;
 constexpr int DA_TRACE_WORDS = 6;
 __device__ unsigned long long da_tile_trace[DA_TRACE_WORDS * DA_TRACE_TILES];
@@ -353,7 +104,6 @@ std::atomic<bool> g_tile_trace{false};
 
 template <typename C, bool A_KS, bool B_KS, bool SYM, int MODE>
 __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
-  constexpr bool FULL = MODE != DA_LOOP_CHECKED;   // the direct-to-LDS K loop
   const bool trace = args.trace && blockIdx.x < DA_TRACE_TILES;
   unsigned long long ts0 = 0, ts1 = 0, tc0 = 0;
   if (trace) {
@@ -367,10 +117,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
     if (q < args.n && (int)blockIdx.x >= args.start[q]) grp = q;
   const GemmDesc& d = args.d[grp];
   const int blk0 = args.start[grp];
-  constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ, NCH = C::NCH, NW = C::NT / 64;
-  constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
-  constexpr int B_BYTES = Tile<BT, B_KS>::bytes;
-  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ;
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   const int tid = threadIdx.x;
@@ -396,148 +143,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
                     k0 * (B_KS ? d.ldb : 1);
 
   f32x16_t acc[TMI][TNJ];
-#pragma unroll
-  for (int i = 0; i < TMI; ++i)
-#pragma unroll
-    for (int j = 0; j < TNJ; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  StageAddr<C, A_KS> sa(A, d.lda, m0, tid, d.M);
-  StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
-  const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
-  const int KT = (dK + BK - 1) / BK;
-  bf16x8_t fa[TMI], fb[TNJ];
-
-#define DA_FREAD(st, ks)                                                                           \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
-        fa[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
-    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        fb[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
-  } while (0)
-#define DA_FREAD2(st, ks, FA, FB)                                                                  \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
-        FA[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
-    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        FB[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
-  } while (0)
-#define DA_MMA2(FA, FB)                                                                            \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
-        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[j], FA[i], acc[i][j], 0, 0, 0); \
-  } while (0)
-#define DA_MMA()                                                                                   \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
-        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0); \
-  } while (0)
-
-  if (FULL) {
-// one stage of both operands, straight into LDS: NCH wave-instructions of 1024 bytes each
-#define DA_DMA(st)                                                                                 \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sa.dbase, sa.doff + i * sa.dstep + koff_a, lds_addr(st) + (i * NW + wave) * 1024);   \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
-    koff_a += (unsigned)(sa.tstep * 2);                                                            \
-    if (koff_a == wrap_a) koff_a = 0;                                                              \
-    koff_b += (unsigned)(sb.tstep * 2);                                                            \
-  } while (0)
-    unsigned koff_a = 0, koff_b = 0;   // byte offset of the stage within the operand (< 4 GiB: checked by the launcher)
-    const unsigned wrap_a = (unsigned)d.a_kwrap * 2u;   // A read again from its first column (0: never, koff_a > 0 here)
-    DA_DMA(lds);
-    dma_wait();
-    __syncthreads();
-    // Fragments are double buffered in registers: the ds_reads of k-step s+1 are issued before
-    // the MFMAs of k-step s (scheduling fences keep the compiler from sinking them back down to
-    // their first use), and the stage barrier sits before the last k-step so that the first
-    // fragments of the next stage are fetched under the last MFMAs of this one.
-    bf16x8_t ga[TMI], gb[TNJ];
-    DA_FREAD(lds, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-      char* cur = lds + (kt & 1) * STAGE;
-      char* nxt = lds + ((kt + 1) & 1) * STAGE;
-      const bool more = kt + 1 < KT;
-      if (more) DA_DMA(nxt);
-      DA_FREAD2(cur, 1, ga, gb);
-      __builtin_amdgcn_sched_barrier(0);
-      DA_MMA();
-      __builtin_amdgcn_sched_barrier(0);
-      DA_FREAD(cur, 2);
-      __builtin_amdgcn_sched_barrier(0);
-      DA_MMA2(ga, gb);
-      __builtin_amdgcn_sched_barrier(0);
-      DA_FREAD2(cur, 3, ga, gb);
-      __builtin_amdgcn_sched_barrier(0);
-      DA_MMA();
-      __builtin_amdgcn_sched_barrier(0);
-      dma_wait();
-      __syncthreads();
-      if (more) DA_FREAD(nxt, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      DA_MMA2(ga, gb);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();
-#undef DA_DMA
-  } else {
-    u32x4_t ra[NCH], rb[NCH];
-    constexpr int A_RSTEP = A_KS ? C::NT / (BT / 8) : C::NT / 8;  // tile rows (k rows if k-strided) per chunk
-    constexpr int B_RSTEP = B_KS ? C::NT / (BT / 8) : C::NT / 8;
-#define DA_GLOAD(kt)                                                                               \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
-      const int r_ = sa.row + i * A_RSTEP;                                                         \
-      const bool ok = A_KS ? ((kt) * BK + r_ < dK && m0 + sa.col < d.M)                            \
-                           : (m0 + r_ < d.M && (kt) * BK + sa.col < dK);                           \
-      const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
-      ra[i] = ok ? *reinterpret_cast<const u32x4_t*>(sa.g + i * sa.gstep) : z_;                    \
-    }                                                                                              \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
-      const int r_ = sb.row + i * B_RSTEP;                                                         \
-      const bool ok = B_KS ? ((kt) * BK + r_ < dK && n0 + sb.col < d.N)                            \
-                           : (n0 + r_ < d.N && (kt) * BK + sb.col < dK);                           \
-      const u32x4_t z_ = {0u, 0u, 0u, 0u};                                                         \
-      rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;                    \
-    }                                                                                              \
-    sa.g += sa.tstep;                                                                              \
-    sb.g += sb.tstep;                                                                              \
-  } while (0)
-#define DA_LSTORE(st)                                                                              \
-  do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        *reinterpret_cast<u32x4_t*>((st) + sa.l + i * sa.lstep) = ra[i];                           \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        *reinterpret_cast<u32x4_t*>((st) + A_BYTES + sb.l + i * sb.lstep) = rb[i];                 \
-  } while (0)
-    DA_GLOAD(0);
-    DA_LSTORE(lds);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-      char* cur = lds + (kt & 1) * STAGE;
-      char* nxt = lds + ((kt + 1) & 1) * STAGE;
-      const bool more = kt + 1 < KT;
-      if (more) DA_GLOAD(kt + 1);
-#pragma unroll
-      for (int ks = 0; ks < BK / 16; ++ks) {
-        DA_FREAD(cur, ks);
-        DA_MMA();
-      }
-      if (more) DA_LSTORE(nxt);
-      __syncthreads();
-    }
-#undef DA_GLOAD
-#undef DA_LSTORE
-  }
-#undef DA_FREAD
-#undef DA_MMA
-#undef DA_FREAD2
-#undef DA_MMA2
+  gemm_tile_k_loop<C, A_KS, B_KS, MODE>(acc, d, A, B, dK, m0, n0, lds, tid, lane, wave, wm, wn);
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
   epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, tile.b, ti, tj, m0, n0, wave, lane, wm, wn);
   if (trace) {

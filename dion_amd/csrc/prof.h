@@ -19,7 +19,8 @@ enum DaProfKind {
   DA_PROF_DION_ELEM = 12, // B = M + G, column norms, guards
   DA_PROF_SCALAR_OPT = 13,// fused Lion / AdamW pass over non-matrix parameters
   DA_PROF_DION_EFUPD = 14,// error feedback and weight update in one pass
-  DA_PROF_KINDS = 15
+  DA_PROF_NS_FLOW = 15,   // all Newton-Schulz iterations of a set of buckets in one persistent launch
+  DA_PROF_KINDS = 16
 };
 
 struct DaProfScope {

@@ -320,7 +320,8 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
 #define DION_AMD_PROF_DION_ELEM 12
 #define DION_AMD_PROF_SCALAR_OPT 13
 #define DION_AMD_PROF_DION_EFUPD 14
-#define DION_AMD_PROF_KINDS 15
+#define DION_AMD_PROF_NS_FLOW 15
+#define DION_AMD_PROF_KINDS 16
 int dion_amd_profile_enable(int on);
 int dion_amd_profile_reset(void);
 /* Waits for the recorded events of `kind`; returns launch count, summed milliseconds and
@@ -334,6 +335,13 @@ int dion_amd_profile_read(int kind, long long* launches, double* total_ms, doubl
  *                   0: always as two products with the update in their epilogues (reference dion/dion.py:851-853
  *                   and 865-872 as two calls); -1: the default (one pass unless DION_AMD_NO_FUSED is set in the
  *                   environment).  Both roads give the same bits.
+ *   "ns_flow"       how the Newton-Schulz iterations of a bucket set are launched: 0 product by product (three
+ *                   grouped launches per iteration); 1 as one persistent launch whenever the shapes allow (wide
+ *                   dimensions multiples of 256); 2 the same with an L2 write-back after every tile (cross-check);
+ *                   -1 the default: DION_AMD_NS_FLOW in the environment if set, else the persistent launch for
+ *                   workloads of many small matrices.  All give the same bits.
+ *   "ns_flow_fail"  test hook: 1 makes every persistent launch start with its status word set, as if a wait had
+ *                   run into its limit; the results of such a launch are NaN.
  * The value applies to calls that start after this one returns, on every thread.  Unknown name:
  * DION_AMD_ERR_ARG. */
 int dion_amd_set_option(const char* name, int value);
@@ -347,6 +355,14 @@ int dion_amd_set_option(const char* name, int value);
  * CU ran at). */
 int dion_amd_tile_trace_enable(int on);
 int dion_amd_tile_trace_read(void* host_dst, int tiles);
+
+/* Time line of the persistent Newton-Schulz launch (no counterpart in the reference; used by the benchmark only).
+ * While enabled, every tile of such a launch records four readings of the 100 MHz counter -- taken from the queue,
+ * dependency met, K loop done, result published -- plus (queue << 48 | (3 * iteration + product) << 32 | ticket) and
+ * (XCC id << 32 | HW_ID).  `read` waits for the device and copies up to `max_tiles` records (six 64-bit words each)
+ * of the most recent traced launch to HOST memory; *tiles receives their number. */
+int dion_amd_ns_flow_trace_enable(int on);
+int dion_amd_ns_flow_trace_read(void* host_dst, int max_tiles, int* tiles);
 
 #ifdef __cplusplus
 }
