@@ -14,6 +14,8 @@ Workloads (numbered as the benchmark's configurations):
   dion_gpt_small_r025   (configs[2]) full Dion step on the same matrices, rank fraction 0.25,
   dion_gpt_small_r1     rank fraction 1.0; bf16 weights / momentum, fp32 Q, G seed 3.
   muon_llama8b_layer    (configs[3], one of the 32 layers) Muon on 7 bf16 matrices incl. 4096x14336.
+  muon_4096x14336       one bucket of 32 matrices of 4096x14336 (W_down of the 32 layers): the shape the
+                        Newton-Schulz target is quoted on, per-product fractions of the bf16 peak.
   dion_llama70b_layer   (configs[4], one of the 8 layers) Dion r=512 on 2 x 28672x8192 + 8192x28672.
   muon_llama8b          (configs[3], all 32 layers) 224 bf16 matrices, 6.98e9 elements, drawn on the GPU.
   dion_llama70b_mlp     (configs[4], all 8 layers) 24 bf16 matrices, 5.64e9 elements, drawn on the GPU.
@@ -46,6 +48,9 @@ WORKLOADS = {
                                desc="Muon step, one Llama-3-8B layer: 7 bf16 matrices incl. 4096x14336"),
     "dion_llama70b_layer": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER, seed=5, rank_fraction=1.0 / 16,
                                 desc="Dion step, one Llama-3-70B MLP layer (28672x8192 x2, 8192x28672), r=512"),
+    "muon_4096x14336": dict(kind="muon", shapes=[(4096, 14336)] * 32, seed=4, on_device=True,
+                            desc="Muon step on the bucket of 32 4096x14336 bf16 matrices (W_down of a Llama-3-8B stack): "
+                                 "the shape the 60 % target names"),
     "muon_llama8b": dict(kind="muon", shapes=LLAMA8B_LAYER * 32, seed=4, on_device=True,
                          desc="Full Muon step, Llama-3-8B-shaped stack: 32 layers x 7 bf16 matrices (6.98e9 elements)"),
     "dion_llama70b_mlp": dict(kind="dion", shapes=LLAMA70B_MLP_LAYER * 8, seed=5, rank_fraction=1.0 / 16, on_device=True,
@@ -319,6 +324,89 @@ def stream_ceiling(dev):
     return out
 
 
+def ceiling(dev):
+    """`--ceiling`: what the engines under a bf16 GEMM's K loop deliver on this GPU in this run, from probe kernels of
+    the library (dion_amd_probe): matrix cores alone (random operands in registers) with the shader clock they ran at,
+    and the L2 -> LDS stream of the operand staging alone."""
+    import ctypes
+
+    import torch
+    from dion_amd import _lib
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    src = torch.randn(max(cus * 49152, (cus + 31) // 32 * 65536) // 2, device=dev).bfloat16()
+    rec = torch.zeros(cus * 8 * 4, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, device=dev)
+    out = {}
+    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000)):
+        best = None
+        for _ in range(3):
+            ms = ctypes.c_double(0)
+            _lib.check(lib.dion_amd_probe(which, src.data_ptr(), src.numel() * 2, iters, rec.data_ptr(), rec.numel() * 8,
+                                          sink.data_ptr(), ctypes.byref(ms), _lib.stream_ptr(dev)), "dion_amd_probe")
+            r = rec.cpu().view(-1, 4)
+            mhz = float((r[:, 3] - r[:, 2]).sum()) / float((r[:, 1] - r[:, 0]).sum()) * 100.0
+            if best is None or ms.value < best[0]:
+                best = (ms.value, mhz)
+        ms, mhz = best
+        if which == 0:
+            flops = cus * 8 * iters * 32 * 32768.0
+            out[name] = dict(pflops=round(flops / (ms * 1e-3) / 1e15, 3), frac_of_2_5_pflops=round(flops / (ms * 1e-3) / PEAK_BF16_FLOPS, 3),
+                             shader_clock_mhz=round(mhz), ms=round(ms, 3),
+                             peak_at_that_clock_pflops=round(cus * 4096 * mhz * 1e6 / 1e15, 3))
+        else:
+            nbytes = cus * iters * 65536.0
+            out[name] = dict(tbps=round(nbytes / (ms * 1e-3) / 1e12, 2), shader_clock_mhz=round(mhz), ms=round(ms, 3),
+                             bytes_per_clock_per_cu=round(nbytes / cus / (ms * 1e-3) / (mhz * 1e6), 1))
+    out["streaming_kernel_gbps"] = stream_ceiling(dev)
+    return out
+
+
+def vendor_matmul(dev):
+    """`--vendor-matmul`: the three Newton-Schulz products of 4096 x 14336 matrices (a bucket of 32) as plain out-of-place
+    `torch.matmul` calls (the vendor GEMM library) next to this library's kernels on the same operands in the same run.
+    Dense flops 2 M N K for both, so the symmetric kernels' figures count the half they do not execute."""
+    import torch
+    from dion_amd.newton_schulz import gemm, ns_line_1, ns_line_2
+
+    bf = torch.bfloat16
+    b, m, n = 32, 4096, 14336
+    X = (torch.randn(b, m, n, device=dev) * 0.01).to(bf)
+    A = (torch.randn(b, m, m, device=dev) * 0.01).to(bf)
+    A = ((A + A.mT) * 0.5).contiguous()
+    Y = torch.empty_like(X)
+    A2 = torch.empty_like(A)
+
+    def timed(fn, reps=5):
+        for _ in range(2):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    cases = {
+        "X X^T (32 x 4096x14336)": (2.0 * b * m * m * n, lambda: torch.matmul(X, X.mT, out=A2), lambda: ns_line_1(X, out=A2)),
+        "A A (32 x 4096^3)": (2.0 * b * m * m * m, lambda: torch.matmul(A, A, out=A2),
+                             lambda: ns_line_2(A, 2.0315, -4.775, out=A2, faithful=True)),
+        "B X (32 x 4096x4096x14336)": (2.0 * b * m * m * n, lambda: torch.matmul(A, X, out=Y),
+                                      lambda: gemm(A, X, b_kstrided=True, E=X, s0=3.4445, s1=1.0, out=Y, faithful=True)),
+    }
+    out = {}
+    for name, (flops, vend, ours) in cases.items():
+        tv, to = timed(vend), timed(ours)
+        out[name] = dict(vendor_ms=round(tv, 3), vendor_dense_pflops=round(flops / (tv * 1e-3) / 1e15, 3),
+                         this_library_ms=round(to, 3), this_library_dense_pflops=round(flops / (to * 1e-3) / 1e15, 3),
+                         note="this library's launch includes the rounding-faithful epilogue (and the polynomial / axpy "
+                              "combine) and runs here on contiguous operands (row pitch a multiple of 4 KiB; the "
+                              "optimizer's working matrices carry 128 bytes of padding: see workload muon_4096x14336)")
+    return out
+
+
 def tile_trace(dev):
     """Time line of single bf16 GEMM launches (`--tile-trace`): per output tile, when its workgroup started, finished
     its K loop and finished its epilogue, and on which CU.  Prints one summary line per product: mean duration of the
@@ -405,6 +493,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--tile-trace", action="store_true",
                     help="instead of a workload: time lines of single bf16 GEMM launches (one JSON line per product)")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="instead of a workload: matrix-core-only and L2->LDS-only probe kernels with the shader clock")
+    ap.add_argument("--vendor-matmul", action="store_true",
+                    help="instead of a workload: torch.matmul on the 4096x14336 Newton-Schulz products next to this library")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three plain 512 MiB device copies (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -421,6 +513,12 @@ def main():
     dev = torch.device("cuda:0")
     if args.tile_trace:
         tile_trace(dev)
+        return
+    if args.ceiling:
+        print(json.dumps(dict(device=device_info(dev), ceiling=ceiling(dev))))
+        return
+    if args.vendor_matmul:
+        print(json.dumps(dict(device=device_info(dev), products=vendor_matmul(dev))))
         return
     if args.calibrate_copy:
         src = torch.ones(512 << 20, dtype=torch.uint8, device=dev)
@@ -457,12 +555,12 @@ def main():
     out.update({k: v for k, v in main_sum.items() if k not in ("workload", "ms_per_step", "steps")})
     if not args.no_extra:
         extra = {}
-        for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "dion_llama70b_layer",
+        for name in ("dion_gpt_small_r025", "dion_gpt_small_r1", "muon_llama8b_layer", "muon_4096x14336", "dion_llama70b_layer",
                      "muon_llama8b", "dion_llama70b_mlp", "scalar_gpt_small"):
             if name == args.workload:
                 continue
             w = WORKLOADS[name]
-            big = name in ("muon_llama8b", "dion_llama70b_mlp")   # hundreds of ms and tens of GB per step
+            big = name in ("muon_llama8b", "dion_llama70b_mlp", "muon_4096x14336")   # hundreds of ms and tens of GB per step
             r = measure(w, dev, 3 if big else 10, 1 if big else 2)
             s = summarize(name, w, r)
             s["roofline"] = roofline_of(r, w["kind"], name)

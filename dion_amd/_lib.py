@@ -63,6 +63,7 @@ _SIGNATURES = {
     "dion_amd_tile_trace_read": (_i, [_vp, _i]),
     "dion_amd_ns_flow_trace_enable": (_i, [_i]),
     "dion_amd_ns_flow_trace_read": (_i, [_vp, _i, _c.POINTER(_i)]),
+    "dion_amd_probe": (_i, [_i, _vp, _sz, _i, _vp, _sz, _vp, _c.POINTER(_c.c_double), _vp]),
     "dion_amd_profile_enable": (_i, [_i]),
     "dion_amd_profile_reset": (_i, []),
     "dion_amd_profile_read": (_i, [_i, _c.POINTER(_ll), _c.POINTER(_c.c_double), _c.POINTER(_c.c_double)]),

@@ -356,6 +356,17 @@ int dion_amd_set_option(const char* name, int value);
 int dion_amd_tile_trace_enable(int on);
 int dion_amd_tile_trace_read(void* host_dst, int tiles);
 
+/* Ceiling probes (no counterpart in the reference; used by the benchmark only).  which = 0: every wavefront of a
+ * launch of one 512-thread workgroup per compute unit issues `iters` x 32 v_mfma_f32_32x32x16_bf16 on operands held in
+ * registers, loaded once from `random_src` (device memory, at least compute units x 49152 bytes of random bf16).
+ * which = 1: every workgroup streams the same 64 KB of `random_src` (at least compute units / 32 x 65536 bytes) into
+ * LDS with direct-to-LDS loads `iters` times.  `records` (device memory, 32 bytes per wavefront = compute units x 256
+ * bytes) receives per wavefront the 100 MHz counter and the shader-clock counter at its start and end; `sink`: one
+ * float of device memory (never written in practice).  The call waits for the launch and returns its duration
+ * between two events on `stream` in *ms. */
+int dion_amd_probe(int which, const void* random_src, size_t src_bytes, int iters, void* records, size_t record_bytes,
+                   float* sink, double* ms, void* stream);
+
 /* Time line of the persistent Newton-Schulz launch (no counterpart in the reference; used by the benchmark only).
  * While enabled, every tile of such a launch records four readings of the 100 MHz counter -- taken from the queue,
  * dependency met, K loop done, result published -- plus (queue << 48 | (3 * iteration + product) << 32 | ticket) and
