@@ -59,6 +59,11 @@ _SIGNATURES = {
     "dion_amd_dion_step_qr": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i, _i,
                                    _vp, _vp, _sz, _vp]),
     "dion_amd_set_option": (_i, [_c.c_char_p, _i]),
+    "dion_amd_orthonormalize_sketch_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "dion_amd_orthonormalize_sketch": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "dion_amd_dion_sketch_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "dion_amd_dion_step_sketch": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i,
+                                       _vp, _i, _vp, _vp, _sz, _vp]),
     "dion_amd_tile_trace_enable": (_i, [_i]),
     "dion_amd_tile_trace_read": (_i, [_vp, _i]),
     "dion_amd_ns_flow_trace_enable": (_i, [_i]),

@@ -667,9 +667,9 @@ struct DionLayout {
   // of 8 (16-byte rows for every working matrix); the extra columns are zero throughout the step.
   int mp, np, r;
   size_t msz;           // bytes per element of the momentum dtype
-  size_t qc, p, rb, qn, orth, part, small;  // per-matrix byte sizes
+  size_t qc, p, rb, qn, orth, sketch, part, small;  // per-matrix byte sizes
   size_t per_matrix;
-  DionLayout(int m, int n, int rank, int m_dtype) {
+  DionLayout(int m, int n, int rank, int m_dtype, int sketch_k = 0) {
     mp = m < n ? n : m;
     np = m < n ? m : n;
     r = (rank + 7) & ~7;
@@ -679,10 +679,12 @@ struct DionLayout {
     rb = qc;
     qn = qc;
     orth = align_up(da_orth_workspace_bytes(1, mp, r), 256);
+    // (a sketched orthonormalisation keeps S P per matrix behind the orthonormaliser's own scratch)
+    sketch = sketch_k > 0 ? align_up(da_orth_sketch_extra_bytes(1, sketch_k, r), 256) : 0;
     // fp32 partial sums of R = B^T P when its inner dimension is cut into DA_MAX_GROUPS slices (bf16 only)
     part = m_dtype == DA_BF16 ? (size_t)DA_MAX_GROUPS * np * r * sizeof(float) : 0;
     small = 256;  // flags, info, pointer-table slots
-    per_matrix = qc + p + rb + qn + orth + part + small + 256;
+    per_matrix = qc + p + rb + qn + orth + sketch + part + small + 256;
   }
   size_t fixed() const { return 4 * DA_MAX_PTRS * sizeof(void*) + 2 * DA_MAX_PTRS * sizeof(int) + 1024; }
   int chunk(int batch, size_t ws_bytes) const {
@@ -701,6 +703,13 @@ struct DionLayout {
   }
 };
 
+}  // namespace
+
+namespace {
+int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
+                   int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
+                   float scaled_lr, float eps, int faithful, int power_iters, int qr_method, const void* sketch,
+                   int sketch_k, int* info, void* workspace, size_t workspace_bytes, void* stream);
 }  // namespace
 
 extern "C" {
@@ -738,6 +747,32 @@ int dion_amd_orthonormalize_method(const void* P, void* out, int dtype, int batc
   return da_orthonormalize(P, out, dtype, batch, rows, r, r, passes, qr_method, workspace, inf, s);
 }
 
+size_t dion_amd_orthonormalize_sketch_workspace_bytes(int batch, int rows, int r, int k) {
+  if (batch <= 0 || rows <= 0 || r <= 0 || k <= 0) return 0;
+  return align_up(dion_amd_orthonormalize_workspace_bytes(batch, rows, r), 256) + da_orth_sketch_extra_bytes(batch, k, r);
+}
+
+int dion_amd_orthonormalize_sketch(const void* P, const void* S, void* out, int dtype, int batch, int rows, int r, int k,
+                                   int* info, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!P || !S || !out || !workspace || batch <= 0 || rows <= 0 || r <= 0 || k < r) return DA_ERR_ARG;
+  if (!dtype_ok(dtype)) return DA_ERR_DTYPE;
+  if (r > rows) return DA_ERR_ARG;
+  // S P runs on the matrix cores of the factor's dtype: 16-byte rows for S, P and the product
+  const int grid = dtype == DA_BF16 ? 7 : 3;
+  if ((rows | r | k) & grid) return DA_ERR_ALIGN;
+  if (workspace_bytes < dion_amd_orthonormalize_sketch_workspace_bytes(batch, rows, r, k)) return DA_ERR_WORKSPACE;
+  if ((uintptr_t)workspace & 255) return DA_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char* base = static_cast<char*>(workspace);
+  const size_t own = align_up(dion_amd_orthonormalize_workspace_bytes(batch, rows, r), 256);
+  int* inf = info;
+  if (!inf) inf = reinterpret_cast<int*>(base + align_up(da_orth_workspace_bytes(batch, rows, r), 256));
+  int rc = da_fill_int(inf, batch, 0, s);
+  if (rc) return rc;
+  DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
+  return da_orthonormalize_sketch(P, S, out, dtype, batch, rows, r, r, k, workspace, base + own, inf, s);
+}
+
 int dion_amd_dion_step(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
                        int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
                        float scaled_lr, float eps, int faithful, int power_iters, int* info, void* workspace,
@@ -750,6 +785,32 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
                           int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
                           float scaled_lr, float eps, int faithful, int power_iters, int qr_method, int* info,
                           void* workspace, size_t workspace_bytes, void* stream) {
+  return dion_step_impl(X, G, M, Q, batch, m, n, rank, x_dtype, g_dtype, m_dtype, q_dtype, ef_alpha, decay, scaled_lr, eps,
+                        faithful, power_iters, qr_method, nullptr, 0, info, workspace, workspace_bytes, stream);
+}
+
+size_t dion_amd_dion_sketch_workspace_bytes(int batch, int m, int n, int r, int m_dtype, int sketch_k) {
+  if (batch <= 0 || m <= 0 || n <= 0 || r <= 0 || sketch_k <= 0 || !dtype_ok(m_dtype)) return 0;
+  return DionLayout(m, n, r, m_dtype, sketch_k).recommended(batch);
+}
+
+int dion_amd_dion_step_sketch(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m,
+                              int n, int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha,
+                              float decay, float scaled_lr, float eps, int faithful, int power_iters, const void* sketch,
+                              int sketch_k, int* info, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!sketch || sketch_k <= 0) return DA_ERR_ARG;
+  return dion_step_impl(X, G, M, Q, batch, m, n, rank, x_dtype, g_dtype, m_dtype, q_dtype, ef_alpha, decay, scaled_lr, eps,
+                        faithful, power_iters, DA_QR_AUTO, sketch, sketch_k, info, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* const* Q, int batch, int m, int n,
+                   int rank, int x_dtype, int g_dtype, int m_dtype, int q_dtype, float ef_alpha, float decay,
+                   float scaled_lr, float eps, int faithful, int power_iters, int qr_method, const void* sketch,
+                   int sketch_k, int* info, void* workspace, size_t workspace_bytes, void* stream) {
   if (qr_method < 0 || qr_method > 2) return DA_ERR_ARG;
   if (!X || !G || !M || !Q || !workspace || batch <= 0 || m <= 0 || n <= 0 || rank <= 0) return DA_ERR_ARG;
   if (power_iters < 1 || power_iters > 64) return DA_ERR_ARG;
@@ -762,8 +823,9 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
     if (((uintptr_t)X[i] | (uintptr_t)G[i] | (uintptr_t)M[i] | (uintptr_t)Q[i]) & 15) return DA_ERR_ALIGN;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const DionLayout L(m, n, rank, m_dtype);
+  const DionLayout L(m, n, rank, m_dtype, sketch ? sketch_k : 0);
   const int r = L.r;   // padded rank: pitch and logical width of Qc, P, R, Qn
+  if (sketch && (sketch_k < rank || (sketch_k & 7))) return DA_ERR_ARG;
   const int chunk = L.chunk(batch, workspace_bytes);
   if (chunk < 1) return DA_ERR_WORKSPACE;
   const bool transposed = m < n;
@@ -788,7 +850,8 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
     char* R = w; w += L.rb * cb;
     char* Qn = w; w += L.qn * cb;
     char* orth_ws = reinterpret_cast<char*>(align_up(reinterpret_cast<uintptr_t>(w), 256));
-    float* parts = reinterpret_cast<float*>(orth_ws + L.orth * cb);
+    char* sketch_ws = orth_ws + L.orth * cb;
+    float* parts = reinterpret_cast<float*>(sketch_ws + L.sketch * cb);
     const long long sQ = (long long)(L.qc / L.msz), sP = (long long)(L.p / L.msz);
 
     DaPtrTable tx{}, tg{}, tm{}, tq{};
@@ -825,7 +888,14 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
       // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
       {
         DaProfScope prof(DA_PROF_DION_ORTH, 0.0, s);
-        rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, qr_method, orth_ws, linfo, s);
+        if (sketch) {
+          // sketches: [power iteration][matrix of the bucket][sketch_k][mp] in the momentum dtype
+          const char* S = static_cast<const char*>(sketch) +
+                          ((size_t)it * batch + b0) * (size_t)sketch_k * mp * L.msz;
+          rc = da_orthonormalize_sketch(P, S, P, m_dtype, cb, mp, r, rank, sketch_k, orth_ws, sketch_ws, linfo, s);
+        } else {
+          rc = da_orthonormalize(P, P, m_dtype, cb, mp, r, rank, 2, qr_method, orth_ws, linfo, s);
+        }
         if (rc) return rc;
         // all-zero / NaN guard on P   (reference dion/dion.py:847, 1416-1444)
         rc = da_fix(P, nullptr, m_dtype, sP, cb, nonzero, s);
@@ -912,4 +982,4 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
   return DA_OK;
 }
 
-}  // extern "C"
+}  // namespace

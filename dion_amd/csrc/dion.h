@@ -36,6 +36,12 @@ size_t da_orth_workspace_bytes(int batch, int rows, int r);
 int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, int r, int r_live, int passes,
                       int method, void* ws, int* info, hipStream_t s);
 
+// Randomised Cholesky QR with a sketch given by the caller (reference dion/dion.py:1287-1303): S is batch x k x rows
+// in P's dtype (k >= r_live); `extra`: da_orth_sketch_extra_bytes(batch, k, r) bytes beyond `ws`.
+size_t da_orth_sketch_extra_bytes(int batch, int k, int r);
+int da_orthonormalize_sketch(const void* P, const void* S, void* out, int dtype, int batch, int rows, int r, int r_live,
+                             int k, void* ws, void* extra, int* info, hipStream_t s);
+
 // Error feedback and weight update in one pass (dion_fused.hip), bf16 factors:
 //   M[b] <- M[b] + ef_alpha P[b] R[b]^T,  X[b] <- decay X[b] - scaled_lr P[b] Qn[b]^T   (R P^T, Qn P^T when `transposed`)
 // with every rounding of the reference's separate tensor ops.  P: batch x mp x r, R / Qn: batch x np x r (contiguous);

@@ -555,10 +555,11 @@ inline int chol_step_real(float* G, float* L, float* W, long long sG, int r, int
 // G = P^T P (K-sliced if that fills the GPU; the slices are added in a fixed order), padded diagonal, and
 // optionally the rows' squared defects.
 template <typename T>
-int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, float* rowdef, DaGate gate, hipStream_t s) {
+int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, float* rowdef, DaGate gate, hipStream_t s,
+         bool unsliced = false) {
   const long long pr = (long long)rows * r, rr = (long long)r * r;
   // (as the fall-back of flagged matrices: unsliced, so that no finishing launch is needed)
-  const int sp = gate.flags ? 1 : gram_slices(batch, rows, r);
+  const int sp = gate.flags || unsliced ? 1 : gram_slices(batch, rows, r);
   RealGemmDesc<T> g{};
   g.batch = batch;
   g.A = P; g.B = P; g.C = sp > 1 ? part : G; g.E = nullptr;
@@ -581,18 +582,8 @@ int gram(const T* P, T* G, T* part, int batch, int rows, int r, int r_live, floa
 // Most 64 x 64 tiles (over the batch) a trailing update may have to ride along in the next step's launch.
 const long long DA_CHOL_DEFER_TILES = [] { const char* e = getenv("DION_AMD_CHOL_DEFER_TILES"); const long long v = e ? atoll(e) : 0; return v > 0 ? v : 256; }();
 
-// One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
-template <typename T>
-int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, int r_live, int* info, DaGate gate,
-                hipStream_t s, T* pstat = nullptr) {
-  const int NB = DA_CHOL_NB;
-  const int nblk = (r + NB - 1) / NB;
-  const long long pr = (long long)rows * r, rr = (long long)r * r;
-  int rc = gram<T>(P0, G, part, batch, rows, r, r_live, nullptr, gate, s);
-  if (rc) return rc;
-  // Two-level blocking: 64-column steps inside panels of `pw` steps.  A step's rank-64 update reaches only the
-  // rest of its panel's columns; what lies right of the panel gets one rank-(64 pw) update when the panel is done
-  // (the trailing matrix is then read and written once per panel instead of once per step).
+// Panel width (in 64-column steps) of the two-level blocking of chol_factor / apply_rinv.
+int chol_panel_steps(int nblk, bool fallback) {
   static const int pw_env = [] {
     const char* e = getenv("DION_AMD_CHOL_PANEL");
     const int v = e ? atoi(e) : 0;
@@ -600,8 +591,22 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
   }();
   // As the pass for flagged matrices only (gated), most launches find nothing to do and what counts is their number:
   // one level, every trailing update deferred into the next step's launch.
+  return fallback ? nblk : pw_env;
+}
+
+// Blocked lower Cholesky G = L L^T of each r x r matrix (G is overwritten), with the inverse-factor blocks W that
+// apply_rinv uses.
+template <typename T>
+int chol_factor(T* G, T* L, T* W, int batch, int r, int* info, DaGate gate, hipStream_t s, T* pstat = nullptr) {
+  const int NB = DA_CHOL_NB;
+  const int nblk = (r + NB - 1) / NB;
+  const long long rr = (long long)r * r;
+  int rc = DA_OK;
+  // Two-level blocking: 64-column steps inside panels of `pw` steps.  A step's rank-64 update reaches only the
+  // rest of its panel's columns; what lies right of the panel gets one rank-(64 pw) update when the panel is done
+  // (the trailing matrix is then read and written once per panel instead of once per step).
   const bool fallback = gate.flags != nullptr;
-  const int pw = fallback ? nblk : pw_env;
+  const int pw = chol_panel_steps(nblk, fallback);
   // (the rank-64 updates inside a panel ride along in the next step's launch instead of taking one of their own)
   static const bool defer = [] { const char* e = getenv("DION_AMD_CHOL_NO_DEFER"); return !(e && atoi(e)); }();
   bool pending = false;   // the previous step left its update to the next launch
@@ -646,7 +651,18 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
       if (rc) return rc;
     }
   }
-  // P0 <- P0 R^-1 with R = L^T, in place, by the same panels: first the solved columns left of the panel are
+  return DA_OK;
+}
+
+// P0 <- P0 R^-1 with R = L^T (L, W from chol_factor), in place, `rows` rows per matrix.
+template <typename T>
+int apply_rinv(T* P0, const T* L, const T* W, int batch, int rows, int r, DaGate gate, hipStream_t s) {
+  const int NB = DA_CHOL_NB;
+  const int nblk = (r + NB - 1) / NB;
+  const long long pr = (long long)rows * r, rr = (long long)r * r;
+  const int pw = chol_panel_steps(nblk, gate.flags != nullptr);
+  int rc = DA_OK;
+  // By the panels of the factorisation: first the solved columns left of the panel are
   // taken out of it in one product,
   //   P0[:, panel] -= P0[:, 0 .. p0] L[panel, 0 .. p0]^T
   // then block column by block column inside it
@@ -681,6 +697,17 @@ int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, in
     if (rc) return rc;
   }
   return DA_OK;
+}
+
+// One blocked CholeskyQR pass in precision T, in place:  P <- P R^-1  with  P^T P = R^T R.
+template <typename T>
+int cholqr_pass(T* P0, T* G, T* L, T* W, T* part, int batch, int rows, int r, int r_live, int* info, DaGate gate,
+                hipStream_t s, T* pstat = nullptr) {
+  int rc = gram<T>(P0, G, part, batch, rows, r, r_live, nullptr, gate, s);
+  if (rc) return rc;
+  rc = chol_factor<T>(G, L, W, batch, r, info, gate, s, pstat);
+  if (rc) return rc;
+  return apply_rinv<T>(P0, L, W, batch, rows, r, gate, s);
 }
 
 // V = I - up(G - I) for each r x r Gram matrix G of an almost orthonormal P, where up() keeps the strict
@@ -1301,3 +1328,54 @@ int da_orthonormalize(const void* P, void* out, int dtype, int batch, int rows, 
   }
   return zero_cols(out, dtype, w.bad, info, batch, rows, r, gate2, s);
 }
+
+// Scratch of da_orthonormalize_sketch beyond da_orth_workspace_bytes: S P in the factor's dtype and in fp64.
+size_t da_orth_sketch_extra_bytes(int batch, int k, int r) {
+  const size_t kr = (size_t)batch * k * r;
+  return orth_align(kr * 4) + orth_align(kr * 8) + 256;
+}
+
+// The reference's randomised Cholesky QR with the sketch S given by the caller (reference dion/dion.py:1287-1303):
+//   SP = S P (in P's dtype);  R1 = R-factor of SP;  P1 = P R1^-1;  R2 = chol(P1^T P1);  Q = P1 R2^-1.
+// R1 is taken as the Cholesky factor of (SP)^T (SP) formed in fp64 -- the R-factor of a Householder QR of SP up to
+// the signs of its rows, which P1's column space does not see -- and both triangular solves and the second
+// factorisation run in fp64 as well (the reference's are fp32).  rows <= r: the reference factors such a P by
+// Householder QR without a sketch (1283-1285); here: the fp64 pass.
+int da_orthonormalize_sketch(const void* P, const void* S, void* out, int dtype, int batch, int rows, int r, int r_live,
+                             int k, void* ws, void* extra, int* info, hipStream_t s) {
+  if (rows <= r_live) return da_orthonormalize(P, out, dtype, batch, rows, r, r_live, 2, DA_QR_FP64, ws, info, s);
+  if (!S || !extra || k < r_live || batch > 65535 || r_live < 1 || r_live > r || r - r_live > 63) return DA_ERR_ARG;
+  const long long pr = (long long)rows * r, kr = (long long)k * r, ks = (long long)k * rows;
+  const OrthWs w(ws, batch, rows, r);
+  const DaGate all{nullptr, 0};
+  char* x = static_cast<char*>(extra);
+  void* SPlow = x;
+  double* SP = reinterpret_cast<double*>(x + orth_align((size_t)batch * kr * 4));
+  // ---- SP = S P, rounded to the factor's dtype as the reference's matmul does
+  GemmDesc g{};
+  g.batch = batch;
+  g.A = S; g.sA = ks; g.lda = rows; g.a_kstrided = 0;
+  g.B = P; g.sB = pr; g.ldb = r; g.b_kstrided = 1;
+  g.C = SPlow; g.sC = kr; g.ldc = r; g.c_dtype = dtype;
+  g.M = k; g.N = r; g.K = rows;
+  g.epilogue = DA_EPI_STORE; g.s1 = 1.f; g.faithful = 0;
+  int rc = dtype == DA_BF16 ? da_gemm_bf16(g, s) : da_gemm_f32(g, s);
+  if (rc) return rc;
+  rc = da_cvt_to_f64(SPlow, dtype, SP, kr, batch, all, s);
+  if (rc) return rc;
+  // ---- R1^T R1 = (SP)^T (SP)
+  rc = gram<double>(SP, w.G, w.part, batch, k, r, r_live, nullptr, all, s, true);
+  if (rc) return rc;
+  rc = chol_factor<double>(w.G, w.L, w.W, batch, r, info, all, s);
+  if (rc) return rc;
+  // ---- P1 = P R1^-1
+  rc = da_cvt_to_f64(P, dtype, w.P0, pr, batch, all, s);
+  if (rc) return rc;
+  rc = apply_rinv<double>(w.P0, w.L, w.W, batch, rows, r, all, s);
+  if (rc) return rc;
+  // ---- Cholesky QR of the preconditioned factor
+  rc = cholqr_pass<double>(w.P0, w.G, w.L, w.W, w.part, batch, rows, r, r_live, info, all, s);
+  if (rc) return rc;
+  return da_cvt_from_f64(w.P0, out, dtype, pr, batch, all, s);
+}
+

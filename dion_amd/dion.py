@@ -6,15 +6,17 @@ arguments, defaults, validation errors, param-group keys and `self.state` layout
 `replicate_mesh`, `outer_shard_mesh` and `inner_shard_mesh` must be None.
 
 Per `step()` the matrices of every "dion" group are bucketed by (shape, dtype) and each bucket
-goes, as arrays of device pointers, to `dion_amd_dion_step`: B = M + G, the tall-skinny MFMA
-GEMMs P = B Q and R = B^T P, a CholeskyQR2 orthonormalisation of P on the device (fp64 pass, fp32 polish), the
-error-feedback and weight updates fused into GEMM epilogues, and the column normalisation
-that yields the next Q.
+goes, as arrays of device pointers, to `dion_amd_dion_step_qr`: B = M + G, the tall-skinny MFMA
+GEMMs P = B Q and R = B^T P, a CholeskyQR orthonormalisation of P on the device (an fp32 pass on the bf16 matrix
+cores, an fp64 pass for the factors whose measured defect asks for it, a closed-form polishing step; no host
+synchronisation), the column normalisation that yields the next Q, and error feedback and weight update as one
+pass over M and X.
 """
 import math
 import os
 from collections import defaultdict
 from concurrent.futures import ThreadPoolExecutor
+from concurrent.futures import wait as wait_futures
 from dataclasses import dataclass
 from typing import Any, Dict, Optional, Tuple
 
@@ -36,10 +38,10 @@ class DionMixedPrecisionConfig:
 
 
 
-def _enqueue_dion_step(lib, device, args):
+def _enqueue_dion_step(fn, device, args):
     """One bucket's library call, made by a worker thread (ctypes releases the interpreter lock for its duration)."""
     torch.cuda.set_device(device)
-    return lib.dion_amd_dion_step_qr(*args)
+    return fn(*args)
 
 
 class Dion(Optimizer):
@@ -53,9 +55,10 @@ class Dion(Optimizer):
         replicate_mesh_grad_sync: accepted; irrelevant on one GPU.
         rank_fraction, rank_multiple_of: r = multiple_of * ceil(fraction * min(m, n) / multiple_of).
         lr, mu, betas, weight_decay, epsilon: as in the reference.
-        power_iters: must be 1.  qr_method: must be "rcqr" (the reference's only accepted value;
-            the device orthonormaliser is a CholeskyQR2 that yields the same factor up to column signs).
-        cqr_warmup_steps, rcqr_oversample: accepted for compatibility (no sketch is drawn).
+        power_iters: must be 1.  qr_method: must be "rcqr" (the batched reference class accepts nothing else); the
+            device orthonormaliser yields the reference's factor up to column signs without drawing a sketch.
+        cqr_warmup_steps: steps during which `DionReference` runs "rcqr" in place of "cqr".
+        rcqr_oversample: sketch rows per rank (`DionReference` with "rcqr" draws the reference's sketches).
         mixed_precision_config: dtypes of momentum / Q / variance.
     """
 
@@ -136,6 +139,7 @@ class Dion(Optimizer):
         self._streams = {}
         self._info = {}
         self._pool = None   # worker threads that enqueue the buckets of a wave side by side
+        self._rng = None    # generator of the random sketches (DionReference with qr_method "rcqr")
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -271,83 +275,109 @@ class Dion(Optimizer):
             self._pool = ThreadPoolExecutor(max_workers=self._max_concurrent_tasks, thread_name_prefix="dion_amd")
         forked = {}
         items = list(buckets.items())
-        for wave0 in range(0, len(items), slots):
-            pending = []
-            for index in range(wave0, min(wave0 + slots, len(items))):
-                (shape, dtype, gdtype, device), plist = items[index]
-                slot = index % slots
-                main = torch.cuda.current_stream(device)
-                if slots == 1:
-                    stream = main
-                else:
-                    pool = self._streams.setdefault(device, [])
-                    while len(pool) < slots:
-                        pool.append(torch.cuda.Stream(device=device))
-                    stream = pool[slot]
-                    if (device, slot) not in forked:
-                        stream.wait_stream(main)   # gradients and earlier updates were produced on `main`
-                        forked[(device, slot)] = (main, stream)
-                states = [self._get_or_initialize_state(p, group) for p in plist]
-                m, n = shape
-                Ms = [s["momentum"] for s in states]
-                Qs = [s["Q"] for s in states]
-                r = Qs[0].size(1)
-                for t in (*plist, *Ms, *Qs):
-                    if not t.is_contiguous():
-                        raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
-                scaled_lr = ((m / n) ** 0.5) * lr
-                mcode = _lib.dtype_code(Ms[0].dtype)
-                info = self._info[(shape, dtype, gdtype, device)]
-                with torch.cuda.device(device), torch.cuda.stream(stream):
-                    # contiguous gradient copies and the workspace belong to this stream
-                    Xs = plist
-                    Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
-                    crops = []
-                    if m % 8 or n % 8:
-                        # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
-                        m, n = _lib.padded_dims(m, n)
-                        Xw, Gw, Mw = (_lib.zero_padded(t, m, n) for t in (plist, Gs, Ms))
-                        Qw = _lib.zero_padded(Qs, min(m, n), r)
-                        crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
-                        Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
-                    ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
-                    # Cholesky QR only after the warm-up, when the factors are well conditioned
-                    # (reference dion/dion_reference.py:296-299)
-                    qr_method = self._qr_method
-                    if qr_method == "cqr" and group["step"] <= self._cqr_warmup_steps:
-                        qr_method = "rcqr"
-                    args = (
-                        _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
-                        len(plist), m, n, r,
-                        _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
-                        ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
-                        _lib.QR_METHODS[qr_method],
-                        info.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_ptr(device),
-                    )
-                    if threaded:
-                        # (the tensors behind the pointers stay referenced until the call has returned)
-                        pending.append((self._pool.submit(_enqueue_dion_step, lib, device, args), device, stream, crops,
-                                        (Xs, Gs, Ms, Qs, ws)))
-                        continue
-                    rc = lib.dion_amd_dion_step_qr(*args)
-                    _lib.check(rc, "dion_amd_dion_step_qr")
-                    for dst, padded in crops:
-                        _lib.crop_back(dst, padded)
-                    del Xs, Gs, Ms, Qs, crops
-            failure = None
-            for future, device, stream, crops, keep in pending:
-                rc = future.result()   # every call of the wave has returned before anything is raised
-                if rc != 0 and failure is None:
-                    failure = rc
-                if rc == 0 and crops:
+        pending = []
+        # Whatever happens while a wave is put together -- a non-contiguous tensor, an allocation that fails, a
+        # library call that returns an error -- the calls already handed to worker threads are waited for (they hold
+        # raw pointers into tensors of this frame) and the forked streams are joined before the exception travels on.
+        try:
+            for wave0 in range(0, len(items), slots):
+                pending = []
+                for index in range(wave0, min(wave0 + slots, len(items))):
+                    (shape, dtype, gdtype, device), plist = items[index]
+                    slot = index % slots
+                    main = torch.cuda.current_stream(device)
+                    if slots == 1:
+                        stream = main
+                    else:
+                        pool = self._streams.setdefault(device, [])
+                        while len(pool) < slots:
+                            pool.append(torch.cuda.Stream(device=device))
+                        stream = pool[slot]
+                        if (device, slot) not in forked:
+                            stream.wait_stream(main)   # gradients and earlier updates were produced on `main`
+                            forked[(device, slot)] = (main, stream)
+                    states = [self._get_or_initialize_state(p, group) for p in plist]
+                    m, n = shape
+                    Ms = [s["momentum"] for s in states]
+                    Qs = [s["Q"] for s in states]
+                    r = Qs[0].size(1)
+                    for t in (*plist, *Ms, *Qs):
+                        if not t.is_contiguous():
+                            raise _lib.DionAmdError("Dion.step: parameters and optimizer states must be contiguous")
+                    scaled_lr = ((m / n) ** 0.5) * lr
+                    mcode = _lib.dtype_code(Ms[0].dtype)
+                    info = self._info[(shape, dtype, gdtype, device)]
                     with torch.cuda.device(device), torch.cuda.stream(stream):
+                        # contiguous gradient copies and the workspace belong to this stream
+                        Xs = plist
+                        Gs = [p.grad if p.grad.is_contiguous() else p.grad.contiguous() for p in plist]
+                        crops = []
+                        if m % 8 or n % 8:
+                            # step zero-padded copies (exact: see _lib.zero_padded) and crop the results back
+                            m, n = _lib.padded_dims(m, n)
+                            Xw, Gw, Mw = (_lib.zero_padded(t, m, n) for t in (plist, Gs, Ms))
+                            Qw = _lib.zero_padded(Qs, min(m, n), r)
+                            crops = [(plist, Xw), (Ms, Mw), (Qs, Qw)]
+                            Xs, Gs, Ms, Qs = (list(t.unbind(0)) for t in (Xw, Gw, Mw, Qw))
+                        # Cholesky QR only after the warm-up, when the factors are well conditioned
+                        # (reference dion/dion_reference.py:296-299)
+                        qr_method = self._qr_method
+                        if qr_method == "cqr" and group["step"] <= self._cqr_warmup_steps:
+                            qr_method = "rcqr"
+                        head = (
+                            _lib.ptr_array(Xs), _lib.ptr_array(Gs), _lib.ptr_array(Ms), _lib.ptr_array(Qs),
+                            len(plist), m, n, r,
+                            _lib.dtype_code(dtype), _lib.dtype_code(gdtype), mcode, _lib.dtype_code(Qs[0].dtype),
+                            ef_alpha.item(), decay.item(), scaled_lr.item(), epsilon.item(), 1, self._power_iters,
+                        )
+                        sketch = None
+                        if self._REFERENCE_OPTIONS and qr_method == "rcqr" and max(m, n) > r:
+                            # the per-matrix reference class preconditions with a random sketch from a generator of its own,
+                            # seeded with 0 (reference dion/dion_reference.py:290-294, 764-775): one sketch per matrix and
+                            # power iteration, drawn here and handed to the library
+                            if self._rng is None:
+                                self._rng = torch.Generator(device=device)
+                                self._rng.manual_seed(0)
+                            sketch = _sketch((self._power_iters * len(plist), max(m, n), r), Ms[0].dtype, device,
+                                             group["oversample"], self._rng)
+                            k = sketch.size(-2)
+                            ws = self._workspaces[slot].get(
+                                lib.dion_amd_dion_sketch_workspace_bytes(len(plist), m, n, r, mcode, k), device)
+                            fn, what = lib.dion_amd_dion_step_sketch, "dion_amd_dion_step_sketch"
+                            args = head + (sketch.data_ptr(), k, info.data_ptr(), ws.data_ptr(), ws.numel(),
+                                           _lib.stream_ptr(device))
+                        else:
+                            ws = self._workspaces[slot].get(lib.dion_amd_dion_workspace_bytes(len(plist), m, n, r, mcode), device)
+                            fn, what = lib.dion_amd_dion_step_qr, "dion_amd_dion_step_qr"
+                            args = head + (_lib.QR_METHODS[qr_method], info.data_ptr(), ws.data_ptr(), ws.numel(),
+                                           _lib.stream_ptr(device))
+                        if threaded:
+                            # (the tensors behind the pointers stay referenced until the call has returned)
+                            pending.append((self._pool.submit(_enqueue_dion_step, fn, device, args), device, stream, crops,
+                                            (Xs, Gs, Ms, Qs, ws, sketch), what))
+                            continue
+                        rc = fn(*args)
+                        _lib.check(rc, what)
                         for dst, padded in crops:
                             _lib.crop_back(dst, padded)
-            del pending
-            if failure is not None:
-                _lib.check(failure, "dion_amd_dion_step_qr")
-        for main, stream in forked.values():
-            main.wait_stream(stream)
+                        del Xs, Gs, Ms, Qs, crops
+                failure = None
+                for future, device, stream, crops, keep, what in pending:
+                    rc = future.result()   # every call of the wave has returned before anything is raised
+                    if rc != 0 and failure is None:
+                        failure = (rc, what)
+                    if rc == 0 and crops:
+                        with torch.cuda.device(device), torch.cuda.stream(stream):
+                            for dst, padded in crops:
+                                _lib.crop_back(dst, padded)
+                pending = []
+                if failure is not None:
+                    _lib.check(*failure)
+        finally:
+            if pending:
+                wait_futures([item[0] for item in pending])
+            for main, stream in forked.values():
+                main.wait_stream(stream)
 
     # ------------------------------------------------------------------ element-wise groups
     def _lion_group_step(self, group: dict):
@@ -374,19 +404,26 @@ class Dion(Optimizer):
         )
 
 
-def generate_random_sketch_matrix(P: Tensor, oversample: float = 1.25, shard_mesh_dim=None) -> Tensor:
+def _sketch(p_shape, dtype, device, oversample, generator=None) -> Tensor:
+    """S ~ N(0, 1/k) of shape (..., k, m) for factors of shape p_shape = (..., m, r), k = oversample * r rounded up to a
+    multiple of 128 (reference dion/dion.py:1234-1261)."""
+    m, r = p_shape[-2], p_shape[-1]
+    k = math.ceil(oversample * r / 128.0) * 128
+    std = math.sqrt(1.0 / k)
+    return torch.empty((*p_shape[:-2], k, m), device=device, dtype=dtype).normal_(std=std, generator=generator)
+
+
+def generate_random_sketch_matrix(P: Tensor, oversample: float = 1.25, shard_mesh_dim=None, generator=None) -> Tensor:
     """The sketch of the reference's randomised Cholesky QR (dion/dion.py:1221-1263) for a batch P of shape
     (..., m, r): S of shape (..., k, m) with k = oversample * r rounded up to a multiple of 128 and entries
-    N(0, 1/k) in P's dtype, drawn from torch's generator for P's device.  The device orthonormaliser draws no
-    sketch (its "rcqr" preconditions with an fp32 CholeskyQR pass instead), so nothing in `Dion.step()` calls this;
-    it is here for callers of the reference's helper.  One GPU: `shard_mesh_dim` must be None."""
+    N(0, 1/k) in P's dtype, drawn from torch's generator for P's device (or from `generator`).
+    `orthonormalize(P, sketch=S)` and `DionReference` (qr_method "rcqr") run the reference's sketched sequence with it;
+    `Dion.step()` itself draws no sketch (its orthonormaliser preconditions with an fp32 CholeskyQR pass instead).
+    One GPU: `shard_mesh_dim` must be None."""
     assert P.ndim >= 3, "P must have batch dimension"
     if shard_mesh_dim is not None:
         raise TypeError("Must use DTensor parameters for sharded random sketch.")
-    m, r = P.size(-2), P.size(-1)
-    k = math.ceil(oversample * r / 128.0) * 128
-    std = math.sqrt(1.0 / k)
-    return torch.empty((*P.shape[:-2], k, m), device=P.device, dtype=P.dtype).normal_(std=std)
+    return _sketch(P.shape, P.dtype, P.device, oversample, generator)
 
 
 class DionReference(Dion):

@@ -146,18 +146,36 @@ def gemm(A: Tensor, B: Tensor, *, a_kstrided=False, b_kstrided=False, E: Tensor 
     return out if A.ndim == 3 else out[0]
 
 
-def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False, qr_method: str = "rcqr"):
+def orthonormalize(P: Tensor, passes: int = 2, return_info: bool = False, qr_method: str = "rcqr",
+                   sketch: Tensor = None):
     """Thin-QR Q factor of P (rows x r) or a batch of them on the device; counterpart of `orthogonalize`
     (reference dion/dion.py:1267-1308, dion/dion_reference.py:733-789), equal up to column signs.
     qr_method: "rcqr" -- CholeskyQR in fp32, in fp64 for the matrices whose measured defect asks for it, then a
     polishing pass; "qr" -- the fp64 pass for every matrix; "cqr" -- one fp32 CholeskyQR pass and nothing else
-    (fp64 pass only if the factorisation fails)."""
+    (fp64 pass only if the factorisation fails).
+    sketch: the reference's randomised Cholesky QR with this random sketch S (k x rows per matrix, P's dtype; see
+    `dion_amd.dion.generate_random_sketch_matrix`), reference dion/dion.py:1287-1303; `qr_method` must be "rcqr"."""
     lib = _lib.load()
     _lib.require_gpu(P, "orthonormalize")
     P3 = (P if P.ndim == 3 else P.unsqueeze(0)).contiguous()
     batch, rows, r = P3.shape
     out = torch.empty_like(P3)
     info = torch.zeros(batch, dtype=torch.int32, device=P.device)
+    if sketch is not None:
+        if qr_method != "rcqr":
+            raise ValueError("a sketch belongs to qr_method='rcqr'")
+        S3 = (sketch if sketch.ndim == 3 else sketch.unsqueeze(0)).contiguous()
+        if S3.dtype != P3.dtype or S3.shape[0] != batch or S3.shape[2] != rows:
+            raise ValueError(f"sketch must be ({batch}, k, {rows}) in {P3.dtype}, got {tuple(S3.shape)} {S3.dtype}")
+        k = S3.shape[1]
+        ws = _workspace.get(lib.dion_amd_orthonormalize_sketch_workspace_bytes(batch, rows, r, k), P.device)
+        with torch.cuda.device(P.device):
+            rc = lib.dion_amd_orthonormalize_sketch(P3.data_ptr(), S3.data_ptr(), out.data_ptr(), _lib.dtype_code(P.dtype),
+                                                    batch, rows, r, k, info.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                    _lib.stream_ptr(P.device))
+        _lib.check(rc, "dion_amd_orthonormalize_sketch")
+        out = out if P.ndim == 3 else out[0]
+        return (out, info) if return_info else out
     nbytes = lib.dion_amd_orthonormalize_workspace_bytes(batch, rows, r)
     ws = _workspace.get(nbytes, P.device)
     with torch.cuda.device(P.device):

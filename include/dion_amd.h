@@ -298,6 +298,31 @@ int dion_amd_dion_step_qr(void* const* X, const void* const* G, void* const* M, 
                           int power_iters, int qr_method,
                           int* info, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The reference's randomised Cholesky QR with the random sketch GIVEN by the caller (the async `orthogonalize`,
+ * reference dion/dion.py:1274-1308, whose sketch comes from generate_random_sketch_matrix, 1221-1263; the same
+ * sequence in dion/dion_reference.py:764-787):
+ *   SP = S P (in P's dtype);  R1 = R-factor of SP;  P1 = P R1^-1;  R2 = chol(P1^T P1);  Q = P1 R2^-1.
+ * S: `batch` contiguous sketches of k x rows in P's dtype (k >= r; the reference draws N(0, 1/k) entries with
+ * k = 128 ceil(1.25 r / 128)).  R1 is formed as the Cholesky factor of (SP)^T (SP) in fp64 -- the R-factor of a
+ * Householder QR of SP up to the signs of its rows -- and the solves and the second factorisation run in fp64 too.
+ * rows <= r: the reference factors such a P by Householder QR and draws no sketch (1283-1285); S is then ignored
+ * and the fp64 pass of dion_amd_orthonormalize_method runs.  The result is the thin-QR factor with a positive
+ * diagonal of R: the reference's up to column signs.  rows, r and k multiples of 8 (bf16) or 4 (f32). */
+size_t dion_amd_orthonormalize_sketch_workspace_bytes(int batch, int rows, int r, int k);
+int dion_amd_orthonormalize_sketch(const void* P, const void* S, void* out, int dtype, int batch, int rows, int r,
+                                   int k, int* info, void* workspace, size_t workspace_bytes, void* stream);
+
+/* dion_amd_dion_step with that orthonormaliser (qr_method "rcqr" of the per-matrix reference class with its own
+ * random sketches, reference dion/dion_reference.py:290-294, 764-775).  sketch: power_iters x batch contiguous
+ * sketches of sketch_k x max(m, n) in the momentum dtype (device memory), sketch_k a multiple of 8 and >= r. */
+size_t dion_amd_dion_sketch_workspace_bytes(int batch, int m, int n, int r, int m_dtype, int sketch_k);
+int dion_amd_dion_step_sketch(void* const* X, const void* const* G, void* const* M, void* const* Q,
+                              int batch, int m, int n, int r,
+                              int x_dtype, int g_dtype, int m_dtype, int q_dtype,
+                              float ef_alpha, float decay, float scaled_lr, float eps, int faithful,
+                              int power_iters, const void* sketch, int sketch_k,
+                              int* info, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Measurement hooks (no counterpart in the reference; used by the benchmark only)
  * ------------------------------------------------------------------------------------- */

@@ -35,14 +35,15 @@ def sketch_matrix(P, oversample, generator=None):
     return torch.empty((*P.shape[:-2], k, m), dtype=P.dtype).normal_(std=std, generator=generator)
 
 
-def orthogonalize(P, oversample=1.25, generator=None):
-    """reference dion/dion.py:1274-1308 (batched input, fp32 internally, result in P's dtype)."""
+def orthogonalize(P, oversample=1.25, generator=None, sketch=None):
+    """reference dion/dion.py:1274-1308 (batched input, fp32 internally, result in P's dtype).  `sketch`: the random
+    sketch S to use instead of drawing one (what the reference obtains from generate_random_sketch_matrix, 1287)."""
     assert P.ndim >= 3
     original_dtype = P.dtype
     if P.size(-2) <= P.size(-1):
         Pl, _ = torch.linalg.qr(P.to(dtype=torch.float32))
     else:
-        S = sketch_matrix(P, oversample, generator)
+        S = sketch if sketch is not None else sketch_matrix(P, oversample, generator)
         SP = S @ P
         _, R = torch.linalg.qr(SP.to(dtype=torch.float32), mode="r")
         Pl = torch.linalg.solve_triangular(R, P.to(dtype=torch.float32), upper=True, left=False)

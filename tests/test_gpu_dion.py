@@ -471,3 +471,37 @@ def test_orthonormalize_bf16_with_rows_off_the_8_grid(dev, rows, r, method):
         diff = rel_fro(_sign_align(Qd, Qh), Qh)
         print(f"{method} {rows}x{r} matrix {b}: ||QtQ-I|| = {orth:.2e}, vs Householder {diff:.2e}")
         assert orth <= 3e-2 and diff <= 5e-3
+
+
+@pytest.mark.parametrize("dtype,rows,r,batch", [(torch.float32, 768, 192, 2), (torch.float32, 520, 72, 3),
+                                                (torch.bfloat16, 3072, 192, 2), (torch.bfloat16, 1024, 64, 1)])
+def test_orthonormalize_with_an_injected_sketch(dev, dtype, rows, r, batch):
+    """The reference's randomised Cholesky QR with the sketch given by the caller (dion/dion.py:1287-1303,
+    `generate_random_sketch_matrix` 1221-1263) against `oracle.orthogonalize` on the SAME sketch, up to column signs;
+    the sketch only preconditions, so the sketch-free orthonormaliser must agree as well."""
+    from dion_amd.dion import generate_random_sketch_matrix
+    from dion_amd.newton_schulz import orthonormalize
+    from oracle import dion_step as O
+
+    torch.manual_seed(17)
+    P = (torch.randn(batch, rows, r, dtype=torch.float64) * torch.logspace(0, -2, r, dtype=torch.float64)).to(dtype)
+    Pd = P.to(dev)
+    S = generate_random_sketch_matrix(Pd, 1.25, generator=torch.Generator(device=dev).manual_seed(3))
+    k = 128 * -(-int(1.25 * r) // 128)
+    assert S.shape == (batch, k, rows) and S.dtype == dtype and S.is_cuda
+    assert abs(S.float().std().item() - (1.0 / k) ** 0.5) <= 0.05 * (1.0 / k) ** 0.5
+    Q, info = orthonormalize(Pd, sketch=S, return_info=True)
+    assert Q.dtype == dtype and (info == 0).all()
+    ref = O.orthogonalize(P, sketch=S.cpu())
+    plain = orthonormalize(Pd)
+    tol = 2e-5 if dtype == torch.float32 else 8e-3
+    for b in range(batch):
+        Qd = Q[b].double().cpu()
+        e_ref = rel_fro(_sign_align(Qd, ref[b]), ref[b])
+        e_plain = rel_fro(_sign_align(plain[b].double().cpu(), Qd), Qd)
+        orth = (Qd.T @ Qd - torch.eye(r, dtype=torch.float64)).norm().item()
+        print(f"sketched {dtype} {rows}x{r} matrix {b}: vs oracle {e_ref:.2e}, vs sketch-free {e_plain:.2e}, ||QtQ-I|| {orth:.2e}")
+        assert e_ref <= tol and e_plain <= tol
+        assert orth <= (ORTH_TOL if dtype == torch.float32 else 5e-2 * (r ** 0.5) / 8)
+    with pytest.raises(ValueError):
+        orthonormalize(Pd, sketch=S, qr_method="cqr")

@@ -270,3 +270,32 @@ def test_scalar_opts_bf16_rounding_points():
     adamw_update_foreach(X, [g0.bfloat16()], M, V, lr, b1, b2, wd, step, eps)
     assert torch.equal(M[0].float(), m1) and torch.equal(V[0].float(), v1)
     assert (X[0].float() != x1).float().mean() < 1e-3
+
+
+def test_sketched_orthogonalize_is_the_thin_qr_factor_whatever_the_sketch():
+    """`orthogonalize` with an injected sketch (reference dion/dion.py:1287-1303): in exact arithmetic the result is
+    the thin-QR Q factor of P for ANY full-rank sketch -- S only preconditions.  Pinned against Householder QR in
+    fp64 (a library routine) up to column signs, for two different sketches and for a deliberately poor one
+    (a dropped `R1^-1`, a transposed solve or a missing second factorisation all fail this)."""
+    from oracle import dion_step as O
+
+    torch.manual_seed(12)
+    rows, r = 384, 48
+    U, _ = torch.linalg.qr(torch.randn(rows, r, dtype=torch.float64))
+    V, _ = torch.linalg.qr(torch.randn(r, r, dtype=torch.float64))
+    P = ((U * torch.logspace(0, -3, r, dtype=torch.float64)) @ V.T).float().unsqueeze(0)      # cond 1e3
+    Qh, _ = torch.linalg.qr(P[0].double())
+    g = torch.Generator().manual_seed(1)
+    for trial in range(3):
+        S = O.sketch_matrix(P, 1.25, g)
+        assert S.shape == (1, 128, rows)
+        if trial == 2:
+            S = S * torch.logspace(0, -2, 128).view(1, -1, 1)      # a badly scaled sketch still spans enough
+        Q = O.orthogonalize(P, sketch=S)[0].double()
+        sgn = torch.sign((Q * Qh).sum(dim=0))
+        assert ((Q * sgn - Qh).norm() / Qh.norm()).item() <= 2e-4
+        assert (Q.T @ Q - torch.eye(r, dtype=torch.float64)).norm().item() <= 1e-4
+    # drawing from a generator and injecting the same draw are the same thing
+    a = O.orthogonalize(P, generator=torch.Generator().manual_seed(7))
+    b = O.orthogonalize(P, sketch=O.sketch_matrix(P, 1.25, torch.Generator().manual_seed(7)))
+    assert torch.equal(a, b)
