@@ -125,8 +125,12 @@ __device__ __forceinline__ void adamw_one(float& x, float gin, float& m, float& 
   x = xd - q;      // rounded by the store
 }
 
-template <bool ADAMW>
-__global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarArgs a) {
+// DT: dtype code shared by X, G, M and V when known at compile time (the common cases: all bf16, all fp32), so that the
+// per-element rounding and load / store forms carry no branches; -1: the codes of `ain` decide at run time.
+template <bool ADAMW, int DT>
+__global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarArgs ain) {
+  ScalarArgs a = ain;
+  if (DT >= 0) { a.x_dtype = DT; a.g_dtype = DT; a.m_dtype = DT; a.v_dtype = DT; }
   // which tensor this workgroup works on: bisection over the block ranges
   int lo = 0, hi = t.count - 1;
   while (lo < hi) {
@@ -143,6 +147,32 @@ __global__ __launch_bounds__(256) void scalar_opt_kernel(ScalarTable t, ScalarAr
   const long long begin = (long long)((int)blockIdx.x - t.first_block[b]) * BLOCK_ELEMS;
   const long long end = begin + BLOCK_ELEMS < n ? begin + BLOCK_ELEMS : n;
   const long long vend = end < nvec ? end : nvec;
+  if (vend - begin == BLOCK_ELEMS) {
+    // a whole block: the four vectors of a lane are requested before the first is used
+    constexpr int NV = BLOCK_ELEMS / (256 * 8);
+    float x[NV][8], g[NV][8], m[NV][8], v[NV][8];
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+      const long long i = begin + (q * 256 + threadIdx.x) * 8;
+      ld8(X, a.x_dtype, i, x[q]);
+      ld8(G, a.g_dtype, i, g[q]);
+      ld8(M, a.m_dtype, i, m[q]);
+      if (ADAMW) ld8(V, a.v_dtype, i, v[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < NV; ++q) {
+      const long long i = begin + (q * 256 + threadIdx.x) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (ADAMW) adamw_one(x[q][e], g[q][e], m[q][e], v[q][e], a);
+        else lion_one(x[q][e], g[q][e], m[q][e], a);
+      }
+      st8(X, a.x_dtype, i, x[q]);
+      st8(M, a.m_dtype, i, m[q]);
+      if (ADAMW) st8(V, a.v_dtype, i, v[q]);
+    }
+    return;
+  }
   for (long long i = begin + threadIdx.x * 8; i < vend; i += 256 * 8) {
     float x[8], g[8], m[8], v[8];
     ld8(X, a.x_dtype, i, x);
@@ -214,8 +244,20 @@ int run(bool adamw, void* const* X, const void* const* G, void* const* M, void* 
     t.count = k;
     for (int i = k; i <= MAX_TENSORS; ++i) t.first_block[i] = (int)blocks;
     DaProfScope prof(DA_PROF_SCALAR_OPT, bytes, s);
-    if (adamw) hipLaunchKernelGGL(scalar_opt_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, t, a);
-    else hipLaunchKernelGGL(scalar_opt_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, t, a);
+    const bool same = a.g_dtype == a.x_dtype && a.m_dtype == a.x_dtype && (!adamw || a.v_dtype == a.x_dtype);
+    const int dt = same ? a.x_dtype : -1;
+    const dim3 grid((unsigned)blocks), block(256);
+#define DA_SCALAR_LAUNCH(AD, DT) hipLaunchKernelGGL((scalar_opt_kernel<AD, DT>), grid, block, 0, s, t, a)
+    if (adamw) {
+      if (dt == DA_BF16) DA_SCALAR_LAUNCH(true, DA_BF16);
+      else if (dt == DA_F32) DA_SCALAR_LAUNCH(true, DA_F32);
+      else DA_SCALAR_LAUNCH(true, -1);
+    } else {
+      if (dt == DA_BF16) DA_SCALAR_LAUNCH(false, DA_BF16);
+      else if (dt == DA_F32) DA_SCALAR_LAUNCH(false, DA_F32);
+      else DA_SCALAR_LAUNCH(false, -1);
+    }
+#undef DA_SCALAR_LAUNCH
     const int rc = da_launch_status();
     if (rc) return rc;
   }
