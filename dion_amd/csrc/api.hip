@@ -39,7 +39,8 @@ struct NsLayout {
     a_bytes = (size_t)mw * lda * esz;
     part_bytes = align_up((size_t)tiles * sizeof(float) + sizeof(float), 256);
     // control words of the persistent Newton-Schulz kernel: cb * flow_bytes >= da_ns_flow_ctl_bytes(cb) for cb >= 1
-    flow_bytes = DA_FLOW_CTR_STRIDE * sizeof(int) + 256;
+    // (+ 16: one slot of the table of weight pointers that the last product's epilogue updates)
+    flow_bytes = DA_FLOW_CTR_STRIDE * sizeof(int) + 256 + 16;
     per_matrix = 2 * x_bytes + 2 * a_bytes + part_bytes + flow_bytes;
   }
   int chunk(int batch, size_t ws_bytes) const {
@@ -61,6 +62,7 @@ struct NsBuffers {
   char *x0 = nullptr, *x1 = nullptr, *a = nullptr, *b = nullptr;
   float *partials = nullptr, *divisor = nullptr;
   int* flow = nullptr;
+  void** xtab = nullptr;   // per-matrix weight pointers (Muon: the last product updates the weights itself)
   NsBuffers() {}
   NsBuffers(const NsLayout& L, void* ws, int cb) {
     char* p = static_cast<char*>(ws);
@@ -71,6 +73,7 @@ struct NsBuffers {
     partials = reinterpret_cast<float*>(p); p += L.part_bytes * cb;
     divisor = partials + (size_t)L.tiles * cb;
     flow = reinterpret_cast<int*>(p);
+    xtab = reinterpret_cast<void**>(p + (DA_FLOW_CTR_STRIDE * sizeof(int) + 256) * (size_t)cb);
   }
 };
 
@@ -106,16 +109,25 @@ struct NsSet {
   NsLayout L;
   NsBuffers W;
   int cb = 0;
+  // Muon: the last X' = aX + BX does not store its result but applies it to the weights W.xtab[b] (x_dtype, rows x
+  // cols as the optimizer holds them: transposed with respect to the wide working matrix when tall)
+  int update = 0, x_dtype = 0, tall = 0, x_ld = 0;
+  float decay = 1.f, step = 1.f;
 };
 
 // steps x { A = X X^T ; B = b A + c A A ; X' = a X + B X } on up to DA_MAX_GROUPS sets of wide
 // matrices at once (each of the three products is one grouped launch over all sets).
 // Returns in result[i] which of x0 / x1 of set i holds the final iterate, and in *poison (if asked for) a device word
-// that is non-zero when the iterates are invalid (null: there is no such word).
+// that is non-zero when the iterates are invalid (null: there is no such word).  With `updated` given and every set
+// carrying its weight table, the last product applies the weight update itself where its launch allows that
+// (*updated = true: result[] then holds nothing of use and the caller skips its own update pass).
 int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int steps, int faithful, hipStream_t s,
-               char** result, const int** poison = nullptr) {
+               char** result, const int** poison = nullptr, bool* updated = nullptr) {
   if (nsets < 1 || nsets > DA_MAX_GROUPS) return DA_ERR_ARG;
   if (poison) *poison = nullptr;
+  if (updated) *updated = false;
+  bool want_update = updated != nullptr && dtype == DA_BF16 && steps >= 1;
+  for (int i = 0; i < nsets; ++i) want_update = want_update && sets[i].update;
   if (dtype == DA_BF16 && steps >= 1) {
     // many small matrices: all iterations of all sets as one persistent launch (ns_flow.hip); the sets are dealt to
     // its queues most expensive first
@@ -128,10 +140,17 @@ int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int
     for (int k = 0; k < nsets; ++k) {
       const NsLayout& L = sets[order[k]].L;
       const NsBuffers& W = sets[order[k]].W;
+      const NsSet& S = sets[order[k]];
       fg[k] = DaNsFlowGroup{W.x0, W.x1, W.a, W.b, (long long)(L.x_bytes / L.esz), (long long)(L.a_bytes / L.esz),
-                            L.mw, L.nw, L.ldx, L.lda, sets[order[k]].cb, W.flow};
+                            L.mw, L.nw, L.ldx, L.lda, S.cb, W.flow,
+                            want_update ? W.xtab : nullptr, S.x_dtype, S.x_ld, S.tall, S.decay, S.step};
     }
-    if (da_ns_flow_applicable(fg, nsets, steps)) {
+    // (the persistent kernel updates bf16 weights only: others get the separate pass)
+    bool flow_update = want_update;
+    for (int i = 0; i < nsets; ++i) flow_update = flow_update && sets[i].x_dtype == DA_BF16;
+    if (!flow_update)
+      for (int k = 0; k < nsets; ++k) fg[k].upd_tab = nullptr;
+    if (da_ns_flow_applicable(fg, nsets, steps, faithful)) {
       double flops = 0.0;
       for (int i = 0; i < nsets; ++i) {
         const NsLayout& L = sets[i].L;
@@ -142,6 +161,7 @@ int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int
       if (rc) return rc;
       for (int i = 0; i < nsets; ++i) result[i] = (steps & 1) ? sets[i].W.x1 : sets[i].W.x0;
       if (poison) *poison = da_ns_flow_status_word(fg);
+      if (flow_update) *updated = true;
       return DA_OK;
     }
   }
@@ -191,6 +211,13 @@ int ns_iterate(const NsSet* sets, int nsets, int dtype, const float* coeffs, int
       g[i].a_kstrided = 0; g[i].b_kstrided = 1; g[i].symmetric = 0;
       g[i].epilogue = DA_EPI_AXPBY; g[i].s0 = a; g[i].s1 = 1.f;
     }
+    if (want_update && it + 1 == steps && da_gemm_bf16_all_interior(g, nsets)) {
+      for (int i = 0; i < nsets; ++i) {
+        g[i].upd_tab = sets[i].W.xtab; g[i].upd_dtype = sets[i].x_dtype; g[i].upd_ld = sets[i].x_ld;
+        g[i].upd_transposed = sets[i].tall; g[i].upd_decay = sets[i].decay; g[i].upd_step = sets[i].step;
+      }
+      *updated = true;
+    }
     rc = gemm_group(g, nsets, dtype, s, DA_PROF_NS_AXPY);
     if (rc) return rc;
     for (int i = 0; i < nsets; ++i) { char* t = x[i]; x[i] = y[i]; y[i] = t; }
@@ -204,6 +231,27 @@ int ns_iterate(const NsLayout& L, const NsBuffers& W, int cb, int dtype, const f
   NsSet one;
   one.L = L; one.W = W; one.cb = cb;
   return ns_iterate(&one, 1, dtype, coeffs, steps, faithful, s, result, poison);
+}
+
+// The weights of `c` matrices starting at X[0] as a device table at `dst`, and the set's update parameters.
+int ns_set_update(NsSet& set, void* const* X, int first, int c, int m, int n, int x_dtype, float decay, float step,
+                  hipStream_t s) {
+  DaPtrTable t{};
+  for (int j = 0; j < c; ++j) t.p[j] = X[j];
+  set.update = 1; set.x_dtype = x_dtype; set.tall = m > n ? 1 : 0; set.x_ld = n; set.decay = decay; set.step = step;
+  return da_upload_ptrs(t, set.W.xtab + first, c, s);
+}
+
+// After a persistent launch that updated the weights itself: NaN in all of them if the launch gave up.
+int ns_poison_weights(void* const* X, int batch, int m, int n, int x_dtype, const int* poison, hipStream_t s) {
+  for (int j0 = 0; j0 < batch; j0 += DA_MAX_PTRS) {
+    const int c = batch - j0 < DA_MAX_PTRS ? batch - j0 : DA_MAX_PTRS;
+    DaPtrTable t{};
+    for (int j = 0; j < c; ++j) t.p[j] = X[j0 + j];
+    const int rc = da_poison_if(t, c, (long long)m * n, x_dtype, poison, s);
+    if (rc) return rc;
+  }
+  return DA_OK;
 }
 
 int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
@@ -475,8 +523,20 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M, int
     if (rc) return rc;
     char* res = nullptr;
     const int* poison = nullptr;
-    rc = ns_iterate(L, W, cb, DA_BF16, coeffs, steps, faithful, s, &res, &poison);
+    bool updated = false;
+    NsSet one;
+    one.L = L; one.W = W; one.cb = cb;
+    rc = ns_set_update(one, X + b0, 0, cb, m, n, x_dtype, decay, adjusted_lr, s);
     if (rc) return rc;
+    rc = ns_iterate(&one, 1, DA_BF16, coeffs, steps, faithful, s, &res, &poison, &updated);
+    if (rc) return rc;
+    if (updated) {
+      if (poison) {
+        rc = ns_poison_weights(X + b0, cb, m, n, x_dtype, poison, s);
+        if (rc) return rc;
+      }
+      continue;
+    }
     DaUnstage us{};
     us.poison = poison;
     for (int i = 0; i < cb; ++i) us.x.p[i] = X[b0 + i];
@@ -631,9 +691,23 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
     }
     char* res[DA_MAX_GROUPS];
     const int* poison = nullptr;
-    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res, &poison);
-    if (rc) return rc;
+    bool updated = false;
     for (int i = 0; i < nr; ++i) {
+      const dion_amd_muon_bucket& k = buckets[r0 + i];
+      for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {
+        const int c = k.batch - j0 < DA_MAX_PTRS ? k.batch - j0 : DA_MAX_PTRS;
+        const int rc = ns_set_update(sets[i], k.X + j0, j0, c, k.m, k.n, x_dtype, k.decay, k.adjusted_lr, s);
+        if (rc) return rc;
+      }
+    }
+    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res, &poison, &updated);
+    if (rc) return rc;
+    for (int i = 0; i < nr && updated && poison; ++i) {
+      const dion_amd_muon_bucket& k = buckets[r0 + i];
+      rc = ns_poison_weights(k.X, k.batch, k.m, k.n, x_dtype, poison, s);
+      if (rc) return rc;
+    }
+    for (int i = 0; i < nr && !updated; ++i) {
       const dion_amd_muon_bucket& k = buckets[r0 + i];
       const NsLayout& L = sets[i].L;
       for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {

@@ -131,6 +131,13 @@ struct GemmDesc {
   // matrices s * batch ... s * batch + batch - 1 of C, which therefore holds k_slices * batch matrices sC apart,
   // and the caller adds them in a fixed order.  Plain fp32 store only (no E, no tables, no second output).
   int k_slices, k_slice;
+  // bf16 kernel, optional (bf16 result with an epilogue operand, not symmetric, interior tiles).  upd_tab != null:
+  // the result C is not stored; it is the update of the matrix upd_tab[b] (upd_dtype, row pitch upd_ld), in place:
+  //   W <- r_W( r_W(W * upd_decay) - r_bf16(C * upd_step) )
+  // element (i, j) of C updating W[i][j], or W[j][i] when upd_transposed (W is stored N x M).
+  void* const* upd_tab;
+  int upd_dtype, upd_ld, upd_transposed;
+  float upd_decay, upd_step;
 };
 
 // Epilogues.  With `faithful` set the rounding points of the reference's separate
@@ -151,3 +158,5 @@ int da_gemm_bf16_grouped(const GemmDesc* d, int n, hipStream_t stream);
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream);
 // Tile edge (128 / 256) the bf16 launcher picks for one product, + 1 if its K loop is the direct-to-LDS one.
 int da_gemm_bf16_plan(const GemmDesc& d);
+// Whether da_gemm_bf16_grouped would run every tile of these products in its interior (unchecked) form.
+bool da_gemm_bf16_all_interior(const GemmDesc* d, int n);

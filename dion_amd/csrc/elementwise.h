@@ -48,3 +48,7 @@ int da_norm_finish(const float* partials, int tiles, int batch, float eps, int b
                    hipStream_t s);
 int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor, hipStream_t s);
 int da_unstage(const DaUnstage& d, hipStream_t s);
+// dst[i] = t.p[i] for i < n <= DA_MAX_PTRS: a table of per-matrix pointers in device memory
+int da_upload_ptrs(const DaPtrTable& t, void** dst, int n, hipStream_t s);
+// If *flag != 0 when the kernel runs, every element of the n matrices (numel contiguous elements each) becomes NaN.
+int da_poison_if(const DaPtrTable& t, int n, long long numel, int dtype, const int* flag, hipStream_t s);

@@ -500,6 +500,34 @@ int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const
   return da_launch_status();
 }
 
+namespace {
+__global__ __launch_bounds__(64) void upload_ptrs_kernel(DaPtrTable t, void** dst, int n) {
+  if ((int)threadIdx.x < n) dst[threadIdx.x] = t.p[threadIdx.x];
+}
+// every element of the matrices becomes NaN if *flag != 0 (the launch that produced them gave up)
+__global__ __launch_bounds__(256) void poison_kernel(DaPtrTable t, long long numel, int f32, const int* flag) {
+  if (*flag == 0) return;
+  const float nan = __builtin_nanf("");
+  void* p = t.p[blockIdx.y];
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < numel; i += (long long)gridDim.x * 256) {
+    if (f32) static_cast<float*>(p)[i] = nan;
+    else static_cast<bf16_t*>(p)[i] = f2bf(nan);
+  }
+}
+}  // namespace
+
+int da_upload_ptrs(const DaPtrTable& t, void** dst, int n, hipStream_t s) {
+  if (!dst || n < 1 || n > DA_MAX_PTRS) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL(upload_ptrs_kernel, dim3(1), dim3(64), 0, s, t, dst, n);
+  return da_launch_status();
+}
+
+int da_poison_if(const DaPtrTable& t, int n, long long numel, int dtype, const int* flag, hipStream_t s) {
+  if (!flag || n < 1 || n > DA_MAX_PTRS || numel < 1) return DA_ERR_ARG;
+  hipLaunchKernelGGL(poison_kernel, dim3(64, (unsigned)n), dim3(256), 0, s, t, numel, dtype == DA_F32 ? 1 : 0, flag);
+  return da_launch_status();
+}
+
 int da_unstage(const DaUnstage& d, hipStream_t s) {
   if (d.batch <= 0 || d.batch > DA_MAX_PTRS) return DA_ERR_LIMIT;
   if ((d.rows | d.cols | d.ld) & 7) return DA_ERR_ALIGN;

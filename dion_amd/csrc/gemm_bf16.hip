@@ -234,6 +234,8 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   if (!full && !edge)   // the bounds-checked K loop walks A with a pointer: no wrap-around there
     for (int g = 0; g < n; ++g)
       if (d[g].a_kwrap) return DA_ERR_ARG;
+  for (int g = 0; g < n; ++g)   // the weight-update epilogue exists for interior tiles of plain bf16 AXPBY products
+    if (d[g].upd_tab && (!full || SYM || d[g].c_dtype != DA_BF16 || d[g].epilogue != DA_EPI_AXPBY)) return DA_ERR_ARG;
   hipLaunchKernelGGL(full ? kfull : (edge ? kedge : kgen), dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
   return da_launch_status();
 }
@@ -348,6 +350,13 @@ int da_gemm_bf16_plan(const GemmDesc& d) {
 }
 
 int da_gemm_bf16(const GemmDesc& d, hipStream_t stream) { return da_gemm_bf16_grouped(&d, 1, stream); }
+
+// Whether the grouped launch of these products runs the interior (direct-to-LDS, unchecked) form for every tile:
+// the form the weight-update epilogue (GemmDesc::upd_tab) exists in.
+bool da_gemm_bf16_all_interior(const GemmDesc* d, int n) {
+  if (!d || n <= 0 || n > DA_MAX_GROUPS) return false;
+  return all_interior(d, n, choose_tile(d, n));
+}
 
 // ---- measurement hook: time stamps of the tiles of the bf16 GEMM launches (see include/dion_amd.h)
 extern "C" int dion_amd_tile_trace_enable(int on) {

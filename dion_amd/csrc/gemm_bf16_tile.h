@@ -84,7 +84,41 @@ struct StageAddr {
 // stages through its own LDS region, so only wavefront-level ordering is needed inside.
 // Output dtype, epilogue form and rounding mode are compile-time here: evaluated per element at
 // run time they cost more than the MFMAs of a short-K product.
-template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL, bool S1_ONE>
+// The weight update of the reference's post-orthogonalisation pass on 8 consecutive elements of the weights at `Wp`
+// (dion/muon.py:569-573): W <- r_W(r_W(W * decay) - r_bf16(U * step)), U = the eight bf16 results in `pk`; the old
+// weights come in x0 (bf16: all eight) resp. x0, x1 (fp32), requested a band earlier.
+__device__ __forceinline__ void update_weights8(char* Wp, bool w_f32, u32x4_t x0, u32x4_t x1, u32x4_t pk, float decay,
+                                                float step) {
+  if (!w_f32) {
+    u32x4_t o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const unsigned x = x0[q], u = pk[q];
+      const unsigned xd = cvt_pk_bf16(lo_f(x) * decay, hi_f(x) * decay);
+      const unsigned t = cvt_pk_bf16(lo_f(u) * step, hi_f(u) * step);
+      o[q] = cvt_pk_bf16(lo_f(xd) - lo_f(t), hi_f(xd) - hi_f(t));
+    }
+    stg16(Wp, o);
+  } else {
+    u32x4_t o0, o1;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const unsigned u = pk[q];
+      const unsigned t = cvt_pk_bf16(lo_f(u) * step, hi_f(u) * step);
+      const unsigned xa = q < 2 ? x0[2 * q] : x1[2 * q - 4], xb = q < 2 ? x0[2 * q + 1] : x1[2 * q - 3];
+      const float ra = __builtin_bit_cast(float, xa) * decay - lo_f(t);
+      const float rb = __builtin_bit_cast(float, xb) * decay - hi_f(t);
+      if (q < 2) { o0[2 * q] = __builtin_bit_cast(unsigned, ra); o0[2 * q + 1] = __builtin_bit_cast(unsigned, rb); }
+      else { o1[2 * q - 4] = __builtin_bit_cast(unsigned, ra); o1[2 * q - 3] = __builtin_bit_cast(unsigned, rb); }
+    }
+    stg16(Wp, o0);
+    stg16(Wp + 16, o1);
+  }
+}
+
+// UPD: 0 the result is stored in C; 1 / 2 it is not stored but updates the weights d.upd_tab[b] in place (2: those are
+// stored transposed), see GemmDesc.
+template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL, bool S1_ONE, int UPD = 0, bool WF32 = false>
 __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
                                               bool mirror, int m0, int n0, int wave, int lane, int wm, int wn) {
   constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
@@ -108,10 +142,37 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
                                      : static_cast<const char*>(d.E) + (long long)b * d.sE * CSZ;
   const int lr = lane / CPR, c8 = (lane % CPR) * 8;
   const bool col_ok = FULL || wn0 + c8 < dN;
+  char* const Wbase = UPD ? static_cast<char*>(d.upd_tab[b]) : nullptr;
+  constexpr bool w_f32 = WF32;   // (a compile-time variant: the prefetch buffers differ in size)
+  constexpr int wsz = w_f32 ? 4 : 2;
+  const long long ldw = d.upd_ld;
+  const float w_decay = d.upd_decay, w_step = d.upd_step;
   // E is requested up to three bands ahead (registers that the K loop's fragments no longer need), so that a
   // tile's epilogue pays one memory latency and not one per band; an fp32 E (twice the registers) one band ahead.
-  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (C::TMI < 3 ? C::TMI : 3);
+  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (UPD ? 2 : (C::TMI < 3 ? C::TMI : 3));
   u32x4_t ev[DEPTH][NPASS][NV];
+  // the weights a band updates are requested when the band starts, ahead of its staging through LDS and of the
+  // arithmetic on E (two vectors per 8 elements when they are fp32)
+  constexpr int NWP = UPD == 2 ? (W / 64) * 4 : NPASS;
+  constexpr int NWV = WF32 ? 2 : 1;
+  u32x4_t wv[NWP][NWV];
+  auto weight_ptr = [&](int band, int pass) -> char* {
+    if (UPD == 2) {
+      const int n = wn0 + (pass >> 2) * 64 + lane, m = wm0 + band * 32 + (pass & 3) * 8;
+      return Wbase + ((long long)n * ldw + m) * wsz;
+    }
+    const int m = wm0 + band * 32 + pass * RPP + lr;
+    return Wbase + ((long long)m * ldw + wn0 + c8) * wsz;
+  };
+  auto load_w = [&](int band, u32x4_t (&dst)[NWP][NWV]) {
+#pragma unroll
+    for (int pass = 0; pass < NWP; ++pass) {
+      const char* p = weight_ptr(band, pass);
+#pragma unroll
+      for (int h = 0; h < NWV; ++h) dst[pass][h] = ldg16(p + 16 * h);
+    }
+  };
+
   auto load_e = [&](int band, u32x4_t (&dst)[NPASS][NV]) {
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
@@ -132,6 +193,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
   }
 #pragma unroll
   for (int i = 0; i < C::TMI; ++i) {
+    if (UPD) load_w(i, wv);
     {
       float* row = stg + (lane & 31) * PITCH + (lane >> 5) * 4;
 #pragma unroll
@@ -151,6 +213,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
         for (int h = 0; h < NV; ++h) ec[pass][h] = ev[i % DEPTH][pass][h];
       if (i + DEPTH < C::TMI) load_e(i + DEPTH, ev[i % DEPTH]);
     }
+
 #pragma unroll
     for (int pass = 0; pass < NPASS; ++pass) {
       const int r = pass * RPP + lr;
@@ -188,7 +251,12 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
               v[2 * q + 1] = hi_f(o);
             }
           }
-          stg16(Cp, pk);
+          if (UPD == 0) stg16(Cp, pk);
+          if (UPD == 1) update_weights8(weight_ptr(i, pass), w_f32, wv[pass][0], wv[pass][NWV - 1], pk, w_decay, w_step);
+          if (UPD == 2) {   // the final values stay in the staging area for the transposed pass below
+            *reinterpret_cast<float4*>(sp) = make_float4(lo_f(pk[0]), hi_f(pk[0]), lo_f(pk[1]), hi_f(pk[1]));
+            *reinterpret_cast<float4*>(sp + 4) = make_float4(lo_f(pk[2]), hi_f(pk[2]), lo_f(pk[3]), hi_f(pk[3]));
+          }
           if (!HAS_E && !FAITHFUL && !SYM && c2) {
             // what the stored bf16 leaves of s1 * acc, as a second bf16 matrix
             u32x4_t lo;
@@ -200,6 +268,22 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
         if (SYM && mirror) {  // keep the final values for the transposed store
           *reinterpret_cast<float4*>(sp) = make_float4(v[0], v[1], v[2], v[3]);
           *reinterpret_cast<float4*>(sp + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+      }
+    }
+    if (UPD == 2) {
+      wave_sync_lds();
+      // the weights are stored transposed: row n of W holds 32 consecutive m of this band
+#pragma unroll
+      for (int pass = 0; pass < (W / 64) * 4; ++pass) {
+        const int nl = (pass >> 2) * 64 + lane;
+        const int mg = (pass & 3) * 8;
+        const int n = wn0 + nl, m = band_m + mg;
+        if (FULL || (n < dN && m < dM)) {
+          u32x4_t pk;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) pk[q] = cvt_pk_bf16(stg[(mg + 2 * q) * PITCH + nl], stg[(mg + 2 * q + 1) * PITCH + nl]);
+          update_weights8(weight_ptr(i, pass), w_f32, wv[pass][0], wv[pass][NWV - 1], pk, w_decay, w_step);
         }
       }
     }
@@ -244,6 +328,20 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
   const bool one = d.s1 == 1.f;   // rounding-faithful bf16 output: the exact multiplication by 1 is left out
 #define DA_EPI(CF, HE, FA, S1) \
   epilogue_impl<C, SYM, FULL, CF, HE, FA, S1>(acc, d, lds, b, mirror, m0, n0, wave, lane, wm, wn)
+#define DA_EPI_UPD(FA, S1, U, WF) \
+  epilogue_impl<C, false, FULL, false, true, FA, S1, U, WF>(acc, d, lds, b, false, m0, n0, wave, lane, wm, wn)
+#define DA_EPI_UPD_FA(U, WF)                                                              \
+  do {                                                                                    \
+    if (fa) { if (one) DA_EPI_UPD(true, true, U, WF); else DA_EPI_UPD(true, false, U, WF); } \
+    else DA_EPI_UPD(false, false, U, WF);                                                 \
+  } while (0)
+  if (!SYM && FULL && !cf32 && has_e && d.upd_tab) {
+    // (the launcher only sets upd_tab where these conditions hold)
+    const bool wf = d.upd_dtype == DA_F32;
+    if (d.upd_transposed) { if (wf) DA_EPI_UPD_FA(2, true); else DA_EPI_UPD_FA(2, false); }
+    else                  { if (wf) DA_EPI_UPD_FA(1, true); else DA_EPI_UPD_FA(1, false); }
+    return;
+  }
   if (!cf32) {
     if (has_e) {
       if (fa) { if (one) DA_EPI(false, true, true, true); else DA_EPI(false, true, true, false); }
@@ -257,6 +355,8 @@ __device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const 
     else       { if (fa) DA_EPI(true, false, true, false); else DA_EPI(true, false, false, false); }
   }
 #undef DA_EPI
+#undef DA_EPI_UPD
+#undef DA_EPI_UPD_FA
 }
 
 

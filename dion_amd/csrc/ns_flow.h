@@ -15,12 +15,16 @@ struct DaNsFlowGroup {
   long long sx, sa;
   int mw, nw, ldx, lda, cnt;
   int* ctl;
+  // upd_tab != null: the last iteration's X' is not stored but updates the bf16 weights upd_tab[b] in place (see GemmDesc)
+  void* const* upd_tab;
+  int upd_dtype, upd_ld, upd_transposed;
+  float upd_decay, upd_step;
 };
 
 size_t da_ns_flow_ctl_bytes(int cnt);
 // Whether the persistent kernel runs these groups (shapes on the 256 grid and, unless forced, a workload it is
 // faster on: many small matrices that deal evenly to the eight queues).
-bool da_ns_flow_applicable(const DaNsFlowGroup* g, int n, int steps);
+bool da_ns_flow_applicable(const DaNsFlowGroup* g, int n, int steps, int faithful);
 int da_ns_flow(const DaNsFlowGroup* g, int n, const float* coeffs, int steps, int faithful, hipStream_t s);
 // Device word that is non-zero after a launch that gave up (a wait beyond the spin limit): results are then invalid.
 const int* da_ns_flow_status_word(const DaNsFlowGroup* g);

@@ -43,6 +43,9 @@ struct FlowGroupDev {
   char *x0, *x1, *a, *b;
   long long sx, sa;          // elements between consecutive matrices
   int* counters;             // [cnt][DA_FLOW_CTR_STRIDE]
+  void* const* upd_tab;      // weights updated by the last iteration's X' (or null: X' is stored)
+  float upd_decay, upd_step;
+  int upd_dtype, upd_ld, upd_transposed;
   int mw, nw, ldx, lda;
   int cnt, first;            // matrices; index of the first one in the dealing order
   int tm, tn;                // tiles per side
@@ -263,6 +266,10 @@ __global__ __launch_bounds__(Big::NT) void ns_flow_kernel(FlowArgs a) {
         d.lda = G.lda; d.ldb = G.ldx; d.ldc = G.ldx; d.lde = G.ldx;
         d.M = G.mw; d.N = G.nw; d.K = G.mw;
         d.b_kstrided = 1; d.epilogue = DA_EPI_AXPBY;
+        if (G.upd_tab != nullptr && w.it + 1 == a.steps) {
+          d.upd_tab = G.upd_tab + w.b; d.upd_dtype = G.upd_dtype; d.upd_ld = G.upd_ld;
+          d.upd_transposed = G.upd_transposed; d.upd_decay = G.upd_decay; d.upd_step = G.upd_step;
+        }
       }
       // epilogue scalars, C = s0 E + s1 acc.  (As selects on purpose: assigned inside the three branches above, hipcc 7.2
       // passed the polynomial's b as s0 of X' = aX + BX; the bit-level tests against the product launches cover it.)
@@ -273,8 +280,18 @@ __global__ __launch_bounds__(Big::NT) void ns_flow_kernel(FlowArgs a) {
       if (trace) ts[2] = now_ticks();
       // the next ticket is requested before the epilogue, which hides its latency
       if (tid == 0) next = take_ticket(a.tickets + q, xcd, total, true);
-      if (w.p == 2) epilogue<Big, false, true>(acc, d, lds, 0, ti, tj, m0, n0, wave, lane, wm, wn);
-      else epilogue<Big, true, true>(acc, d, lds, 0, ti, tj, m0, n0, wave, lane, wm, wn);
+      // the epilogue forms this kernel needs, and no others (every form compiled in costs registers here): bf16
+      // results, rounding-faithful; X X^T stores acc, the polynomial and X' combine with E, the last X' may update
+      // bf16 weights instead of being stored
+      const bool mirror = ti != tj;
+#define DA_FLOW_EPI(SYMM, HE, ONE, U) \
+  epilogue_impl<Big, SYMM, true, false, HE, true, ONE, U, false>(acc, d, lds, 0, SYMM && mirror, m0, n0, wave, lane, wm, wn)
+      if (w.p == 0) DA_FLOW_EPI(true, false, true, 0);
+      else if (w.p == 1) DA_FLOW_EPI(true, true, false, 0);
+      else if (d.upd_tab == nullptr) DA_FLOW_EPI(false, true, true, 0);
+      else if (d.upd_transposed) DA_FLOW_EPI(false, true, true, 2);
+      else DA_FLOW_EPI(false, true, true, 1);
+#undef DA_FLOW_EPI
       // ---- to be published under the next tile
       pend = ctr + phase;
       if (tid == 0) {
@@ -352,7 +369,8 @@ void da_ns_flow_set_spin_limit(long long ticks) { g_flow_spin.store(ticks, std::
 
 size_t da_ns_flow_ctl_bytes(int cnt) { return (size_t)cnt * DA_FLOW_CTR_STRIDE * sizeof(int) + 256; }
 
-bool da_ns_flow_applicable(const DaNsFlowGroup* g, int n, int steps) {
+bool da_ns_flow_applicable(const DaNsFlowGroup* g, int n, int steps, int faithful) {
+  if (!faithful) return false;   // (the kernel carries the rounding-faithful epilogues only)
   int mode = g_flow_mode.load(std::memory_order_relaxed);
   if (mode < 0) {
     static const int env = [] { const char* e = getenv("DION_AMD_NS_FLOW"); return e ? atoi(e) : -1; }();
@@ -401,18 +419,21 @@ bool da_ns_flow_applicable(const DaNsFlowGroup* g, int n, int steps) {
 }
 
 int da_ns_flow(const DaNsFlowGroup* g, int n, const float* coeffs, int steps, int faithful, hipStream_t s) {
-  if (!g || !coeffs || n < 1 || n > DA_MAX_GROUPS || steps < 1 || steps > DA_FLOW_MAX_STEPS) return DA_ERR_ARG;
+  if (!g || !coeffs || n < 1 || n > DA_MAX_GROUPS || steps < 1 || steps > DA_FLOW_MAX_STEPS || !faithful) return DA_ERR_ARG;
   FlowArgs a{};
   ResetArgs r{};
   int first = 0;
   for (int i = 0; i < n; ++i) {
     const DaNsFlowGroup& G = g[i];
     if (!G.x0 || !G.x1 || !G.a || !G.b || !G.ctl || G.cnt < 1) return DA_ERR_ARG;
+    if (G.upd_tab && G.upd_dtype != DA_BF16) return DA_ERR_DTYPE;   // (weights of another dtype: the caller's own pass)
     if (G.mw % BT || G.nw % BT || G.mw > G.nw || (G.ldx & 7) || (G.lda & 7) || (G.sx & 7) || (G.sa & 7)) return DA_ERR_ALIGN;
     FlowGroupDev& D = a.g[i];
     D.x0 = G.x0; D.x1 = G.x1; D.a = G.a; D.b = G.b;
     D.sx = G.sx; D.sa = G.sa;
     D.counters = G.ctl;
+    D.upd_tab = G.upd_tab; D.upd_dtype = G.upd_dtype; D.upd_ld = G.upd_ld; D.upd_transposed = G.upd_transposed;
+    D.upd_decay = G.upd_decay; D.upd_step = G.upd_step;
     D.mw = G.mw; D.nw = G.nw; D.ldx = G.ldx; D.lda = G.lda;
     D.cnt = G.cnt; D.first = first;
     D.tm = G.mw / BT; D.tn = G.nw / BT;
