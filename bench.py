@@ -38,11 +38,11 @@ LLAMA8B_LAYER = [(4096, 4096)] * 2 + [(1024, 4096)] * 2 + [(14336, 4096)] * 2 + 
 LLAMA70B_MLP_LAYER = [(28672, 8192)] * 2 + [(8192, 28672)]
 
 WORKLOADS = {
-    "muon_gpt_small": dict(kind="muon", shapes=GPT_SMALL_LAYER * 12, seed=1,
+    "muon_gpt_small": dict(kind="muon", shapes=GPT_SMALL_LAYER * 12, seed=1, graph=True,
                            desc="Full Muon step, GPT-small (12 layers, d=768): 72 bf16 matrices"),
-    "dion_gpt_small_r025": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=0.25,
+    "dion_gpt_small_r025": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=0.25, graph=True,
                                 desc="Full Dion step, GPT-small matrices, rank fraction 0.25 (r=192), bf16 M, fp32 Q"),
-    "dion_gpt_small_r1": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=1.0,
+    "dion_gpt_small_r1": dict(kind="dion", shapes=GPT_SMALL_LAYER * 12, seed=3, rank_fraction=1.0, graph=True,
                               desc="Full Dion step, GPT-small matrices, rank fraction 1.0 (r=768), bf16 M, fp32 Q"),
     "muon_llama8b_layer": dict(kind="muon", shapes=LLAMA8B_LAYER, seed=4,
                                desc="Muon step, one Llama-3-8B layer: 7 bf16 matrices incl. 4096x14336"),
@@ -126,6 +126,33 @@ def measure(wl, dev, steps, warmup):
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
 
+    # The same step captured once in a HIP graph and replayed (no per-launch host work): what a training loop that
+    # captures its optimizer step gets.  Only for the workloads whose step is short enough to be bound by the host.
+    graph_ms = None
+    if wl.get("graph"):
+        try:
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    opt.step()
+            torch.cuda.synchronize()
+            for _ in range(warmup):
+                graph.replay()
+            torch.cuda.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            tg = time.perf_counter()
+            g0.record()
+            for _ in range(steps):
+                graph.replay()
+            g1.record()
+            torch.cuda.synchronize()
+            graph_ms = max((time.perf_counter() - tg) * 1e3 / steps, g0.elapsed_time(g1) / steps)
+            del graph
+        except Exception as exc:   # the figure is an extra: the run goes on without it
+            graph_ms = f"capture failed: {exc}"
+
     # Second pass for the per-launch figures.  Dion runs its buckets on up to three streams; for this
     # pass they run one at a time so that a launch's duration is that of the kernel alone.
     if hasattr(opt, "_max_concurrent_tasks"):
@@ -150,7 +177,7 @@ def measure(wl, dev, steps, warmup):
             k.update(gbps=round(rate / 1e9, 1), frac_hbm=round(rate / PEAK_HBM_BPS, 4))
         kernels[name] = k
     res = dict(ms_per_step=max(wall_ms, ev_ms), wall_ms=wall_ms, event_ms=ev_ms, kernels=kernels, prof=prof,
-               optimizer=desc, steps=steps)
+               optimizer=desc, steps=steps, graph_ms=graph_ms)
     del opt, params
     torch.cuda.empty_cache()
     return res
@@ -160,6 +187,9 @@ def summarize(name, wl, res):
     shapes = wl["shapes"]
     out = dict(workload=name, ms_per_step=round(res["ms_per_step"], 4), steps=res["steps"],
                orthogonalisations_per_s=round(len(shapes) / (res["ms_per_step"] * 1e-3), 1))
+    if res.get("graph_ms") is not None:
+        g = res["graph_ms"]
+        out["hip_graph_replay_ms_per_step"] = round(g, 4) if isinstance(g, float) else g
     prof = res["prof"]
     if wl["kind"] == "muon":
         ns_ms = sum(prof[k][1] for k in ("ns_syrk", "ns_poly", "ns_axpy", "ns_flow") if k in prof) / res["steps"]
@@ -215,7 +245,24 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def roofline_of(res, kind, workload=None):
+def dion_hbm_bytes(wl):
+    """Algorithmic HBM bytes per step of the Dion products over all matrices of the workload (bf16 momentum / weights,
+    factors in the momentum dtype) and the rank, keyed by kernel kind."""
+    import math
+
+    rd = upd = fused = 0.0
+    rank = 0
+    for m, n in wl["shapes"]:
+        r = min(math.ceil(wl["rank_fraction"] * min(m, n)), m, n)   # reference dion/dion.py:672-676
+        rank = max(rank, r)
+        rd += 2.0 * (m * n + (m + n) * r)
+        upd += 2.0 * (2 * m * n + (m + n) * r)
+        fused += 2.0 * (4 * m * n + (max(m, n) + 2 * min(m, n)) * r)
+    return {"dion_bq": (rd, rank), "dion_btp": (rd, rank), "dion_ef": (upd, rank), "dion_upd": (upd, rank),
+            "dion_ef_upd": (fused, rank)}
+
+
+def roofline_of(res, kind, workload=None, hbm_bytes=None):
     """Dominant kernel of the run: algorithmic flops (bytes for the HBM-bound passes) per launch / average launch
     duration."""
     prof = res["prof"]
@@ -230,6 +277,16 @@ def roofline_of(res, kind, workload=None):
                          else ("dion_bq", "dion_btp", "dion_ef", "dion_upd", "dion_ef_upd")) if k in prof]
     dom = max(cands, key=lambda k: prof[k][1])
     n, ms, work = prof[dom]
+    if kind == "dion" and hbm_bytes is not None and dom in hbm_bytes:
+        # A rank-r product moves m n bytes-ish per 2 m n r flops: below r = 312 flop/byte (2.5 PFLOP/s over 8 TB/s) the HBM
+        # roofline binds it -- the low-rank configurations; priced against HBM then (algorithmic bytes per launch).
+        nbytes, rank = hbm_bytes[dom]
+        if rank < PEAK_BF16_FLOPS / PEAK_HBM_BPS:
+            achieved = nbytes / (ms / res["steps"] * 1e-3) / 1e9
+            return dict(bound="hbm", kernel=dom, achieved=round(achieved, 1), peak=PEAK_HBM_BPS / 1e9, unit="GB/s",
+                        frac=round(achieved * 1e9 / PEAK_HBM_BPS, 4), traffic=MEASURED_TRAFFIC_BYTES.get((workload, dom)),
+                        avg_launch_ms=round(ms / n, 5), bytes_per_launch=nbytes * res["steps"] / n,
+                        mfma_frac=round(work / (ms * 1e-3) / PEAK_BF16_FLOPS, 4))
     achieved = work / (ms * 1e-3) / 1e12
     return dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=PEAK_BF16_FLOPS / 1e12, unit="TFLOP/s",
                 frac=round(achieved * 1e12 / PEAK_BF16_FLOPS, 4),
@@ -548,7 +605,7 @@ def main():
                    "optimizer": res["optimizer"], "grad": f"N(0,1e-3) seed {wl['seed']}", "parallelism": "single GPU"},
         "event_ms_per_step": round(res["event_ms"], 4),
         "wall_ms_per_step": round(res["wall_ms"], 4),
-        "roofline": roofline_of(res, wl["kind"], args.workload),
+        "roofline": roofline_of(res, wl["kind"], args.workload, dion_hbm_bytes(wl) if wl["kind"] == "dion" else None),
         "device": device_info(dev),
     }
     out["device"]["streaming_kernel_gbps"] = stream_ceiling(dev)
@@ -563,7 +620,7 @@ def main():
             big = name in ("muon_llama8b", "dion_llama70b_mlp", "muon_4096x14336")   # hundreds of ms and tens of GB per step
             r = measure(w, dev, 3 if big else 10, 1 if big else 2)
             s = summarize(name, w, r)
-            s["roofline"] = roofline_of(r, w["kind"], name)
+            s["roofline"] = roofline_of(r, w["kind"], name, dion_hbm_bytes(w) if w["kind"] == "dion" else None)
             extra[name] = s
         out["extra"] = extra
     if not args.no_cpu_baseline:
