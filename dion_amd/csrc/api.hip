@@ -256,9 +256,8 @@ int ns_poison_weights(void* const* X, int batch, int m, int n, int x_dtype, cons
 
 int ns_normalize_chunk(const NsLayout& L, const NsBuffers& W, int cb, int dtype, float eps, hipStream_t s) {
   DaProfScope prof(DA_PROF_NORMALIZE, 2.0 * (double)L.mw * L.nw * L.esz * cb, s);  // algorithmic bytes (pad excluded)
-  int rc = da_norm_finish(W.partials, L.tiles, cb, eps, dtype == DA_BF16, W.divisor, s);
-  if (rc) return rc;
-  return da_normalize(W.x0, dtype, (long long)(L.x_bytes / L.esz), cb, W.divisor, s);
+  // (the divisor is formed inside the launch from the partial sums: no separate finishing launch)
+  return da_normalize_from_partials(W.x0, dtype, (long long)(L.x_bytes / L.esz), cb, nullptr, W.partials, L.tiles, eps, s);
 }
 
 bool dtype_ok(int d) { return d == DA_BF16 || d == DA_F32; }
@@ -692,19 +691,44 @@ int dion_amd_muon_step_buckets(const dion_amd_muon_bucket* buckets, int nbuckets
     char* res[DA_MAX_GROUPS];
     const int* poison = nullptr;
     bool updated = false;
+    // the weights' pointer tables for the last product's epilogue: as few launches as the tables need
+    DaPtrUploads up{};
+    DaPoisonShape shape{};
+    shape.f32 = x_dtype == DA_F32;
+    auto flush_uploads = [&](int count, bool poisoning) -> int {
+      if (count == 0) return DA_OK;
+      return poisoning ? da_poison_multi_if(up, count, shape, poison, s) : da_upload_ptrs_multi(up, count, s);
+    };
+    auto for_all_tables = [&](bool poisoning) -> int {
+      int count = 0;
+      for (int i = 0; i < nr; ++i) {
+        const dion_amd_muon_bucket& k = buckets[r0 + i];
+        for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {
+          const int c = k.batch - j0 < DA_MAX_PTRS ? k.batch - j0 : DA_MAX_PTRS;
+          for (int j = 0; j < c; ++j) up.t[count].p[j] = k.X[j0 + j];
+          up.dst[count] = sets[i].W.xtab + j0;
+          up.n[count] = c;
+          shape.numel[count] = (long long)k.m * k.n;
+          if (++count == DA_MAX_UPLOADS) {
+            const int rc = flush_uploads(count, poisoning);
+            if (rc) return rc;
+            count = 0;
+          }
+        }
+      }
+      return flush_uploads(count, poisoning);
+    };
     for (int i = 0; i < nr; ++i) {
       const dion_amd_muon_bucket& k = buckets[r0 + i];
-      for (int j0 = 0; j0 < k.batch; j0 += DA_MAX_PTRS) {
-        const int c = k.batch - j0 < DA_MAX_PTRS ? k.batch - j0 : DA_MAX_PTRS;
-        const int rc = ns_set_update(sets[i], k.X + j0, j0, c, k.m, k.n, x_dtype, k.decay, k.adjusted_lr, s);
-        if (rc) return rc;
-      }
+      NsSet& S = sets[i];
+      S.update = 1; S.x_dtype = x_dtype; S.tall = k.m > k.n ? 1 : 0; S.x_ld = k.n; S.decay = k.decay; S.step = k.adjusted_lr;
     }
-    int rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res, &poison, &updated);
+    int rc = for_all_tables(false);
     if (rc) return rc;
-    for (int i = 0; i < nr && updated && poison; ++i) {
-      const dion_amd_muon_bucket& k = buckets[r0 + i];
-      rc = ns_poison_weights(k.X, k.batch, k.m, k.n, x_dtype, poison, s);
+    rc = ns_iterate(sets, nr, DA_BF16, coeffs, steps, faithful, s, res, &poison, &updated);
+    if (rc) return rc;
+    if (updated && poison) {
+      rc = for_all_tables(true);
       if (rc) return rc;
     }
     for (int i = 0; i < nr && !updated; ++i) {

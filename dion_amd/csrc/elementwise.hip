@@ -279,10 +279,29 @@ __device__ __forceinline__ float div_by(float x, float d, float rd) {
   return __builtin_fmaf(rem, rd, q);
 }
 
+// The divisor of matrix b from its partial sums of squares: the same fixed-order fp64 sum and the same roundings as
+// norm_finish_kernel, so every workgroup of the matrix arrives at the same bits.
+__device__ __forceinline__ float divisor_of(const float* partials, int n, float eps, int bf16_mode, double* red) {
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256) s += (double)partials[i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+    __syncthreads();
+  }
+  const float nrm = sqrtf((float)red[0]);
+  return bf16_mode ? rbf(rbf(nrm) + eps) : nrm + eps;
+}
+
+// `partials` != null: the divisor is formed here from the matrix's partial sums (n per matrix) instead of being
+// read from `divisor` -- one launch less in front of every normalisation.
 template <typename TW>
-__global__ __launch_bounds__(256) void normalize_kernel(TW* W, long long per_matrix, const float* divisor) {
+__global__ __launch_bounds__(256) void normalize_kernel(TW* W, long long per_matrix, const float* divisor,
+                                                        const float* partials, int n, float eps, int bf16_mode) {
   const int b = blockIdx.y;
-  const float d = divisor[b];
+  __shared__ double red[256];
+  const float d = partials ? divisor_of(partials + (long long)b * n, n, eps, bf16_mode, red) : divisor[b];
   const float rd = 1.f / d;
   const bool fast = __builtin_isfinite(rd) && rd != 0.f;   // (the same for the whole matrix)
   TW* p = W + (long long)b * per_matrix;
@@ -489,14 +508,22 @@ int da_norm_finish(const float* partials, int tiles, int batch, float eps, int b
 }
 
 int da_normalize(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor, hipStream_t s) {
+  return da_normalize_from_partials(wide, w_dtype, per_matrix, batch, divisor, nullptr, 0, 0.f, s);
+}
+
+int da_normalize_from_partials(void* wide, int w_dtype, long long per_matrix, int batch, const float* divisor,
+                               const float* partials, int tiles, float eps, hipStream_t s) {
   if (per_matrix & 7) return DA_ERR_ALIGN;
+  if (!divisor && !partials) return DA_ERR_ARG;
   long long blocks = (per_matrix + 8191) / 8192;
   if (blocks > 2048) blocks = 2048;
   dim3 grid((unsigned)blocks, batch);
   if (w_dtype == DA_BF16)
-    hipLaunchKernelGGL(normalize_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(wide), per_matrix, divisor);
+    hipLaunchKernelGGL(normalize_kernel<bf16_t>, grid, dim3(256), 0, s, static_cast<bf16_t*>(wide), per_matrix, divisor,
+                       partials, tiles, eps, 1);
   else
-    hipLaunchKernelGGL(normalize_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(wide), per_matrix, divisor);
+    hipLaunchKernelGGL(normalize_kernel<float>, grid, dim3(256), 0, s, static_cast<float*>(wide), per_matrix, divisor,
+                       partials, tiles, eps, 0);
   return da_launch_status();
 }
 
@@ -515,6 +542,36 @@ __global__ __launch_bounds__(256) void poison_kernel(DaPtrTable t, long long num
   }
 }
 }  // namespace
+
+namespace {
+__global__ __launch_bounds__(64) void upload_ptrs_multi_kernel(DaPtrUploads u) {
+  const int k = blockIdx.x;
+  if ((int)threadIdx.x < u.n[k]) u.dst[k][threadIdx.x] = u.t[k].p[threadIdx.x];
+}
+__global__ __launch_bounds__(256) void poison_multi_kernel(DaPtrUploads u, DaPoisonShape sh, const int* flag) {
+  if (*flag == 0) return;
+  const int k = blockIdx.z;
+  if ((int)blockIdx.y >= u.n[k]) return;
+  const float nan = __builtin_nanf("");
+  void* p = u.t[k].p[blockIdx.y];
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < sh.numel[k]; i += (long long)gridDim.x * 256) {
+    if (sh.f32) static_cast<float*>(p)[i] = nan;
+    else static_cast<bf16_t*>(p)[i] = f2bf(nan);
+  }
+}
+}  // namespace
+
+int da_upload_ptrs_multi(const DaPtrUploads& u, int count, hipStream_t s) {
+  if (count < 1 || count > DA_MAX_UPLOADS) return DA_ERR_LIMIT;
+  hipLaunchKernelGGL(upload_ptrs_multi_kernel, dim3((unsigned)count), dim3(64), 0, s, u);
+  return da_launch_status();
+}
+
+int da_poison_multi_if(const DaPtrUploads& u, int count, const DaPoisonShape& sh, const int* flag, hipStream_t s) {
+  if (!flag || count < 1 || count > DA_MAX_UPLOADS) return DA_ERR_ARG;
+  hipLaunchKernelGGL(poison_multi_kernel, dim3(64, DA_MAX_PTRS, (unsigned)count), dim3(256), 0, s, u, sh, flag);
+  return da_launch_status();
+}
 
 int da_upload_ptrs(const DaPtrTable& t, void** dst, int n, hipStream_t s) {
   if (!dst || n < 1 || n > DA_MAX_PTRS) return DA_ERR_LIMIT;
