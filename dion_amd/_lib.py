@@ -77,7 +77,7 @@ _SIGNATURES = {
     "dion_amd_adamw_step": (_i, [_vpp, _vpp, _vpp, _vpp, _c.POINTER(_ll), _i, _i, _i, _i, _i,
                                  _f, _f, _f, _f, _f, _f, _vp]),
     "dion_amd_muon_pre": (_i, [_vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _f, _i, _vp]),
-    "dion_amd_muon_post": (_i, [_vpp, _vpp, _i, _i, _i, _i, _f, _f, _vp]),
+    "dion_amd_muon_post": (_i, [_vpp, _vpp, _i, _i, _i, _i, _i, _f, _f, _vp]),
     "dion_amd_gemm_plan": (_i, [_i, _i, _i, _i, _i, _i, _i]),
     "dion_amd_muon_buckets_workspace_bytes": (_sz, [_bkp, _i]),
     "dion_amd_muon_step_buckets": (_i, [_bkp, _i, _i, _i, _f, _i, _fp, _i, _f, _i, _vp, _sz, _vp]),

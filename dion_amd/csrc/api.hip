@@ -582,10 +582,10 @@ int dion_amd_muon_pre(const void* const* G, void* const* M, void* const* U, int 
   return DA_OK;
 }
 
-int dion_amd_muon_post(void* const* X, const void* const* O, int batch, int m, int n, int x_dtype, float decay,
-                       float adjusted_lr, void* stream) {
+int dion_amd_muon_post(void* const* X, const void* const* O, int batch, int m, int n, int x_dtype, int o_dtype,
+                       float decay, float adjusted_lr, void* stream) {
   if (!X || !O || batch <= 0 || m <= 0 || n <= 0) return DA_ERR_ARG;
-  if (!dtype_ok(x_dtype)) return DA_ERR_DTYPE;
+  if (!dtype_ok(x_dtype) || !dtype_ok(o_dtype)) return DA_ERR_DTYPE;
   if (n & 7) return DA_ERR_ALIGN;
   for (int i = 0; i < batch; ++i) {
     if (!X[i] || !O[i]) return DA_ERR_ARG;
@@ -602,9 +602,9 @@ int dion_amd_muon_post(void* const* X, const void* const* O, int batch, int m, i
     }
     us.use_wtab = 1; us.wide = nullptr;
     us.batch = cb; us.rows = m; us.cols = n; us.ld = n; us.ldw = n;
-    us.x_dtype = x_dtype; us.w_dtype = DA_BF16;
+    us.x_dtype = x_dtype; us.w_dtype = o_dtype;
     us.decay = decay; us.step = adjusted_lr; us.muon = 1;
-    DaProfScope prof(DA_PROF_UNSTAGE, (double)m * n * (2 * xsz + 2) * cb, s);
+    DaProfScope prof(DA_PROF_UNSTAGE, (double)m * n * (2 * xsz + (o_dtype == DA_BF16 ? 2 : 4)) * cb, s);
     const int rc = da_unstage(us, s);
     if (rc) return rc;
   }

@@ -287,15 +287,25 @@ class Muon(Optimizer):
             else:
                 v = u
             o = self._newton_schulz_func(v, epsilon=epsilon).reshape(p.shape)
-            o = o.to(dtype=torch.bfloat16).reshape(rows, cols)
+            # the update is scaled and subtracted in the dtype the function returned (reference dion/muon.py:569-573):
+            # bf16 and fp32 go to the library as they are, anything else as fp32
+            if o.dtype not in (torch.bfloat16, torch.float32):
+                o = o.to(dtype=torch.float32)
+            o = o.reshape(rows, cols)
             if c8 != cols:
                 o = torch.nn.functional.pad(o, (0, c8 - cols))
-            O.append(o.contiguous())
+            o = o.contiguous()
+            if o.data_ptr() % 16:   # (a contiguous view at an odd offset: the kernels move 16-byte segments)
+                o = o.clone()
+            O.append(o)
+        o_dtypes = {o.dtype for o in O}
+        if len(o_dtypes) > 1:
+            O = [o.to(dtype=torch.float32) for o in O]
         alr = adjusted_lr.item() if isinstance(adjusted_lr, Tensor) else float(torch.tensor(adjusted_lr).item())
         with torch.cuda.device(device):
             rc = lib.dion_amd_muon_post(
                 _lib.ptr_array(X), _lib.ptr_array(O), len(plist), rows, c8, _lib.dtype_code(X[0].dtype),
-                (1 - lr * weight_decay).item(), alr, _lib.stream_ptr(device))
+                _lib.dtype_code(O[0].dtype), (1 - lr * weight_decay).item(), alr, _lib.stream_ptr(device))
         _lib.check(rc, "dion_amd_muon_post")
         for dst, padded in crops:
             _lib.crop_back(dst, padded)

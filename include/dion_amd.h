@@ -156,12 +156,13 @@ int dion_amd_muon_step(void* const* X, const void* const* G, void* const* M,
  * pointers to contiguous m x n matrices (n a multiple of 8); U receives bf16.
  *
  * dion_amd_muon_post replaces muon_update_post_orthogonalize (reference dion/muon.py:556-573):
- * X <- decay X;  X <- X - bf16(adjusted_lr O)  for bf16 O of the same shape. */
+ * X <- decay X;  X <- X - r_O(adjusted_lr O)  for O of the same shape in o_dtype (bf16 or f32: whatever the
+ * orthogonalisation returned; the product adjusted_lr O is rounded to O's dtype as the reference's is). */
 int dion_amd_muon_pre(const void* const* G, void* const* M, void* const* U,
                       int batch, int m, int n, int g_dtype, int m_dtype,
                       float mu, int nesterov, void* stream);
 int dion_amd_muon_post(void* const* X, const void* const* O,
-                       int batch, int m, int n, int x_dtype,
+                       int batch, int m, int n, int x_dtype, int o_dtype,
                        float decay, float adjusted_lr, void* stream);
 
 /* Several buckets (each of one shape) in one call.  Replaces the task generator and the task

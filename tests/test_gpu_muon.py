@@ -311,3 +311,31 @@ def test_muon_step_buckets_equals_per_bucket_calls(dev):
             # tile configuration may differ between a grouped and a single launch; accumulation order
             # per output element does not, so the weights agree to the last bit
             assert torch.equal(Xs[j], Xm[j]), f"weights differ: {shape} #{j}"
+
+
+def test_muon_hook_returning_fp32_keeps_its_precision(dev):
+    """A `newton_schulz_func` that returns fp32 (e.g. for fp32 weights): the reference scales and subtracts the update in
+    the dtype the hook returned (dion/muon.py:569-573); the stand-alone weight update takes that dtype as it is --
+    bit for bit against the oracle, which a bf16 rounding of the hook's result would not survive."""
+    from dion_amd import Muon
+    from oracle import muon_step as O
+
+    def stand_in(X, epsilon):
+        return X.float() * 0.37 + X.float() * X.float()
+
+    shapes = [(64, 96), (40, 27)]
+    gen = torch.Generator().manual_seed(23)
+    X0 = [torch.randn(s, generator=gen) * 0.02 for s in shapes]
+    Xo, Mo = [x.clone() for x in X0], [torch.zeros_like(x) for x in X0]
+    params = [torch.nn.Parameter(x.clone().to(dev)) for x in X0]
+    opt = Muon(params, lr=0.02, mu=0.9, weight_decay=0.01, nesterov=True, newton_schulz_func=stand_in)
+    for step in range(2):
+        G = [torch.randn(s, generator=gen) * 1e-1 for s in shapes]
+        for p, g in zip(params, G):
+            p.grad = g.to(dev)
+        for i in range(len(shapes)):
+            O.muon_step([Xo[i]], [G[i]], [Mo[i]], lr=0.02, mu=0.9, weight_decay=0.01, nesterov=True, ns_func=stand_in)
+        opt.step()
+        for i, p in enumerate(params):
+            assert torch.equal(opt.state[p]["momentum"].cpu(), Mo[i]), (step, i)
+            assert torch.equal(p.detach().cpu(), Xo[i]), (step, i)
