@@ -396,7 +396,7 @@ def ceiling(dev):
     rec = torch.zeros(cus * 8 * 4, dtype=torch.int64, device=dev)
     sink = torch.zeros(1, device=dev)
     out = {}
-    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000)):
+    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000), (2, "l2_to_vgpr_stream", 20000)):
         best = None
         for _ in range(3):
             ms = ctypes.c_double(0)

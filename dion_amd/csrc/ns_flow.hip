@@ -19,7 +19,8 @@
 // every finished tile; it is the memory model's own recipe for any placement and serves as the cross-check.)
 //
 // Order.  Tickets of a queue run (iteration, product, matrix, tile); matrices are dealt to the queues round-robin
-// in the order given (the caller sorts them by cost).  The order is topological -- a tile's producers hold smaller
+// in the order given (the caller sorts the groups by cost, costliest first); X X^T takes the groups in that order,
+// the two products behind it in the opposite one.  The order is topological -- a tile's producers hold smaller
 // tickets of the same queue -- so a waiting workgroup only ever waits for workgroups that are running: no deadlock,
 // whatever the placement and however many workgroups are resident.  Every wait is bounded all the same: after
 // `spin_limit` ticks of the 100 MHz counter a workgroup sets the status word and every workgroup leaves at its
@@ -91,13 +92,17 @@ __device__ __forceinline__ Item decode(const FlowArgs& a, int q, int t) {
   r.g = 0;
   int per = 1, first = 0;
   bool found = false;
+  // X X^T takes the groups costliest first (their tiles are the long ones: K is the matrix's long side); the two
+  // products behind it take them cheapest first, so that the tickets that follow X X^T belong to matrices whose
+  // X X^T was over first, and the costly group's tiles are requested when its long tiles have had time to finish
 #pragma unroll
-  for (int g = 0; g < DA_MAX_GROUPS; ++g) {
-    if (g < a.ngroups && !found) {
+  for (int i = 0; i < DA_MAX_GROUPS; ++i) {
+    if (i < a.ngroups && !found) {
+      const int g = r.p == 0 ? i : a.ngroups - 1 - i;
       const FlowGroupDev& G = a.g[g];
       const int nq = ceil8(G.first + G.cnt - q) - ceil8(G.first - q);
       const int tiles = r.p == 2 ? G.tm * G.tn : G.tm * (G.tm + 1) / 2;
-      if (rem < nq * tiles || g + 1 == a.ngroups) {
+      if (rem < nq * tiles || i + 1 == a.ngroups) {
         found = true;
         r.g = g; per = tiles; first = G.first;
       } else {

@@ -6,6 +6,7 @@
 //                  the clock the chip sustains, depends on the data), two wavefronts per SIMD as in the GEMM kernel.
 //   L2 -> LDS    : every workgroup streams the same 64 KB (two operand stages of a 256 x 256 tile: L2 hits after the
 //                  first pass) into LDS with direct-to-LDS loads, as the K loop's staging does, and nothing else.
+//   L2 -> VGPR   : the same 64 KB per pass with 16-byte loads into registers (the other way to stage an operand).
 //
 // Each wavefront also reads the shader-clock counter and the 100 MHz counter at its start and end: their ratio is
 // the clock the compute unit ran at under that load.
@@ -82,6 +83,29 @@ __global__ __launch_bounds__(512) void probe_lds_stream_kernel(const char* __res
   if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
 }
 
+// The same 64 KB per pass into registers (16-byte loads, one per lane and wave-instruction), no LDS involved.
+__global__ __launch_bounds__(512) void probe_reg_stream_kernel(const char* __restrict__ src, int iters, ProbeOut* out,
+                                                               float* sink) {
+  const int lane = threadIdx.x & 63;
+  const int wave = wave_uniform((int)(threadIdx.x >> 6));
+  const char* base = src + (size_t)(blockIdx.x >> 5) * 65536;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  __syncthreads();
+  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+    u32x4_t v[8];
+    const char* b = base;
+    asm volatile("" : "+s"(b));     // (opaque per pass: the loads stay inside the loop)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = ldg16(b + ((i * 8 + wave) * 64 + lane) * 16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc ^= v[i];
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memrealtime(), c1 = __builtin_amdgcn_s_memtime();
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[0] = 1.f;
+  if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
+}
+
 }  // namespace
 
 extern "C" int dion_amd_probe(int which, const void* random_src, size_t src_bytes, int iters, void* records,
@@ -112,6 +136,12 @@ extern "C" int dion_amd_probe(int which, const void* random_src, size_t src_byte
     DA_HIP_CHECK(hipEventRecord(e0, s));
     hipLaunchKernelGGL(probe_lds_stream_kernel, dim3(grid), dim3(512), 131072, s, static_cast<const char*>(random_src),
                        iters, static_cast<ProbeOut*>(records), sink);
+    rc = da_launch_status();
+  } else if (which == 2) {
+    if (src_bytes < (size_t)((grid + 31) / 32) * 65536) return DA_ERR_WORKSPACE;
+    DA_HIP_CHECK(hipEventRecord(e0, s));
+    hipLaunchKernelGGL(probe_reg_stream_kernel, dim3(grid), dim3(512), 0, s, static_cast<const char*>(random_src), iters,
+                       static_cast<ProbeOut*>(records), sink);
     rc = da_launch_status();
   } else {
     return DA_ERR_ARG;
