@@ -228,9 +228,12 @@ def summarize(name, wl, res):
 # (workload, kernel); measured 2026-11-25 on the kernels of this revision (profiles/*_hbm_traffic.md hold the runs);
 # a kernel kind that is not listed has not been measured since it last changed and reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("muon_gpt_small", "ns_axpy"): 676308 * 1024,
+    # the persistent Newton-Schulz launch: all 15 products of all 72 matrices
+    ("muon_gpt_small", "ns_flow"): 5907409 * 1024,
+    # X' = aX + BX over the 32 matrices (mean of the five launches; the last one updates the weights instead of storing X')
+    ("muon_4096x14336", "ns_axpy"): 30005963 * 1024,
     # one Llama-3-8B layer: the grouped X' = aX + BX launch over its four buckets
-    ("muon_llama8b_layer", "ns_axpy"): 3435386 * 1024,
+    ("muon_llama8b_layer", "ns_axpy"): 3534510 * 1024,
     # error feedback + weight update in one pass: mean over the buckets of the workload
     ("dion_gpt_small_r025", "dion_ef_upd"): 277687 * 1024,
     ("dion_llama70b_layer", "dion_ef_upd"): 4027315 * 1024,
@@ -239,9 +242,9 @@ MEASURED_TRAFFIC_BYTES = {
     # the 16-matrix and the 8-matrix bucket: mean of the two launches
     ("dion_llama70b_mlp", "dion_ef_upd"): 33113826 * 1024,
     # the grouped X' = aX + BX launch over all 224 matrices
-    ("muon_llama8b", "ns_axpy"): 105288904 * 1024,
+    ("muon_llama8b", "ns_axpy"): 108577476 * 1024,
     # mean of the AdamW launch (lm_head) and the Lion launch (embedding, norms)
-    ("scalar_gpt_small", "scalar_opt"): 452944 * 1024,
+    ("scalar_gpt_small", "scalar_opt"): 453078 * 1024,
 }
 
 
@@ -396,7 +399,8 @@ def ceiling(dev):
     rec = torch.zeros(cus * 8 * 4, dtype=torch.int64, device=dev)
     sink = torch.zeros(1, device=dev)
     out = {}
-    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000), (2, "l2_to_vgpr_stream", 20000)):
+    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000), (2, "l2_to_vgpr_stream", 20000),
+                               (3, "lds_read_stream", 20000)):
         best = None
         for _ in range(3):
             ms = ctypes.c_double(0)
@@ -540,6 +544,55 @@ def tile_trace(dev):
         del X, A
 
 
+def flow_trace(dev):
+    """`--flow-trace`: time line of the persistent Newton-Schulz launch of one GPT-small Muon step.  Per tile the kernel
+    records when its workgroup took it up, when its dependency was met, when its K loop and when its epilogue ended.
+    One JSON line: per product the mean of the three phases, and per compute unit the sums."""
+    import ctypes
+
+    import numpy as np
+    import torch
+    from dion_amd import _lib
+
+    lib = _lib.load()
+    opt, params, _ = build_optimizer(WORKLOADS["muon_gpt_small"], dev)
+    for _ in range(5):
+        opt.step()
+    torch.cuda.synchronize()
+    lib.dion_amd_ns_flow_trace_enable(1)
+    opt.step()
+    torch.cuda.synchronize()
+    lib.dion_amd_ns_flow_trace_enable(0)
+    cap = 65536
+    buf = np.zeros((cap, 6), dtype=np.uint64)
+    n = ctypes.c_int(0)
+    _lib.check(lib.dion_amd_ns_flow_trace_read(ctypes.c_void_p(buf.ctypes.data), cap, ctypes.byref(n)),
+               "dion_amd_ns_flow_trace_read")
+    buf = buf[:n.value]
+    t = (buf[:, :4].astype(np.int64) - buf[:, 0].astype(np.int64).min()) / 100.0   # microseconds
+    phase = ((buf[:, 4] >> np.uint64(32)) & np.uint64(0xffff)).astype(int)
+    wait, kloop, epi = t[:, 1] - t[:, 0], t[:, 2] - t[:, 1], t[:, 3] - t[:, 2]
+    cus = len(np.unique(buf[:, 5]))
+    # gaps between consecutive tiles of a compute unit
+    order = np.argsort(t[:, 0])
+    last, gaps = {}, []
+    for i in order:
+        k = int(buf[i, 5])
+        if k in last:
+            gaps.append(t[i, 0] - last[k])
+        last[k] = t[i, 3]
+    out = dict(tiles=int(n.value), compute_units=int(cus), launch_us=round(float(t[:, 3].max()), 1), products={})
+    for p, name in enumerate(("A = X X^T", "B = bA + cAA", "X' = aX + BX")):
+        m = (phase % 3) == p
+        out["products"][name] = dict(tiles=int(m.sum()), wait_us=round(float(wait[m].mean()), 2),
+                                     k_loop_us=round(float(kloop[m].mean()), 2),
+                                     epilogue_us=round(float(epi[m].mean()), 2))
+    out["per_compute_unit_us"] = dict(wait=round(float(wait.sum() / cus), 1), k_loop=round(float(kloop.sum() / cus), 1),
+                                      epilogue=round(float(epi.sum() / cus), 1),
+                                      between_tiles=round(float(np.sum(gaps) / cus), 1))
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -550,6 +603,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--tile-trace", action="store_true",
                     help="instead of a workload: time lines of single bf16 GEMM launches (one JSON line per product)")
+    ap.add_argument("--flow-trace", action="store_true",
+                    help="instead of a workload: per-tile time line of the persistent Newton-Schulz launch (GPT-small)")
     ap.add_argument("--ceiling", action="store_true",
                     help="instead of a workload: matrix-core-only and L2->LDS-only probe kernels with the shader clock")
     ap.add_argument("--vendor-matmul", action="store_true",
@@ -568,6 +623,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.flow_trace:
+        flow_trace(dev)
+        return
     if args.tile_trace:
         tile_trace(dev)
         return

@@ -7,6 +7,7 @@
 //   L2 -> LDS    : every workgroup streams the same 64 KB (two operand stages of a 256 x 256 tile: L2 hits after the
 //                  first pass) into LDS with direct-to-LDS loads, as the K loop's staging does, and nothing else.
 //   L2 -> VGPR   : the same 64 KB per pass with 16-byte loads into registers (the other way to stage an operand).
+//   LDS -> VGPR  : 16-byte LDS reads, conflict free, 8 KB per wavefront and pass (what the fragment reads can get).
 //
 // Each wavefront also reads the shader-clock counter and the 100 MHz counter at its start and end: their ratio is
 // the clock the compute unit ran at under that load.
@@ -106,6 +107,31 @@ __global__ __launch_bounds__(512) void probe_reg_stream_kernel(const char* __res
   if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
 }
 
+// LDS reads alone: every wavefront reads 16 bytes per lane, conflict free (consecutive lanes, consecutive addresses),
+// eight reads in flight, from a 64 KB region.
+__global__ __launch_bounds__(512) void probe_lds_read_kernel(int iters, ProbeOut* out, float* sink) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = wave_uniform((int)(threadIdx.x >> 6));
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<float*>(lds)[i] = (float)i;
+  __syncthreads();
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+    u32x4_t v[8];
+    unsigned off = (unsigned)(it & 7) * 8192u;
+    asm volatile("" : "+s"(off));   // (opaque per pass: the reads stay inside the loop)
+    const char* b = lds + off;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const u32x4_t*>(b + ((i ^ wave) & 7) * 1024 + lane * 16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc ^= v[i];
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memrealtime(), c1 = __builtin_amdgcn_s_memtime();
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) sink[0] = 1.f;
+  if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
+}
+
 }  // namespace
 
 extern "C" int dion_amd_probe(int which, const void* random_src, size_t src_bytes, int iters, void* records,
@@ -142,6 +168,17 @@ extern "C" int dion_amd_probe(int which, const void* random_src, size_t src_byte
     DA_HIP_CHECK(hipEventRecord(e0, s));
     hipLaunchKernelGGL(probe_reg_stream_kernel, dim3(grid), dim3(512), 0, s, static_cast<const char*>(random_src), iters,
                        static_cast<ProbeOut*>(records), sink);
+    rc = da_launch_status();
+  } else if (which == 3) {
+    static DaOncePerDevice configured;
+    rc = configured.run([&]() -> int {
+      DA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(probe_lds_read_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+      return DA_OK;
+    });
+    if (rc) return rc;
+    DA_HIP_CHECK(hipEventRecord(e0, s));
+    hipLaunchKernelGGL(probe_lds_read_kernel, dim3(grid), dim3(512), 65536, s, iters, static_cast<ProbeOut*>(records), sink);
     rc = da_launch_status();
   } else {
     return DA_ERR_ARG;
