@@ -3,7 +3,9 @@
   * error feedback + weight update as one pass vs. as two products (reference dion/dion.py:851-853, 865-872);
   * `Dion.step` with its buckets enqueued by worker threads on three streams vs. one after the other;
   * a matrix inside a bucket of the benchmark's size vs. the same matrix stepped alone (reference dion/muon.py:356-486
-    and dion/dion.py:742-875 treat every matrix of a batch independently).
+    and dion/dion.py:742-875 treat every matrix of a batch independently);
+  * the Muon weight update inside the epilogue of the last Newton-Schulz product vs. as the stand-alone pass behind a
+    stand-alone orthogonalisation (reference dion/muon.py:568-573).
 """
 import os
 
@@ -164,3 +166,37 @@ def test_dion_matrix_in_a_16_matrix_70b_bucket(dev):
     eQ = rel_fro(states_1[0]["Q"], states[pick]["Q"])
     print(f"70B bucket, matrix {pick} alone vs in the bucket: M {eM:.2e} X {eX:.2e} Q {eQ:.2e}")
     assert eM <= 2e-3 and eX <= 2e-4 and eQ <= 2e-3
+
+
+@pytest.mark.parametrize("wdtype", [BF, torch.float32])
+@pytest.mark.parametrize("shapes", [
+    [(768, 768)] * 2 + [(3072, 768)] * 2 + [(768, 3072)] * 2,      # product launches: square, tall (transposed), wide
+    [(768, 768)] * 16 + [(3072, 768)] * 8 + [(768, 3072)] * 8,     # enough matrices for the persistent launch
+])
+def test_muon_update_in_the_last_epilogue_equals_the_stand_alone_pass(dev, shapes, wdtype):
+    """`Muon.step` (momentum pass, Newton-Schulz whose last X' = aX + BX applies the weight update in its epilogue)
+    against the same optimizer with the library's own orthogonalisation passed as `newton_schulz_func`, which makes
+    the step run its three stages as separate calls (dion_amd_muon_pre, dion_amd_newton_schulz per matrix,
+    dion_amd_muon_post): weights and momentum after two steps, bit for bit."""
+    from dion_amd import Muon
+    from dion_amd.newton_schulz import zeropower_via_newtonschulz5
+
+    gen = torch.Generator(device=dev).manual_seed(11)
+    X = [(torch.randn(s, generator=gen, device=dev) * 0.02).to(wdtype) for s in shapes]
+    G = [[(torch.randn(s, generator=gen, device=dev) * 1e-3).to(wdtype) for s in shapes] for _ in range(2)]
+    kw = dict(lr=0.02, mu=0.95, weight_decay=0.01, nesterov=True, adjust_lr="spectral_norm")
+    runs = []
+    for hook in (None, zeropower_via_newtonschulz5):
+        params = [torch.nn.Parameter(x.clone()) for x in X]
+        opt = Muon(params, newton_schulz_func=hook, **kw)
+        for step in range(2):
+            for p, g in zip(params, G[step]):
+                p.grad = g
+            opt.step()
+        torch.cuda.synchronize()
+        runs.append((opt, params))
+    (oa, pa), (ob, pb) = runs
+    for i, (a, b) in enumerate(zip(pa, pb)):
+        assert torch.equal(oa.state[a]["momentum"], ob.state[b]["momentum"]), f"momentum differs, matrix {i}"
+        assert torch.equal(a.detach(), b.detach()), f"weights differ, matrix {i} {tuple(a.shape)}"
+    assert not torch.equal(pa[0].detach(), X[0])
