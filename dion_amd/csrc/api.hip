@@ -273,6 +273,15 @@ bool fused_update_enabled() {
   return !env_off;
 }
 
+// B = M + G inside the launch of P = B Q (the default where it applies) or as a pass of its own.
+std::atomic<int> g_opt_fused_bq{-1};
+bool fused_bq_enabled() {
+  const int v = g_opt_fused_bq.load(std::memory_order_relaxed);
+  if (v >= 0) return v != 0;
+  static const bool env_off = getenv("DION_AMD_NO_FUSED_BQ") != nullptr;
+  return !env_off;
+}
+
 // Number of slices (1, 2 or 4) of the inner dimension `mp` for the product R = B^T P (np x r per matrix, `cb`
 // matrices), by the bf16 launcher's own estimate: workgroup rounds x 64-deep stages per tile, a 256 x 256 tile
 // costing 4 per stage on a whole CU and a 128 x 128 tile 3 on half a CU; a sliced product also pays for writing
@@ -456,6 +465,10 @@ int dion_amd_set_option(const char* name, int value) {
   if (!name) return DA_ERR_ARG;
   if (strcmp(name, "fused_update") == 0) {
     g_opt_fused_update.store(value < 0 ? -1 : (value != 0), std::memory_order_relaxed);
+    return DA_OK;
+  }
+  if (strcmp(name, "fused_bq") == 0) {
+    g_opt_fused_bq.store(value < 0 ? -1 : (value != 0), std::memory_order_relaxed);
     return DA_OK;
   }
   if (strcmp(name, "ns_flow") == 0) {
@@ -957,13 +970,17 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
       tx.p[i] = X[b0 + i]; tg.p[i] = const_cast<void*>(G[b0 + i]); tm.p[i] = M[b0 + i]; tq.p[i] = Q[b0 + i];
     }
     int rc;
+    // B = M + G inside the first P = B Q (bf16 momentum and gradients, whole 256-row tiles of B)
+    const bool bq_sum = fused_bq_enabled() && da_dion_bq_sum_applicable(cb, mp, np, r, n, transposed ? 1 : 0, m_dtype, g_dtype);
     {
-      DaProfScope prof(DA_PROF_DION_ELEM, (double)mn * (2 * msz + gsz) * cb, s);
+      DaProfScope prof(DA_PROF_DION_ELEM, bq_sum ? 0.0 : (double)mn * (2 * msz + gsz) * cb, s);
       rc = da_dion_setup(tm, tabM, tx, tabX, cb, nonzero, linfo, s);
       if (rc) return rc;
       // B = M + G, kept in M   (reference dion/dion.py:794)
-      rc = da_add_grad(tm, tg, m_dtype, g_dtype, mn, cb, nonzero, s);
-      if (rc) return rc;
+      if (!bq_sum) {
+        rc = da_add_grad(tm, tg, m_dtype, g_dtype, mn, cb, nonzero, s);
+        if (rc) return rc;
+      }
       // Q in the momentum dtype   (reference dion/dion.py:1216)
       rc = da_cast_table(tq, q_dtype, Qc, m_dtype, np, rank, r, cb, s);
       if (rc) return rc;
@@ -981,7 +998,12 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
       g.C = P; g.sC = sP; g.ldc = r; g.c_dtype = m_dtype;
       g.M = mp; g.N = r; g.K = np;
       g.epilogue = DA_EPI_STORE; g.s0 = 0.f; g.s1 = 1.f;
-      rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
+      if (it == 0 && bq_sum) {
+        DaProfScope prof(DA_PROF_DION_BQ, gemm_flops(g), s);
+        rc = da_dion_bq_sum(tm, tg, Qc, P, sQ, sP, nonzero, cb, mp, np, r, r, n, transposed ? 1 : 0, faithful, s);
+      } else {
+        rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
+      }
       if (rc) return rc;
       // ---- orthonormalise P   (reference dion/dion.py:822, 1267-1308)
       {

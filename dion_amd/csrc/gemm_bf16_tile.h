@@ -530,4 +530,121 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
 #undef DA_MMA2
 }
 
+// K loop of one BT x BT tile whose row operand is the SUM of two bf16 matrices of the same layout, formed on the way
+// into LDS:  acc += sum_k r_bf16(M + G)(m0 + i, k) * B(n0 + j, k).  The row operand goes through registers (16-byte
+// loads of M and of G one stage ahead, eight additions with one rounding each, one 16-byte LDS store per chunk); the
+// column operand is k-strided and staged with direct-to-LDS loads as in the DA_LOOP_EDGE form (its ragged dimension
+// is kept inside the matrix).  `writeback`: the sums are also stored over M (each element by exactly one tile).
+// `any` is or-ed with "some sum is not zero".  M: whole tiles of rows (no checks), dK a multiple of 64.
+// Ends with a workgroup barrier; stores of the last stage may still be in flight.
+template <typename C, bool A_KS>
+__device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, bf16_t* M,
+                                                     const bf16_t* G, const bf16_t* B, int dK, int m0, int n0,
+                                                     char* lds, int tid, int lane, int wave, int wm, int wn,
+                                                     bool writeback, bool& any) {
+  constexpr bool B_KS = true;
+  constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ, NCH = C::NCH, NW = C::NT / 64;
+  constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
+  constexpr int B_BYTES = Tile<BT, B_KS>::bytes;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  static_assert(NCH == 4, "the stage barrier's wait count below is written for four stores per stage");
+#pragma unroll
+  for (int i = 0; i < TMI; ++i)
+#pragma unroll
+    for (int j = 0; j < TNJ; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  StageAddr<C, A_KS> sa(M, d.lda, m0, tid, d.M);
+  StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
+  // the thread's chunks as 32-bit byte offsets from the matrix's first element (wave-uniform base + lane offset: the
+  // launcher keeps the matrix below 4 GiB)
+  const char* const Mc = reinterpret_cast<const char*>(M);
+  const char* const Gc = reinterpret_cast<const char*>(G);
+  const unsigned gs2 = (unsigned)(sa.gstep * 2), ts2 = (unsigned)(sa.tstep * 2);
+  const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
+  const int KT = dK / BK;
+  bf16x8_t fa[TMI], fb[TNJ];
+  u32x4_t rm[NCH], rg[NCH];
+  unsigned nz = 0u;
+  unsigned koff_b = 0;
+  unsigned aoff = (unsigned)((sa.g - M) * 2);   // chunk 0 of the stage being loaded
+
+#define DA_SUM_LOAD()                                                                              \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        rm[i] = ldg16(Mc + (size_t)(aoff + i * gs2));                                              \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        rg[i] = ldg16(Gc + (size_t)(aoff + i * gs2));                                              \
+  } while (0)
+#define DA_SUM_DMA(st)                                                                             \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
+    koff_b += (unsigned)(sb.tstep * 2);                                                            \
+  } while (0)
+// (the stage loaded last: its chunks lie at aoff; the sums go to LDS and, with writeback, over M)
+#define DA_SUM_STORE(st)                                                                           \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i) {                                              \
+      u32x4_t o;                                                                                   \
+      _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                              \
+        const unsigned x = rm[i][q], y = rg[i][q];                                                 \
+        o[q] = cvt_pk_bf16(lo_f(x) + lo_f(y), hi_f(x) + hi_f(y));                                  \
+        nz |= o[q] & 0x7fff7fffu;                                                                  \
+      }                                                                                            \
+      *reinterpret_cast<u32x4_t*>((st) + sa.l + i * sa.lstep) = o;                                 \
+      if (writeback) stg16(const_cast<char*>(Mc) + (size_t)(aoff + i * gs2), o);                   \
+    }                                                                                              \
+    aoff += ts2;                                                                                   \
+  } while (0)
+#define DA_SUM_FREAD(st, ks, FA, FB)                                                               \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        FA[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
+    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
+        FB[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+  } while (0)
+#define DA_SUM_MMA(FA, FB)                                                                         \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
+        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[j], FA[i], acc[i][j], 0, 0, 0); \
+  } while (0)
+
+  // (fragments are not double buffered here: the registers hold a stage of M and of G instead, and the loop is
+  // bound by the stream of M and G from HBM, not by the matrix cores)
+  DA_SUM_LOAD();
+  DA_SUM_DMA(lds);
+  DA_SUM_STORE(lds);
+  dma_wait();
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    char* cur = lds + (kt & 1) * STAGE;
+    char* nxt = lds + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < KT;
+    if (more) {
+      DA_SUM_LOAD();
+      DA_SUM_DMA(nxt);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      DA_SUM_FREAD(cur, ks, fa, fb);
+      DA_SUM_MMA(fa, fb);
+    }
+    if (more) DA_SUM_STORE(nxt);
+    // the direct-to-LDS loads of the next stage must have landed; the (up to four) stores issued behind them may
+    // stay in flight: memory operations of a wavefront complete in the order issued
+    if (writeback) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else dma_wait();
+    __syncthreads();
+  }
+  any = any || nz != 0u;
+#undef DA_SUM_LOAD
+#undef DA_SUM_DMA
+#undef DA_SUM_STORE
+#undef DA_SUM_FREAD
+#undef DA_SUM_MMA
+}
+
 }  // namespace

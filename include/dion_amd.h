@@ -361,6 +361,10 @@ int dion_amd_profile_read(int kind, long long* launches, double* total_ms, doubl
  *                   0: always as two products with the update in their epilogues (reference dion/dion.py:851-853
  *                   and 865-872 as two calls); -1: the default (one pass unless DION_AMD_NO_FUSED is set in the
  *                   environment).  Both roads give the same bits.
+ *   "fused_bq"      Dion's B = M + G: 1 formed inside the launch of P = B Q where that applies (bf16 momentum and
+ *                   gradients, the longer dimension a multiple of 256, the shorter of 64); 0 as a pass of its own
+ *                   (reference dion/dion.py:794 and 801 as two calls); -1 the default (inside, unless
+ *                   DION_AMD_NO_FUSED_BQ is set in the environment).  Both roads give the same bits.
  *   "ns_flow"       how the Newton-Schulz iterations of a bucket set are launched: 0 product by product (three
  *                   grouped launches per iteration); 1 as one persistent launch whenever the shapes allow (wide
  *                   dimensions multiples of 256); 2 the same with an L2 write-back after every tile (cross-check);

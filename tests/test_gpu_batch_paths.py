@@ -168,6 +168,45 @@ def test_dion_matrix_in_a_16_matrix_70b_bucket(dev):
     assert eM <= 2e-3 and eX <= 2e-4 and eQ <= 2e-3
 
 
+@pytest.mark.parametrize("shapes,rank_fraction", [
+    ([(768, 768)] * 5 + [(3072, 768)] * 3 + [(768, 3072)] * 3, 0.25),     # one column tile of P (r = 192)
+    ([(1024, 512)] * 3 + [(512, 1024)] * 2, 0.07),                        # a rank off the 64-grid (r = 36 -> 40 columns)
+    ([(28672, 8192)] * 2, 1.0 / 16),                                      # two column tiles, walked by one workgroup
+    ([(8192, 28672)] * 2, 1.0 / 16),                                      # the same, B = M^T
+])
+def test_momentum_plus_gradient_inside_the_first_product_equals_the_separate_pass(dev, shapes, rank_fraction):
+    """`B = M + G` formed inside the launch of `P = B Q` (dion_bq.hip) against the separate pass over M followed by the
+    plain product (reference dion/dion.py:794, 801), switched with `dion_amd_set_option("fused_bq", ...)`: M, X and Q
+    after three steps (the momentum is not zero from the second step on), `torch.equal`.  Matrix 0 starts with an
+    all-zero B, which must take the all-zero guard (P = 0, R = Q: reference dion/dion.py:1416-1444) on both roads: a
+    wrong non-zero flag would leave it with Q = 0."""
+    from dion_amd import _lib
+
+    X, gen = _dion_problem(dev, shapes, 33)
+    G = [[(torch.randn(s, generator=gen, device=dev) * 1e-3).to(BF) for s in shapes] for _ in range(3)]
+    G[0][0].zero_()      # matrix 0 starts with B = 0
+    runs = []
+    try:
+        for fused in (1, 0):
+            _lib.set_option("fused_bq", fused)
+            torch.manual_seed(5)
+            opt, params, states = _make_dion(dev, X, rank_fraction)
+            if runs:
+                for st, ref in zip(states, runs[0][3]):
+                    st["Q"].copy_(ref)
+            q0 = [st["Q"].clone() for st in states]
+            for step in range(3):
+                for p, g in zip(params, G[step]):
+                    p.grad = g
+                opt.step()
+            torch.cuda.synchronize()
+            runs.append((opt, params, states, q0))
+    finally:
+        _lib.set_option("fused_bq", -1)
+    _assert_same("sum inside the product vs separate pass", runs[0][1], runs[0][2], runs[1][1], runs[1][2])
+    assert not torch.equal(runs[0][1][1].detach(), X[1])
+
+
 @pytest.mark.parametrize("wdtype", [BF, torch.float32])
 @pytest.mark.parametrize("shapes", [
     [(768, 768)] * 2 + [(3072, 768)] * 2 + [(768, 3072)] * 2,      # product launches: square, tall (transposed), wide
