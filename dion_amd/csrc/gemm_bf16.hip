@@ -143,7 +143,8 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
                     k0 * (B_KS ? d.ldb : 1);
 
   f32x16_t acc[TMI][TNJ];
-  gemm_tile_k_loop<C, A_KS, B_KS, MODE>(acc, d, A, B, dK, m0, n0, lds, tid, lane, wave, wm, wn);
+  gemm_tile_k_loop<C, A_KS, B_KS, MODE>(acc, d, A, B, dK, m0, n0, lds, tid, lane, wave, wm, wn, DaNoHook(),
+                                        SYM && ti == tj && A == B);
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
   epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, tile.b, ti, tj, m0, n0, wave, lane, wm, wn);
   if (trace) {

@@ -375,11 +375,14 @@ constexpr int DA_LOOP_CHECKED = 0, DA_LOOP_INTERIOR = 1, DA_LOOP_EDGE = 2;
 // Ends with a workgroup barrier: the stage buffers are free for the epilogue.
 // `after_first_stage` (direct-to-LDS forms) is called once, behind the barrier that publishes the first stage: every
 // wavefront has waited for all of its outstanding memory operations by then, stores of earlier work included.
+// `same_panel` (direct-to-LDS forms, both operands k-contiguous): the two operands are the same rows of the same
+// matrix -- a diagonal tile of X X^T or A A -- so one panel is staged and both fragment sets are read from it.
 struct DaNoHook { __device__ __forceinline__ void operator()() const {} };
 template <typename C, bool A_KS, bool B_KS, int MODE, typename Hook = DaNoHook>
 __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, const bf16_t* A,
                                                  const bf16_t* B, int dK, int m0, int n0, char* lds, int tid, int lane,
-                                                 int wave, int wm, int wn, Hook after_first_stage = Hook()) {
+                                                 int wave, int wm, int wn, Hook after_first_stage = Hook(),
+                                                 bool same_panel = false) {
   constexpr bool FULL = MODE != DA_LOOP_CHECKED;   // the direct-to-LDS K loop
   constexpr int BT = C::BT, TMI = C::TMI, TNJ = C::TNJ, NCH = C::NCH, NW = C::NT / 64;
   constexpr int A_BYTES = Tile<BT, A_KS>::bytes;
@@ -398,19 +401,20 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
   const int KT = (dK + BK - 1) / BK;
   bf16x8_t fa[TMI], fb[TNJ];
 
+  const int b_at = (FULL && !A_KS && !B_KS && same_panel) ? 0 : A_BYTES;   // where the column operand's panel lies in a stage
 #define DA_FREAD(st, ks)                                                                           \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
         fa[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
     _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        fb[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+        fb[j] = read_frag<BT, B_KS>((st) + b_at, br0 + j * 32, (ks), lane);                        \
   } while (0)
 #define DA_FREAD2(st, ks, FA, FB)                                                                  \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
         FA[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
     _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        FB[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+        FB[j] = read_frag<BT, B_KS>((st) + b_at, br0 + j * 32, (ks), lane);                        \
   } while (0)
 #define DA_MMA2(FA, FB)                                                                            \
   do {                                                                                             \
@@ -431,8 +435,10 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
         dma16(sa.dbase, sa.doff + i * sa.dstep + koff_a, lds_addr(st) + (i * NW + wave) * 1024);   \
-    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
-        dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
+    if (b_at != 0) {                                                                               \
+      _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                              \
+          dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
+    }                                                                                              \
     koff_a += (unsigned)(sa.tstep * 2);                                                            \
     if (koff_a == wrap_a) koff_a = 0;                                                              \
     koff_b += (unsigned)(sb.tstep * 2);                                                            \

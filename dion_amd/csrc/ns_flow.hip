@@ -281,7 +281,7 @@ __global__ __launch_bounds__(Big::NT) void ns_flow_kernel(FlowArgs a) {
       d.s0 = w.p == 2 ? ca : (w.p == 1 ? cb : 0.f);
       d.s1 = w.p == 1 ? cc : 1.f;
       if (w.p == 2) gemm_tile_k_loop<Big, false, true, DA_LOOP_INTERIOR>(acc, d, Aop, Bop, d.K, m0, n0, lds, tid, lane, wave, wm, wn, publish);
-      else gemm_tile_k_loop<Big, false, false, DA_LOOP_INTERIOR>(acc, d, Aop, Bop, d.K, m0, n0, lds, tid, lane, wave, wm, wn, publish);
+      else gemm_tile_k_loop<Big, false, false, DA_LOOP_INTERIOR>(acc, d, Aop, Bop, d.K, m0, n0, lds, tid, lane, wave, wm, wn, publish, ti == tj);
       if (trace) ts[2] = now_ticks();
       // the next ticket is requested before the epilogue, which hides its latency
       if (tid == 0) next = take_ticket(a.tickets + q, xcd, total, true);
