@@ -399,8 +399,8 @@ def ceiling(dev):
     rec = torch.zeros(cus * 8 * 4, dtype=torch.int64, device=dev)
     sink = torch.zeros(1, device=dev)
     out = {}
-    for which, name, iters in ((0, "mfma_only", 20000), (1, "l2_to_lds_stream", 20000), (2, "l2_to_vgpr_stream", 20000),
-                               (3, "lds_read_stream", 20000)):
+    for which, name, iters in ((0, "mfma_only", 20000), (4, "mfma_only_16x16x32", 20000), (1, "l2_to_lds_stream", 20000),
+                               (2, "l2_to_vgpr_stream", 20000), (3, "lds_read_stream", 20000)):
         best = None
         for _ in range(3):
             ms = ctypes.c_double(0)
@@ -411,8 +411,8 @@ def ceiling(dev):
             if best is None or ms.value < best[0]:
                 best = (ms.value, mhz)
         ms, mhz = best
-        if which == 0:
-            flops = cus * 8 * iters * 32 * 32768.0
+        if which in (0, 4):
+            flops = cus * 8 * iters * (32 * 32768.0 if which == 0 else 64 * 16384.0)
             out[name] = dict(pflops=round(flops / (ms * 1e-3) / 1e15, 3), frac_of_2_5_pflops=round(flops / (ms * 1e-3) / PEAK_BF16_FLOPS, 3),
                              shader_clock_mhz=round(mhz), ms=round(ms, 3),
                              peak_at_that_clock_pflops=round(cus * 4096 * mhz * 1e6 / 1e15, 3))

@@ -4,6 +4,7 @@
 //   matrix cores : every wavefront issues v_mfma_f32_32x32x16_bf16 back to back on eight independent accumulators
 //                  with operands held in registers (random bf16 values: the power a matrix core draws, and with it
 //                  the clock the chip sustains, depends on the data), two wavefronts per SIMD as in the GEMM kernel.
+//                  (A second form issues v_mfma_f32_16x16x32_bf16 on sixteen accumulators: the same flops per pass.)
 //   L2 -> LDS    : every workgroup streams the same 64 KB (two operand stages of a 256 x 256 tile: L2 hits after the
 //                  first pass) into LDS with direct-to-LDS loads, as the K loop's staging does, and nothing else.
 //   L2 -> VGPR   : the same 64 KB per pass with 16-byte loads into registers (the other way to stage an operand).
@@ -58,6 +59,43 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(const bf16_t* __restric
 #pragma unroll
       for (int v = 0; v < 16; ++v) r += acc[i][j][v];
   if (r == 12345.678f) sink[0] = r;   // keeps the accumulators alive
+  if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
+}
+
+// The same with v_mfma_f32_16x16x32_bf16 (half the flops per instruction, sixteen independent accumulators).
+__global__ __launch_bounds__(512) void probe_mfma16_kernel(const bf16_t* __restrict__ src, int iters, ProbeOut* out,
+                                                           float* sink) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  bf16x8_t fa[4], fb[4];
+  const u32x4_t* s = reinterpret_cast<const u32x4_t*>(src) + (size_t)((blockIdx.x * 8 + wave) * 64 + lane) * 6;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) fa[i] = __builtin_bit_cast(bf16x8_t, s[i]);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) fb[j] = __builtin_bit_cast(bf16x8_t, s[2 + j]);
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int rep = 0; rep < 4; ++rep)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memrealtime(), c1 = __builtin_amdgcn_s_memtime();
+  float r = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) r += acc[i][j][v];
+  if (r == 12345.678f) sink[0] = r;
   if (lane == 0) out[blockIdx.x * 8 + wave] = ProbeOut{t0, t1, c0, c1};
 }
 
@@ -167,6 +205,12 @@ extern "C" int dion_amd_probe(int which, const void* random_src, size_t src_byte
     if (src_bytes < (size_t)((grid + 31) / 32) * 65536) return DA_ERR_WORKSPACE;
     DA_HIP_CHECK(hipEventRecord(e0, s));
     hipLaunchKernelGGL(probe_reg_stream_kernel, dim3(grid), dim3(512), 0, s, static_cast<const char*>(random_src), iters,
+                       static_cast<ProbeOut*>(records), sink);
+    rc = da_launch_status();
+  } else if (which == 4) {
+    if (src_bytes < (size_t)grid * 8 * 64 * 6 * 16) return DA_ERR_WORKSPACE;
+    DA_HIP_CHECK(hipEventRecord(e0, s));
+    hipLaunchKernelGGL(probe_mfma16_kernel, dim3(grid), dim3(512), 0, s, static_cast<const bf16_t*>(random_src), iters,
                        static_cast<ProbeOut*>(records), sink);
     rc = da_launch_status();
   } else if (which == 3) {

@@ -391,7 +391,7 @@ int dion_amd_tile_trace_read(void* host_dst, int tiles);
  * registers, loaded once from `random_src` (device memory, at least compute units x 49152 bytes of random bf16).
  * which = 1: every workgroup streams the same 64 KB of `random_src` (at least compute units / 32 x 65536 bytes) into
  * LDS with direct-to-LDS loads `iters` times.  which = 2: the same 64 KB per pass with 16-byte loads into registers.  which = 3: 16-byte
- * LDS reads only, 64 KB per pass and workgroup.
+ * LDS reads only, 64 KB per pass and workgroup.  which = 4: as 0 with v_mfma_f32_16x16x32_bf16 on sixteen accumulators.
  * `records` (device memory, 32 bytes per wavefront = compute units x 256
  * bytes) receives per wavefront the 100 MHz counter and the shader-clock counter at its start and end; `sink`: one
  * float of device memory (never written in practice).  The call waits for the launch and returns its duration
