@@ -1001,6 +1001,11 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
       if (it == 0 && bq_sum) {
         DaProfScope prof(DA_PROF_DION_BQ, gemm_flops(g), s);
         rc = da_dion_bq_sum(tm, tg, Qc, P, sQ, sP, nonzero, cb, mp, np, r, r, n, transposed ? 1 : 0, faithful, s);
+        if (rc == DA_OK && r > 256) {
+          // the columns of P beyond the first 256: a plain product on the B that launch left in M
+          g.B = Qc + 256 * L.msz; g.C = P + 256 * L.msz; g.N = r - 256;
+          rc = da_gemm_bf16(g, s);
+        }
       } else {
         rc = gemm_any(g, m_dtype, s, DA_PROF_DION_BQ);
       }
@@ -1079,6 +1084,7 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
     g.lda = r; g.ldb = r; g.K = r;
     g.Ctab = tabM; g.Etab = const_cast<const void* const*>(tabM); g.ldc = n; g.lde = n; g.c_dtype = m_dtype;
     g.epilogue = DA_EPI_AXPBY; g.s0 = 1.f; g.s1 = ef_alpha;
+    g.mi32 = 1;   // (the bits of the one-pass kernel)
     rc = gemm_any(g, m_dtype, s, DA_PROF_DION_EF);
     if (rc) return rc;
     // ---- Q_new = column-normalised R   (reference dion/dion.py:856, 875, 1460-1491, 1533-1561)
@@ -1096,6 +1102,7 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
     g.lda = r; g.ldb = r; g.K = r;
     g.Ctab = tabX; g.Etab = const_cast<const void* const*>(tabX); g.ldc = n; g.lde = n; g.c_dtype = x_dtype;
     g.epilogue = DA_EPI_AXPBY; g.s0 = decay; g.s1 = -scaled_lr;
+    g.mi32 = 1;
     rc = gemm_any(g, m_dtype, s, DA_PROF_DION_UPD);
     if (rc) return rc;
   }

@@ -138,6 +138,10 @@ struct GemmDesc {
   void* const* upd_tab;
   int upd_dtype, upd_ld, upd_transposed;
   float upd_decay, upd_step;
+  // bf16 only, both operands k-contiguous, not symmetric: run the product with v_mfma_f32_32x32x16_bf16 (16 values of k
+  // per instruction instead of 32: another order of the fp32 sums).  Dion's error-feedback and weight-update products
+  // use it so that their bits are those of the one-pass kernel (dion_fused.hip), which is built on that instruction.
+  int mi32;
 };
 
 // Epilogues.  With `faithful` set the rounding points of the reference's separate

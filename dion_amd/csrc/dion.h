@@ -45,7 +45,9 @@ int da_orthonormalize_sketch(const void* P, const void* S, void* out, int dtype,
 // B = M + G and P = B Q in one launch (dion_bq.hip; reference dion/dion.py:794, 801): the product's row operand is
 // formed from M and G on the way into LDS and written back over M.  tabM / tabG: the matrices (bf16, row pitch ldm;
 // `transposed`: B is the transpose of what is stored, mp x np either way); Q: batch x np x ldq, P: batch x mp x ldq
-// (bf16, r live columns); nonzero[b] is set when some element of B[b] is not zero.  Same bits as the two launches.
+// (bf16, r live columns); nonzero[b] is set when some element of B[b] is not zero.  Computes the first 256 columns of
+// P; the caller launches the plain product for the others (on the B this launch leaves in M).  Same bits as the two
+// launches.
 bool da_dion_bq_sum_applicable(int batch, int mp, int np, int r, int ldm, int transposed, int m_dtype, int g_dtype);
 int da_dion_bq_sum(const DaPtrTable& tabM, const DaPtrTable& tabG, const void* Q, void* P, long long sQ, long long sP,
                    int* nonzero, int batch, int mp, int np, int r, int ldq, int ldm, int transposed, int faithful,

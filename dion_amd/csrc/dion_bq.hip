@@ -6,11 +6,11 @@
 // loaded once, added with the reference's one rounding, stored into the operand stage and back over M -- so the
 // addition's three passes over the matrix run under the product's matrix-core work and B is not read again.
 //
-// A workgroup owns 256 rows of B (all of K) and walks the column tiles of P: the first one with the summing K loop
-// (which writes B back), the others -- ranks above 256 -- with the plain direct-to-LDS loop on the B it has just
-// written (its stores acknowledged, its compute unit's L1 lines dropped first).  No other workgroup touches those
-// rows, so no element of M is added to twice.  The products are the batched kernel's tile code with the same
-// order of summation: P has the same bits as from the two launches.
+// A workgroup owns 256 rows of B (all of K) and computes the first 256 columns of P with the summing K loop, which
+// writes B back; no other workgroup touches those rows, so no element of M is added to twice.  Columns of P beyond
+// the first 256 (ranks above 256) are a plain product on the finished B, launched by the caller behind this one.
+// The tile code is the batched kernel's, with the same order of summation: P has the same bits as from the two
+// launches.
 #include "dion.h"
 #include "gemm_bf16_tile.h"
 
@@ -52,26 +52,10 @@ __global__ __launch_bounds__(Big::NT) void dion_bq_sum_kernel(BqArgs a) {
   d.C = a.P + (long long)b * a.sP;
   d.epilogue = DA_EPI_STORE; d.s0 = 0.f; d.s1 = 1.f;
 
-  const int col_tiles = (a.r + BT - 1) / BT;
   bool any = false;
-  f32x16_t acc[Big::TMI][Big::TNJ];
-  for (int tj = 0; tj < col_tiles; ++tj) {
-    const int n0 = tj * BT;
-    if (tj == 0) {
-      gemm_tile_k_loop_sum<Big, A_KS>(acc, d, M, G, Q, d.K, m0, n0, lds, tid, lane, wave, wm, wn, true, any);
-    } else {
-      if (tj == 1) {
-        // B is complete for these rows once this workgroup's stores are acknowledged; what its compute unit's L1
-        // holds of M is stale
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        asm volatile("buffer_inv sc0" ::: "memory");
-      }
-      gemm_tile_k_loop<Big, A_KS, true, DA_LOOP_EDGE>(acc, d, M, Q, d.K, m0, n0, lds, tid, lane, wave, wm, wn);
-    }
-    epilogue<Big, false, false>(acc, d, lds, 0, ti, tj, m0, n0, wave, lane, wm, wn);
-    __syncthreads();   // (the epilogue stages through the buffers the next column tile's first stage goes into)
-  }
+  Big::acc_t acc[Big::TMI][Big::TNJ];
+  gemm_tile_k_loop_sum<Big, A_KS>(acc, d, M, G, Q, d.K, m0, 0, lds, tid, lane, wave, wm, wn, true, any);
+  epilogue<Big, false, false>(acc, d, lds, 0, ti, 0, m0, 0, wave, lane, wm, wn);
   // every writer stores the same value: no atomic needed
   if (__any(any) && lane == 0) a.nonzero[b] = 1;
 }
@@ -85,8 +69,8 @@ long long span_bytes(bool kstrided, long long ld, long long K) {
 }  // namespace
 
 // bf16 momentum and gradients; whole 256-row tiles of B; K in whole stages; the rank a multiple of 8 (the working
-// matrices' pitch).  With more than one column tile a workgroup walks them one after the other: worth it only while
-// the row blocks alone keep most of the compute units busy.
+// matrices' pitch).  Ranks above 256 leave the other column tiles to a second launch: worth it only while the row
+// blocks alone keep most of the compute units busy.
 bool da_dion_bq_sum_applicable(int batch, int mp, int np, int r, int ldm, int transposed, int m_dtype, int g_dtype) {
   if (m_dtype != DA_BF16 || g_dtype != DA_BF16) return false;
   if (mp % 256 || np % BK || (r & 7) || r < 8) return false;

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const bf16_t* B = (d.Btab ? static_cast<const bf16_t*>(d.Btab[b]) : static_cast<const bf16_t*>(d.B) + (long long)b * d.sB) +
                     k0 * (B_KS ? d.ldb : 1);
 
-  f32x16_t acc[TMI][TNJ];
+  typename C::acc_t acc[TMI][TNJ];
   gemm_tile_k_loop<C, A_KS, B_KS, MODE>(acc, d, A, B, dK, m0, n0, lds, tid, lane, wave, wm, wn, DaNoHook(),
                                         SYM && ti == tj && A == B);
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
@@ -299,6 +299,8 @@ double launch_cost(const GemmDesc* d, int n, int slots, double unit) {
 
 typedef Cfg<256, 2, 4> Big;
 typedef Cfg<128, 2, 2> Small;
+typedef Cfg<256, 2, 4, 32> Big32;      // (GemmDesc::mi32)
+typedef Cfg<128, 2, 2, 32> Small32;
 
 // Tile choice by cost model: 256 x 256 tiles run one per CU, 128 x 128 tiles two per CU; a small
 // tile does a quarter of the work on half a CU at about 2/3 of the large tile's MFMA efficiency
@@ -332,12 +334,17 @@ int da_gemm_bf16_grouped(const GemmDesc* din, int n, hipStream_t stream) {
     if (rc) return rc;
     const GemmDesc &a = din[g], &f = din[0];
     if (a.symmetric != f.symmetric || a.a_kstrided != f.a_kstrided || a.b_kstrided != f.b_kstrided ||
-        a.epilogue != f.epilogue || a.c_dtype != f.c_dtype || a.faithful != f.faithful)
+        a.epilogue != f.epilogue || a.c_dtype != f.c_dtype || a.faithful != f.faithful || (a.mi32 != 0) != (f.mi32 != 0))
       return DA_ERR_ARG;
+    if (a.mi32 && (a.symmetric || a.a_kstrided || a.b_kstrided)) return DA_ERR_ARG;
     // insertion sort, longest K first: long tiles start early, short ones fill the tail
     int pos = g;
     while (pos > 0 && d[pos - 1].K < a.K) { d[pos] = d[pos - 1]; --pos; }
     d[pos] = a;
+  }
+  if (d[0].mi32) {
+    if (choose_tile(d, n) == 256) return launch<Big32, false, false, false>(d, n, stream);
+    return launch<Small32, false, false, false>(d, n, stream);
   }
   if (choose_tile(d, n) == 256) return dispatch_layout<Big>(d, n, stream);
   return dispatch_layout<Small>(d, n, stream);

@@ -10,14 +10,27 @@
 
 namespace {
 
-template <int BT_, int WGM_, int WGN_>
+// MI: edge of the MFMA's output block -- 32: v_mfma_f32_32x32x16_bf16 (16 accumulator registers per block, 16-deep
+// k-steps), 16: v_mfma_f32_16x16x32_bf16 (4 registers, 32-deep k-steps; the chip holds a higher clock under it).
+template <int MI> struct AccOf;
+template <> struct AccOf<32> { typedef f32x16_t type; };
+template <> struct AccOf<16> { typedef f32x4_t type; };
+
+#ifndef DA_MI
+#define DA_MI 16   // the MFMA shape the kernels of this library are built with (32: the 32x32x16 form)
+#endif
+
+template <int BT_, int WGM_, int WGN_, int MI_ = DA_MI>
 struct Cfg {
-  static constexpr int BT = BT_, WGM = WGM_, WGN = WGN_;
+  static constexpr int BT = BT_, WGM = WGM_, WGN = WGN_, MI = MI_;
   static constexpr int NT = 64 * WGM * WGN;        // threads
-  static constexpr int TMI = BT / (32 * WGM);      // accumulators per wavefront, row direction
-  static constexpr int TNJ = BT / (32 * WGN);      // ... column direction
+  static constexpr int TMI = BT / (MI * WGM);      // accumulator blocks per wavefront, row direction
+  static constexpr int TNJ = BT / (MI * WGN);      // ... column direction
+  static constexpr int AV = MI * MI / 64;          // accumulator registers per block
   static constexpr int NCH = BT * 8 / NT;          // 16-byte chunks per thread per operand stage
   static constexpr int WROWS = BT / WGM, WCOLS = BT / WGN;
+  static constexpr int NB = WROWS / 32;            // 32-row bands of a wavefront's sub-tile (the epilogue's unit)
+  typedef typename AccOf<MI>::type acc_t;
 };
 
 template <int BT, bool KS>
@@ -119,7 +132,7 @@ __device__ __forceinline__ void update_weights8(char* Wp, bool w_f32, u32x4_t x0
 // UPD: 0 the result is stored in C; 1 / 2 it is not stored but updates the weights d.upd_tab[b] in place (2: those are
 // stored transposed), see GemmDesc.
 template <typename C, bool SYM, bool FULL, bool CF32, bool HAS_E, bool FAITHFUL, bool S1_ONE, int UPD = 0, bool WF32 = false>
-__device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
+__device__ __forceinline__ void epilogue_impl(typename C::acc_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b,
                                               bool mirror, int m0, int n0, int wave, int lane, int wm, int wn) {
   constexpr int W = C::WCOLS;        // columns of a wavefront's sub-tile
   constexpr int PITCH = W + 4;       // floats; 16-byte aligned rows, conflict-free float4 writes
@@ -149,7 +162,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
   const float w_decay = d.upd_decay, w_step = d.upd_step;
   // E is requested up to three bands ahead (registers that the K loop's fragments no longer need), so that a
   // tile's epilogue pays one memory latency and not one per band; an fp32 E (twice the registers) one band ahead.
-  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (UPD ? 2 : (C::TMI < 3 ? C::TMI : 3));
+  constexpr int DEPTH = (!HAS_E || CF32) ? 1 : (UPD ? 2 : (C::NB < 3 ? C::NB : 3));
   u32x4_t ev[DEPTH][NPASS][NV];
   // the weights a band updates are requested when the band starts, ahead of its staging through LDS and of the
   // arithmetic on E (two vectors per 8 elements when they are fp32)
@@ -192,16 +205,26 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
     for (int q = 0; q < DEPTH; ++q) load_e(q, ev[q]);
   }
 #pragma unroll
-  for (int i = 0; i < C::TMI; ++i) {
+  for (int i = 0; i < C::NB; ++i) {
     if (UPD) load_w(i, wv);
-    {
+    if (C::MI == 32) {
       float* row = stg + (lane & 31) * PITCH + (lane >> 5) * 4;
 #pragma unroll
       for (int j = 0; j < C::TNJ; ++j)
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq)
+        for (int vq = 0; vq < C::AV / 4; ++vq)
           *reinterpret_cast<float4*>(row + j * 32 + vq * 8) =
               make_float4(acc[i][j][vq * 4], acc[i][j][vq * 4 + 1], acc[i][j][vq * 4 + 2], acc[i][j][vq * 4 + 3]);
+    } else {
+      // 16 x 16 blocks: a lane holds, for row (lane & 15) of a block, the four columns 4 (lane >> 4) .. + 3
+      float* row = stg + (lane & 15) * PITCH + (lane >> 4) * 4;
+#pragma unroll
+      for (int ib = 0; ib < 2; ++ib)
+#pragma unroll
+        for (int j = 0; j < C::TNJ; ++j) {
+          const typename C::acc_t& a = acc[(2 * i + ib) % C::TMI][j];
+          *reinterpret_cast<float4*>(row + ib * 16 * PITCH + j * 16) = make_float4(a[0], a[1], a[2], a[3]);
+        }
     }
     wave_sync_lds();
     const int band_m = wm0 + i * 32;
@@ -211,7 +234,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
       for (int pass = 0; pass < NPASS; ++pass)
 #pragma unroll
         for (int h = 0; h < NV; ++h) ec[pass][h] = ev[i % DEPTH][pass][h];
-      if (i + DEPTH < C::TMI) load_e(i + DEPTH, ev[i % DEPTH]);
+      if (i + DEPTH < C::NB) load_e(i + DEPTH, ev[i % DEPTH]);
     }
 
 #pragma unroll
@@ -321,7 +344,7 @@ __device__ __forceinline__ void epilogue_impl(f32x16_t (&acc)[C::TMI][C::TNJ], c
 }
 
 template <typename C, bool SYM, bool FULL>
-__device__ __forceinline__ void epilogue(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
+__device__ __forceinline__ void epilogue(typename C::acc_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, char* lds, int b, int ti,
                                          int tj, int m0, int n0, int wave, int lane, int wm, int wn) {
   const bool mirror = SYM && (ti != tj);
   const bool cf32 = d.c_dtype == DA_F32, has_e = d.epilogue == DA_EPI_AXPBY, fa = d.faithful != 0;
@@ -379,7 +402,7 @@ constexpr int DA_LOOP_CHECKED = 0, DA_LOOP_INTERIOR = 1, DA_LOOP_EDGE = 2;
 // matrix -- a diagonal tile of X X^T or A A -- so one panel is staged and both fragment sets are read from it.
 struct DaNoHook { __device__ __forceinline__ void operator()() const {} };
 template <typename C, bool A_KS, bool B_KS, int MODE, typename Hook = DaNoHook>
-__device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, const bf16_t* A,
+__device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, const bf16_t* A,
                                                  const bf16_t* B, int dK, int m0, int n0, char* lds, int tid, int lane,
                                                  int wave, int wm, int wn, Hook after_first_stage = Hook(),
                                                  bool same_panel = false) {
@@ -393,15 +416,16 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
 #pragma unroll
     for (int j = 0; j < TNJ; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < C::AV; ++v) acc[i][j][v] = 0.f;
 
   StageAddr<C, A_KS> sa(A, d.lda, m0, tid, d.M);
   StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
   const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
   const int KT = (dK + BK - 1) / BK;
-  bf16x8_t fa[TMI], fb[TNJ];
+  bf16x8_t fa[C::MI == 32 ? TMI : 1], fb[C::MI == 32 ? TNJ : 1];   // (the 16 x 16 form keeps its own sets below)
 
   const int b_at = (FULL && !A_KS && !B_KS && same_panel) ? 0 : A_BYTES;   // where the column operand's panel lies in a stage
+  if constexpr (C::MI == 32) {
 #define DA_FREAD(st, ks)                                                                           \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
@@ -534,6 +558,144 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
 #undef DA_MMA
 #undef DA_FREAD2
 #undef DA_MMA2
+  } else {
+  // ---- v_mfma_f32_16x16x32_bf16: a stage is two 32-deep k-steps; per k-step TMI row fragments (two halves H0, H1) and
+  // TNJ column fragments.  Read-ahead in registers: while the MFMAs of one half run, the other half's row fragments
+  // (and, under H1, the next k-step's column fragments and H0 row fragments) are fetched.
+  constexpr int TH = TMI / 2;
+#define DA16_RA(FA, st, ks, h)                                                                     \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TH; ++i)                                                 \
+        FA[i] = read_frag16<BT, A_KS>((st), ar0 + ((h) * TH + i) * 16, (ks), lane);                \
+  } while (0)
+#define DA16_RB(FB, st, ks)                                                                        \
+  do {                                                                                             \
+    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
+        FB[j] = read_frag16<BT, B_KS>((st) + b_at, br0 + j * 16, (ks), lane);                      \
+  } while (0)
+#define DA16_MMA(FA, FB, h)                                                                        \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TH; ++i)                                                 \
+        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
+            acc[(h) * TH + i][j] =                                                                 \
+                __builtin_amdgcn_mfma_f32_16x16x32_bf16(FB[j], FA[i], acc[(h) * TH + i][j], 0, 0, 0); \
+  } while (0)
+  if (FULL) {
+#define DA16_DMA(st)                                                                               \
+  do {                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                                \
+        dma16(sa.dbase, sa.doff + i * sa.dstep + koff_a, lds_addr(st) + (i * NW + wave) * 1024);   \
+    if (b_at != 0) {                                                                               \
+      _Pragma("unroll") for (int i = 0; i < NCH; ++i)                                              \
+          dma16(sb.dbase, sb.doff + i * sb.dstep + koff_b, lds_addr(st) + A_BYTES + (i * NW + wave) * 1024); \
+    }                                                                                              \
+    koff_a += (unsigned)(sa.tstep * 2);                                                            \
+    if (koff_a == wrap_a) koff_a = 0;                                                              \
+    koff_b += (unsigned)(sb.tstep * 2);                                                            \
+  } while (0)
+    unsigned koff_a = 0, koff_b = 0;
+    const unsigned wrap_a = (unsigned)d.a_kwrap * 2u;
+    DA16_DMA(lds);
+    dma_wait();
+    __syncthreads();
+    after_first_stage();
+    bf16x8_t a0[TH], a1[TH], b0[TNJ], b1[TNJ];
+    DA16_RB(b0, lds, 0);
+    DA16_RA(a0, lds, 0, 0);
+    for (int kt = 0; kt < KT; ++kt) {
+      char* cur = lds + (kt & 1) * STAGE;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE;
+      const bool more = kt + 1 < KT;
+      if (more) DA16_DMA(nxt);
+      DA16_RA(a1, cur, 0, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_MMA(a0, b0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_RB(b1, cur, 1);
+      DA16_RA(a0, cur, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_MMA(a1, b0, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_RA(a1, cur, 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_MMA(a0, b1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      dma_wait();
+      __syncthreads();
+      if (more) {
+        DA16_RB(b0, nxt, 0);
+        DA16_RA(a0, nxt, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      DA16_MMA(a1, b1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+#undef DA16_DMA
+  } else {
+    u32x4_t ra[NCH], rb[NCH];
+    constexpr int A_RSTEP = A_KS ? C::NT / (BT / 8) : C::NT / 8;
+    constexpr int B_RSTEP = B_KS ? C::NT / (BT / 8) : C::NT / 8;
+    auto gload = [&](int kt) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int r_ = sa.row + i * A_RSTEP;
+        const bool ok = A_KS ? (kt * BK + r_ < dK && m0 + sa.col < d.M) : (m0 + r_ < d.M && kt * BK + sa.col < dK);
+        const u32x4_t z_ = {0u, 0u, 0u, 0u};
+        ra[i] = ok ? *reinterpret_cast<const u32x4_t*>(sa.g + i * sa.gstep) : z_;
+      }
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int r_ = sb.row + i * B_RSTEP;
+        const bool ok = B_KS ? (kt * BK + r_ < dK && n0 + sb.col < d.N) : (n0 + r_ < d.N && kt * BK + sb.col < dK);
+        const u32x4_t z_ = {0u, 0u, 0u, 0u};
+        rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;
+      }
+      sa.g += sa.tstep;
+      sb.g += sb.tstep;
+    };
+    auto lstore = [&](char* st) {
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) *reinterpret_cast<u32x4_t*>(st + sa.l + i * sa.lstep) = ra[i];
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) *reinterpret_cast<u32x4_t*>(st + A_BYTES + sb.l + i * sb.lstep) = rb[i];
+    };
+    bf16x8_t a0[TH], a1[TH], b0[TNJ];
+    gload(0);
+    lstore(lds);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      char* cur = lds + (kt & 1) * STAGE;
+      char* nxt = lds + ((kt + 1) & 1) * STAGE;
+      const bool more = kt + 1 < KT;
+      if (more) gload(kt + 1);
+#pragma unroll
+      for (int ks = 0; ks < BK / 32; ++ks) {
+        DA16_RB(b0, cur, ks);
+        DA16_RA(a0, cur, ks, 0);
+        DA16_RA(a1, cur, ks, 1);
+        DA16_MMA(a0, b0, 0);
+        DA16_MMA(a1, b0, 1);
+      }
+      if (more) lstore(nxt);
+      __syncthreads();
+    }
+  }
+#undef DA16_RA
+#undef DA16_RB
+#undef DA16_MMA
+  }
+}
+
+template <typename C, bool KS>
+__device__ __forceinline__ bf16x8_t read_frag_of(const char* lds, int r0, int ks, int lane) {
+  if constexpr (C::MI == 32) return read_frag<C::BT, KS>(lds, r0, ks, lane);
+  else return read_frag16<C::BT, KS>(lds, r0, ks, lane);
+}
+template <typename C>
+__device__ __forceinline__ void mma_of(typename C::acc_t& acc, bf16x8_t col, bf16x8_t row) {
+  if constexpr (C::MI == 32) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(col, row, acc, 0, 0, 0);
+  else acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(col, row, acc, 0, 0, 0);
 }
 
 // K loop of one BT x BT tile whose row operand is the SUM of two bf16 matrices of the same layout, formed on the way
@@ -544,7 +706,7 @@ __device__ __forceinline__ void gemm_tile_k_loop(f32x16_t (&acc)[C::TMI][C::TNJ]
 // `any` is or-ed with "some sum is not zero".  M: whole tiles of rows (no checks), dK a multiple of 64.
 // Ends with a workgroup barrier; stores of the last stage may still be in flight.
 template <typename C, bool A_KS>
-__device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, bf16_t* M,
+__device__ __forceinline__ void gemm_tile_k_loop_sum(typename C::acc_t (&acc)[C::TMI][C::TNJ], const GemmDesc& d, bf16_t* M,
                                                      const bf16_t* G, const bf16_t* B, int dK, int m0, int n0,
                                                      char* lds, int tid, int lane, int wave, int wm, int wn,
                                                      bool writeback, bool& any) {
@@ -559,7 +721,7 @@ __device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::
 #pragma unroll
     for (int j = 0; j < TNJ; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < C::AV; ++v) acc[i][j][v] = 0.f;
 
   StageAddr<C, A_KS> sa(M, d.lda, m0, tid, d.M);
   StageAddr<C, B_KS> sb(B, d.ldb, n0, tid, d.N);
@@ -570,7 +732,7 @@ __device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::
   const unsigned gs2 = (unsigned)(sa.gstep * 2), ts2 = (unsigned)(sa.tstep * 2);
   const int ar0 = wm * C::WROWS, br0 = wn * C::WCOLS;
   const int KT = dK / BK;
-  bf16x8_t fa[TMI], fb[TNJ];
+  bf16x8_t fa[C::MI == 32 ? TMI : TMI / 2], fb[TNJ];
   u32x4_t rm[NCH], rg[NCH];
   unsigned nz = 0u;
   unsigned koff_b = 0;
@@ -607,15 +769,15 @@ __device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::
 #define DA_SUM_FREAD(st, ks, FA, FB)                                                               \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
-        FA[i] = read_frag<BT, A_KS>((st), ar0 + i * 32, (ks), lane);                               \
+        FA[i] = read_frag_of<C, A_KS>((st), ar0 + i * C::MI, (ks), lane);                          \
     _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        FB[j] = read_frag<BT, B_KS>((st) + A_BYTES, br0 + j * 32, (ks), lane);                     \
+        FB[j] = read_frag_of<C, B_KS>((st) + A_BYTES, br0 + j * C::MI, (ks), lane);                \
   } while (0)
 #define DA_SUM_MMA(FA, FB)                                                                         \
   do {                                                                                             \
     _Pragma("unroll") for (int i = 0; i < TMI; ++i)                                                \
         _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FB[j], FA[i], acc[i][j], 0, 0, 0); \
+            mma_of<C>(acc[i][j], FB[j], FA[i]);                                                    \
   } while (0)
 
   // (fragments are not double buffered here: the registers hold a stage of M and of G instead, and the loop is
@@ -633,10 +795,28 @@ __device__ __forceinline__ void gemm_tile_k_loop_sum(f32x16_t (&acc)[C::TMI][C::
       DA_SUM_LOAD();
       DA_SUM_DMA(nxt);
     }
+    if constexpr (C::MI == 32) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      DA_SUM_FREAD(cur, ks, fa, fb);
-      DA_SUM_MMA(fa, fb);
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        DA_SUM_FREAD(cur, ks, fa, fb);
+        DA_SUM_MMA(fa, fb);
+      }
+    } else {
+      // (16 x 16 blocks: the row fragments of a 32-deep k-step in two halves through the same registers)
+#pragma unroll
+      for (int ks = 0; ks < BK / 32; ++ks) {
+#pragma unroll
+        for (int j = 0; j < TNJ; ++j) fb[j] = read_frag16<BT, B_KS>(cur + A_BYTES, br0 + j * 16, ks, lane);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+          for (int i = 0; i < TMI / 2; ++i) fa[i] = read_frag16<BT, A_KS>(cur, ar0 + (h * (TMI / 2) + i) * 16, ks, lane);
+#pragma unroll
+          for (int i = 0; i < TMI / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < TNJ; ++j) mma_of<C>(acc[h * (TMI / 2) + i][j], fb[j], fa[i]);
+        }
+      }
     }
     if (more) DA_SUM_STORE(nxt);
     // the direct-to-LDS loads of the next stage must have landed; the (up to four) stores issued behind them may

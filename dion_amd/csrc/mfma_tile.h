@@ -40,6 +40,31 @@ __device__ __forceinline__ bf16x8_t read_frag(const char* lds, int r0, int ks, i
   }
 }
 
+// Fragment of 16 rows x 32 k for one v_mfma_f32_16x16x32_bf16: lane l gets row (l & 15), k = 8 * (l >> 4) .. +8 of
+// the 32-deep k-step `ks` (0 or 1) of a stage.
+template <int BT, bool KS>
+__device__ __forceinline__ bf16x8_t read_frag16(const char* lds, int r0, int ks, int lane) {
+  if (!KS) {
+    const int row = r0 + (lane & 15);
+    const int phys = kc_swizzle(ks * 4 + (lane >> 4), row);
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * 128 + phys * 16);
+    return __builtin_bit_cast(bf16x8_t, v);
+  } else {
+    // All four 16-lane groups read the same 16 rows, group g the k-rows 8 g .. 8 g + 7: the four lanes 4q .. 4q+3
+    // supply the 16 rows of k-row q (then q + 4), and the transpose read hands lane i the four k values of row i.
+    const int g = lane >> 4;
+    const int q = (lane & 15) >> 2;
+    const int slot = (r0 >> 4) ^ q;
+    const int kr = ks * 32 + g * 8 + q;
+    const char* p = lds + kr * (BT * 2) + slot * 32 + (lane & 3) * 8;
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, p));
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(DA_LDS_PTR(s16x4_t, p + 4 * (BT * 2)));
+    typedef short s16x8_t __attribute__((ext_vector_type(8)));
+    const s16x8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, v);
+  }
+}
+
 __device__ __forceinline__ int wave_uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
 // 16 bytes per lane from global memory straight into LDS: lane p's data lands at LDS byte

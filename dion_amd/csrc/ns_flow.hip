@@ -248,7 +248,7 @@ __global__ __launch_bounds__(Big::NT) void ns_flow_kernel(FlowArgs a) {
       tj = wave_uniform(tj);
       const int m0 = ti * BT, n0 = tj * BT;
       int next = -1;           // (thread 0) the next ticket
-      f32x16_t acc[Big::TMI][Big::TNJ];
+      Big::acc_t acc[Big::TMI][Big::TNJ];
       const bf16_t *Aop, *Bop;
       if (w.p == 0) {
         Aop = Bop = reinterpret_cast<const bf16_t*>(xcur) + (long long)w.b * G.sx;
