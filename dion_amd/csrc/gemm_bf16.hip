@@ -44,6 +44,7 @@ struct GemmArgs {
   int start[DA_MAX_GROUPS + 1];
   int n;
   int trace;   // 1: every workgroup records its time stamps (measurement hook)
+  int diag_k;  // diagonal tiles of a symmetric product stage one panel for both operands when K is at most this
 };
 
 // Which output tile a workgroup owns.  Workgroups are dealt round-robin to the 8 XCDs (each
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
 
   typename C::acc_t acc[TMI][TNJ];
   gemm_tile_k_loop<C, A_KS, B_KS, MODE>(acc, d, A, B, dK, m0, n0, lds, tid, lane, wave, wm, wn, DaNoHook(),
-                                        SYM && ti == tj && A == B);
+                                        SYM && ti == tj && A == B && dK <= args.diag_k);
   if (trace) ts1 = __builtin_amdgcn_s_memrealtime();
   epilogue<C, SYM, MODE == DA_LOOP_INTERIOR>(acc, d, lds, tile.b, ti, tj, m0, n0, wave, lane, wm, wn);
   if (trace) {
@@ -222,6 +223,7 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   GemmArgs args{};
   args.n = n;
   args.trace = g_tile_trace.load(std::memory_order_relaxed) ? 1 : 0;
+
   const bool full = all_interior(d, n, BT);
   static const bool edge_on = [] { const char* e = getenv("DION_AMD_NO_EDGE_LOOP"); return !(e && atoi(e)); }();
   const bool edge = !full && edge_on && (A_KS || B_KS) && !SYM && edge_loop_ok(d, n, BT);
@@ -235,6 +237,12 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
     if (blocks > 0x7fffffffLL) return DA_ERR_LIMIT;
   }
   for (int g = n; g <= DA_MAX_GROUPS; ++g) args.start[g] = (int)blocks;
+  // A diagonal tile that stages one panel runs ahead of the tiles it shares that panel with.  In a launch of a few
+  // rounds that shortens the tail (Llama-8B layer: X X^T 0.81 -> 0.77 ms); over many rounds of a long K the tiles
+  // lose each other in the L2 (32 x 4096 x 14336: 1.7 x the fetched bytes, 6.93 -> 7.35 ms), so there only up to
+  // K = 4096 (bA + cAA: 2 % faster with it).  DION_AMD_DIAG_K overrides the limit (0: never).
+  static const int diag_k_env = [] { const char* e = getenv("DION_AMD_DIAG_K"); return e ? atoi(e) : -1; }();
+  args.diag_k = diag_k_env >= 0 ? diag_k_env : (blocks <= 4LL * da_cu_count() ? 0x7fffffff : 4096);
   if (!full && !edge)   // the bounds-checked K loop walks A with a pointer: no wrap-around there
     for (int g = 0; g < n; ++g)
       if (d[g].a_kwrap) return DA_ERR_ARG;
