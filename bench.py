@@ -206,14 +206,24 @@ def summarize(name, wl, res):
         # products read and write an m x n matrix; each also moves its m' x r and n' x r factors.
         import math
 
-        rd = upd = fused = 0.0
-        for m, n in shapes:
+        from collections import Counter
+
+        from dion_amd import _lib
+        lib = _lib.load()
+        rd = bq = upd = fused = 0.0
+        for (m, n), count in Counter(shapes).items():
             r = min(math.ceil(wl["rank_fraction"] * min(m, n)), m, n)   # reference dion/dion.py:672-676
+            # P = BQ with B = M + G formed inside it also reads G and writes M (the separate pass's bytes are the
+            # dion_elem kind's otherwise)
+            inside = lib.dion_amd_dion_bq_fused(count, m, n, r, 0, 0)
+            bq += count * 2.0 * (m * n * (3 if inside else 1) + (m + n) * r)
+        for m, n in shapes:
+            r = min(math.ceil(wl["rank_fraction"] * min(m, n)), m, n)
             rd += 2.0 * (m * n + (m + n) * r)
             upd += 2.0 * (2 * m * n + (m + n) * r)
             # error feedback and weight update as one pass: M and X read and written once, P, R and Q_new read
             fused += 2.0 * (4 * m * n + (max(m, n) + 2 * min(m, n)) * r)
-        for name, nbytes in (("dion_bq", rd), ("dion_btp", rd), ("dion_ef", upd), ("dion_upd", upd),
+        for name, nbytes in (("dion_bq", bq), ("dion_btp", rd), ("dion_ef", upd), ("dion_upd", upd),
                              ("dion_ef_upd", fused)):
             k = out["kernels"].get(name)
             if k and k["ms_per_step"] > 0:

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "dion_amd_orthonormalize": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "dion_amd_orthonormalize_method": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "dion_amd_dion_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "dion_amd_dion_bq_fused": (_i, [_i, _i, _i, _i, _i, _i]),
     "dion_amd_dion_step": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i,
                                 _vp, _vp, _sz, _vp]),
     "dion_amd_dion_step_qr": (_i, [_vpp, _vpp, _vpp, _vpp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _f, _f, _i, _i, _i,

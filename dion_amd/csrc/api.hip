@@ -825,6 +825,13 @@ int dion_step_impl(void* const* X, const void* const* G, void* const* M, void* c
 
 extern "C" {
 
+int dion_amd_dion_bq_fused(int batch, int m, int n, int rank, int m_dtype, int g_dtype) {
+  if (batch <= 0 || m <= 0 || n <= 0 || rank <= 0 || rank > m || rank > n || !dtype_ok(m_dtype) || !dtype_ok(g_dtype)) return 0;
+  const DionLayout L(m, n, rank, m_dtype);
+  const int cb = batch < DA_MAX_PTRS ? batch : DA_MAX_PTRS;
+  return fused_bq_enabled() && da_dion_bq_sum_applicable(cb, L.mp, L.np, L.r, n, m < n ? 1 : 0, m_dtype, g_dtype) ? 1 : 0;
+}
+
 size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype) {
   if (batch <= 0 || m <= 0 || n <= 0 || r <= 0 || !dtype_ok(m_dtype)) return 0;
   return DionLayout(m, n, r, m_dtype).recommended(batch);

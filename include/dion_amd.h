@@ -263,6 +263,10 @@ int dion_amd_orthonormalize_method(const void* P, void* out, int dtype, int batc
                                    int qr_method, int* info, void* workspace, size_t workspace_bytes, void* stream);
 
 size_t dion_amd_dion_workspace_bytes(int batch, int m, int n, int r, int m_dtype);
+/* 1 if dion_amd_dion_step forms B = M + G inside the launch of P = B Q for a bucket of these dimensions (a chunk of
+ * at most 64 matrices at a time), 0 if it runs the addition as a pass of its own (reference dion/dion.py:794, 801).
+ * No counterpart in the reference: the benchmark uses it to price that launch's HBM traffic. */
+int dion_amd_dion_bq_fused(int batch, int m, int n, int rank, int m_dtype, int g_dtype);
 
 /* Replaces dion_update_ddp with replicate_mesh=None (reference dion/dion.py:742-875) and its
  * helpers tensor_list_to_batch (1200-1218), orthogonalize (1267-1308), fix_all_zero_or_nan
