@@ -10,7 +10,11 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
-LIB = os.path.join(HERE, "libdion_amd.so")
+# Measurement builds: DION_AMD_BUILD_DEFINES holds extra compiler options (e.g. "-DDA_MI=32"), DION_AMD_BUILD_LIB the
+# library to write instead of the in-tree one (its objects go beside it); load it with DION_AMD_LIB.
+LIB = os.environ.get("DION_AMD_BUILD_LIB") or os.path.join(HERE, "libdion_amd.so")
+if os.environ.get("DION_AMD_BUILD_LIB"):
+    OBJ = LIB + ".obj"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -23,6 +27,7 @@ FLAGS = [
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    *os.environ.get("DION_AMD_BUILD_DEFINES", "").split(),
 ]
 
 

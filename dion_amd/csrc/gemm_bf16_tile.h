@@ -19,6 +19,9 @@ template <> struct AccOf<16> { typedef f32x4_t type; };
 #ifndef DA_MI
 #define DA_MI 16   // the MFMA shape the kernels of this library are built with (32: the 32x32x16 form)
 #endif
+#ifndef DA_KLOOP_ABLATE
+#define DA_KLOOP_ABLATE 0   // see gemm_tile_k_loop: measurement builds only
+#endif
 
 template <int BT_, int WGM_, int WGN_, int MI_ = DA_MI>
 struct Cfg {
@@ -563,15 +566,25 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
   // TNJ column fragments.  Read-ahead in registers: while the MFMAs of one half run, the other half's row fragments
   // (and, under H1, the next k-step's column fragments and H0 row fragments) are fetched.
   constexpr int TH = TMI / 2;
+  // Measurement builds (-DDA_KLOOP_ABLATE=<bits>, WRONG RESULTS): what the direct-to-LDS loop costs without 1 its
+  // fragment reads (the first stage's are kept), 2 its staging loads (after the first two stages), 4 the per-stage
+  // wait and barrier.
+  constexpr bool ABL_READ = (DA_KLOOP_ABLATE & 1) != 0, ABL_DMA = (DA_KLOOP_ABLATE & 2) != 0,
+                 ABL_BAR = (DA_KLOOP_ABLATE & 4) != 0;
+  bool abl_first = true;
 #define DA16_RA(FA, st, ks, h)                                                                     \
   do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TH; ++i)                                                 \
-        FA[i] = read_frag16<BT, A_KS>((st), ar0 + ((h) * TH + i) * 16, (ks), lane);                \
+    if (!(FULL && ABL_READ) || abl_first) {                                                        \
+      _Pragma("unroll") for (int i = 0; i < TH; ++i)                                               \
+          FA[i] = read_frag16<BT, A_KS>((st), ar0 + ((h) * TH + i) * 16, (ks), lane);              \
+    }                                                                                              \
   } while (0)
 #define DA16_RB(FB, st, ks)                                                                        \
   do {                                                                                             \
-    _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                                \
-        FB[j] = read_frag16<BT, B_KS>((st) + b_at, br0 + j * 16, (ks), lane);                      \
+    if (!(FULL && ABL_READ) || abl_first) {                                                        \
+      _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                              \
+          FB[j] = read_frag16<BT, B_KS>((st) + b_at, br0 + j * 16, (ks), lane);                    \
+    }                                                                                              \
   } while (0)
 #define DA16_MMA(FA, FB, h)                                                                        \
   do {                                                                                             \
@@ -600,13 +613,13 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
     __syncthreads();
     after_first_stage();
     bf16x8_t a0[TH], a1[TH], b0[TNJ], b1[TNJ];
+    if (KT > 1) DA16_DMA(lds + STAGE);
     DA16_RB(b0, lds, 0);
     DA16_RA(a0, lds, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
       char* cur = lds + (kt & 1) * STAGE;
       char* nxt = lds + ((kt + 1) & 1) * STAGE;
       const bool more = kt + 1 < KT;
-      if (more) DA16_DMA(nxt);
       DA16_RA(a1, cur, 0, 1);
       __builtin_amdgcn_sched_barrier(0);
       DA16_MMA(a0, b0, 0);
@@ -620,8 +633,13 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
       __builtin_amdgcn_sched_barrier(0);
       DA16_MMA(a0, b1, 0);
       __builtin_amdgcn_sched_barrier(0);
-      dma_wait();
-      __syncthreads();
+      if (!ABL_BAR) {
+        dma_wait();
+        __syncthreads();
+      }
+      // this stage's buffer is free (every wavefront holds its last fragments): the stage after the next is requested
+      // here, a full stage ahead of the barrier that needs it
+      if (!ABL_DMA && kt + 2 < KT) DA16_DMA(cur);
       if (more) {
         DA16_RB(b0, nxt, 0);
         DA16_RA(a0, nxt, 0, 0);
@@ -629,7 +647,9 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
       __builtin_amdgcn_sched_barrier(0);
       DA16_MMA(a1, b1, 1);
       __builtin_amdgcn_sched_barrier(0);
+      abl_first = false;
     }
+    if (ABL_BAR) dma_wait();
     __syncthreads();
 #undef DA16_DMA
   } else {
