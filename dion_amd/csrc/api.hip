@@ -476,6 +476,10 @@ int dion_amd_set_option(const char* name, int value) {
     da_ns_flow_set_mode(value);
     return DA_OK;
   }
+  if (strcmp(name, "edge_loop") == 0) {
+    da_gemm_bf16_set_edge_loop(value);
+    return DA_OK;
+  }
   if (strcmp(name, "ns_flow_fail") == 0) {
     da_ns_flow_set_fail(value != 0);
     return DA_OK;

@@ -162,5 +162,7 @@ int da_gemm_bf16_grouped(const GemmDesc* d, int n, hipStream_t stream);
 int da_gemm_f32(const GemmDesc& d, hipStream_t stream);
 // Tile edge (128 / 256) the bf16 launcher picks for one product, + 1 if its K loop is the direct-to-LDS one.
 int da_gemm_bf16_plan(const GemmDesc& d);
+// -1 / 0 / 1: whether ragged products may take the direct-to-LDS K loop with edge tiles (see dion_amd_set_option)
+void da_gemm_bf16_set_edge_loop(int v);
 // Whether da_gemm_bf16_grouped would run every tile of these products in its interior (unchecked) form.
 bool da_gemm_bf16_all_interior(const GemmDesc* d, int n);

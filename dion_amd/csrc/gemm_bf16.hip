@@ -31,6 +31,7 @@
 // accumulators through LDS so that C and E move as 16-byte row segments.  For a symmetric
 // result only tiles on or above the diagonal are computed and every off-diagonal tile is
 // also written transposed.
+#include <atomic>
 #include "common.h"
 #include "mfma_tile.h"
 #include "gemm_bf16_tile.h"
@@ -203,6 +204,10 @@ long long tiles_of(const GemmDesc& d) {
   return (d.symmetric ? tm * (tm + 1) / 2 : tm * tn) * d.batch * (d.k_slices > 1 ? d.k_slices : 1);
 }
 
+// dion_amd_set_option("edge_loop"): -1 the environment decides (DION_AMD_NO_EDGE_LOOP), 0 ragged products take the
+// bounds-checked K loop, 1 the direct-to-LDS loop with edge tiles where it applies.
+std::atomic<int> g_opt_edge_loop{-1};
+
 template <typename C, bool A_KS, bool B_KS, bool SYM>
 int launch(const GemmDesc* d, int n, hipStream_t stream) {
   constexpr int BT = C::BT;
@@ -225,7 +230,9 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   args.trace = g_tile_trace.load(std::memory_order_relaxed) ? 1 : 0;
 
   const bool full = all_interior(d, n, BT);
-  static const bool edge_on = [] { const char* e = getenv("DION_AMD_NO_EDGE_LOOP"); return !(e && atoi(e)); }();
+  static const bool edge_env = [] { const char* e = getenv("DION_AMD_NO_EDGE_LOOP"); return !(e && atoi(e)); }();
+  const int edge_opt = g_opt_edge_loop.load(std::memory_order_relaxed);
+  const bool edge_on = edge_opt >= 0 ? edge_opt != 0 : edge_env;
   const bool edge = !full && edge_on && (A_KS || B_KS) && !SYM && edge_loop_ok(d, n, BT);
   long long blocks = 0;
   for (int g = 0; g < n; ++g) {
@@ -243,9 +250,6 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   // K = 4096 (bA + cAA: 2 % faster with it).  DION_AMD_DIAG_K overrides the limit (0: never).
   static const int diag_k_env = [] { const char* e = getenv("DION_AMD_DIAG_K"); return e ? atoi(e) : -1; }();
   args.diag_k = diag_k_env >= 0 ? diag_k_env : (blocks <= 4LL * da_cu_count() ? 0x7fffffff : 4096);
-  if (!full && !edge)   // the bounds-checked K loop walks A with a pointer: no wrap-around there
-    for (int g = 0; g < n; ++g)
-      if (d[g].a_kwrap) return DA_ERR_ARG;
   for (int g = 0; g < n; ++g)   // the weight-update epilogue exists for interior tiles of plain bf16 AXPBY products
     if (d[g].upd_tab && (!full || SYM || d[g].c_dtype != DA_BF16 || d[g].epilogue != DA_EPI_AXPBY)) return DA_ERR_ARG;
   hipLaunchKernelGGL(full ? kfull : (edge ? kedge : kgen), dim3((unsigned)blocks), dim3(C::NT), smem, stream, args);
@@ -360,6 +364,8 @@ int da_gemm_bf16_grouped(const GemmDesc* din, int n, hipStream_t stream) {
   if (choose_tile(d, n) == 256) return dispatch_layout<Big>(d, n, stream);
   return dispatch_layout<Small>(d, n, stream);
 }
+
+void da_gemm_bf16_set_edge_loop(int v) { g_opt_edge_loop.store(v < 0 ? -1 : (v != 0), std::memory_order_relaxed); }
 
 // What the launcher would do with one product of these dimensions, without launching anything:
 // tile edge (128 or 256), plus 1 if the K loop is the direct-to-LDS one.

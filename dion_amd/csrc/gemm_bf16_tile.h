@@ -529,6 +529,7 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
       rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;                    \
     }                                                                                              \
     sa.g += sa.tstep;                                                                              \
+    if (!A_KS && d.a_kwrap && (((kt) + 1) * BK) % d.a_kwrap == 0) sa.g -= d.a_kwrap;               \
     sb.g += sb.tstep;                                                                              \
   } while (0)
 #define DA_LSTORE(st)                                                                              \
@@ -672,6 +673,7 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
         rb[i] = ok ? *reinterpret_cast<const u32x4_t*>(sb.g + i * sb.gstep) : z_;
       }
       sa.g += sa.tstep;
+      if (!A_KS && d.a_kwrap && ((kt + 1) * BK) % d.a_kwrap == 0) sa.g -= d.a_kwrap;   // A again from its first column
       sb.g += sb.tstep;
     };
     auto lstore = [&](char* st) {

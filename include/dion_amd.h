@@ -374,6 +374,9 @@ int dion_amd_profile_read(int kind, long long* launches, double* total_ms, doubl
  *                   dimensions multiples of 256); 2 the same with an L2 write-back after every tile (cross-check);
  *                   -1 the default: DION_AMD_NS_FLOW in the environment if set, else the persistent launch for
  *                   workloads of many small matrices.  All give the same bits.
+ *   "edge_loop"     bf16 products with a ragged dimension on a k-strided operand (Dion's rank-r products at r = 192):
+ *                   1 the direct-to-LDS K loop with edge tiles, 0 the bounds-checked K loop, -1 the default (1 unless
+ *                   DION_AMD_NO_EDGE_LOOP is set in the environment).  Both give the same bits.
  *   "ns_flow_fail"  test hook: 1 makes every persistent launch start with its status word set, as if a wait had
  *                   run into its limit; the results of such a launch are NaN.
  * The value applies to calls that start after this one returns, on every thread.  Unknown name:

@@ -41,6 +41,27 @@ def test_orthonormalize(dev, rows, r, dtype):
     assert (torch.diagonal(Rm) > 0).all()
 
 
+@pytest.mark.parametrize("rows,r", [(768, 192), (2048, 320), (1024, 64)])
+def test_ragged_rank_products_same_bits_on_either_k_loop(dev, rows, r):
+    """The bf16 products of a rank that is not a whole number of tiles run the direct-to-LDS K loop with edge tiles;
+    the bounds-checked K loop (option "edge_loop" = 0) gives the same bits -- including the stacked product
+    `[P P] [T_hi; T_lo]`, whose A operand is read twice along k."""
+    from dion_amd import _lib
+    from dion_amd.newton_schulz import orthonormalize
+
+    torch.manual_seed(3)
+    P = (torch.randn(2, rows, r, dtype=torch.float64) * torch.logspace(0, -2, r, dtype=torch.float64)).to(torch.bfloat16).to(dev)
+    try:
+        _lib.set_option("edge_loop", 1)
+        Q1, i1 = orthonormalize(P.clone(), return_info=True)
+        _lib.set_option("edge_loop", 0)
+        Q0, i0 = orthonormalize(P.clone(), return_info=True)
+    finally:
+        _lib.set_option("edge_loop", -1)
+    assert bool((i1 == 0).all()) and bool((i0 == 0).all())
+    assert torch.equal(Q1, Q0)
+
+
 @pytest.mark.parametrize("rows,r,batch", [(1536, 200, 3), (1024, 72, 2), (2048, 192, 4), (3072, 520, 1),
                                           (16384, 256, 1), (12296, 136, 2)])
 def test_orthonormalize_bf16_ragged_ranks(dev, rows, r, batch):
