@@ -569,9 +569,9 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
   constexpr int TH = TMI / 2;
   // Measurement builds (-DDA_KLOOP_ABLATE=<bits>, WRONG RESULTS): what the direct-to-LDS loop costs without 1 its
   // fragment reads (the first stage's are kept), 2 its staging loads (after the first two stages), 4 the per-stage
-  // wait and barrier.
+  // wait and barrier, 8 its matrix-core instructions.
   constexpr bool ABL_READ = (DA_KLOOP_ABLATE & 1) != 0, ABL_DMA = (DA_KLOOP_ABLATE & 2) != 0,
-                 ABL_BAR = (DA_KLOOP_ABLATE & 4) != 0;
+                 ABL_BAR = (DA_KLOOP_ABLATE & 4) != 0, ABL_MMA = (DA_KLOOP_ABLATE & 8) != 0;
   bool abl_first = true;
 #define DA16_RA(FA, st, ks, h)                                                                     \
   do {                                                                                             \
@@ -589,10 +589,15 @@ __device__ __forceinline__ void gemm_tile_k_loop(typename C::acc_t (&acc)[C::TMI
   } while (0)
 #define DA16_MMA(FA, FB, h)                                                                        \
   do {                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TH; ++i)                                                 \
-        _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                            \
-            acc[(h) * TH + i][j] =                                                                 \
-                __builtin_amdgcn_mfma_f32_16x16x32_bf16(FB[j], FA[i], acc[(h) * TH + i][j], 0, 0, 0); \
+    if (FULL && ABL_MMA) {   /* the fragments are consumed (waited for), nothing is computed */   \
+      _Pragma("unroll") for (int i = 0; i < TH; ++i) asm volatile("" ::"v"(FA[i]));               \
+      _Pragma("unroll") for (int j = 0; j < TNJ; ++j) asm volatile("" ::"v"(FB[j]));              \
+    } else {                                                                                       \
+      _Pragma("unroll") for (int i = 0; i < TH; ++i)                                               \
+          _Pragma("unroll") for (int j = 0; j < TNJ; ++j)                                          \
+              acc[(h) * TH + i][j] =                                                               \
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(FB[j], FA[i], acc[(h) * TH + i][j], 0, 0, 0); \
+    }                                                                                              \
   } while (0)
   if (FULL) {
 #define DA16_DMA(st)                                                                               \
