@@ -46,6 +46,7 @@ struct GemmArgs {
   int n;
   int trace;   // 1: every workgroup records its time stamps (measurement hook)
   int diag_k;  // diagonal tiles of a symmetric product stage one panel for both operands when K is at most this
+  int interleave;   // bit g: group g's tiles are dealt to the XCDs in turns (see decode_tile)
 };
 
 // Which output tile a workgroup owns.  Workgroups are dealt round-robin to the 8 XCDs (each
@@ -54,11 +55,23 @@ struct GemmArgs {
 struct TileId { int b, ti, tj; };
 
 template <int BT, bool SYM>
-__device__ __forceinline__ TileId decode_tile(const GemmDesc& d, int bid, int nblk, bool xcd_aligned) {
+__device__ __forceinline__ TileId decode_tile(const GemmDesc& d, int bid, int nblk, bool xcd_aligned, int interleave) {
   const int tiles_m = (d.M + BT - 1) / BT;
   const int tiles_n = (d.N + BT - 1) / BT;
   const int per_batch = SYM ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
-  if (xcd_aligned && (nblk & 7) == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  if (xcd_aligned && (nblk & 7) == 0) {
+    // `interleave`: the XCDs take turns at runs of G logical tiles (a super-tile; an eighth of a symmetric matrix), so
+    // that all eight work on the same matrix at the same time; otherwise each XCD owns a contiguous eighth of the launch
+    const bool sup = !SYM && (((tiles_m % 8) == 0 && (tiles_n % 4) == 0) || ((tiles_m % 4) == 0 && (tiles_n % 8) == 0));
+    const int G = sup ? 32 : ((SYM && (per_batch & 7) == 0) ? per_batch >> 3 : 0);
+    const int nfull = (interleave && G > 0) ? nblk - nblk % (8 * G) : 0;
+    if (bid < nfull) {
+      const int xcd = bid & 7, idx = bid >> 3;
+      bid = ((idx / G) * 8 + xcd) * G + idx % G;
+    } else {   // (the rest of the launch, or all of it: a contiguous eighth per XCD)
+      bid = nfull + ((bid - nfull) & 7) * ((nblk - nfull) >> 3) + ((bid - nfull) >> 3);
+    }
+  }
   TileId r;
   r.b = bid / per_batch;
   int t = bid - r.b * per_batch;
@@ -72,8 +85,12 @@ __device__ __forceinline__ TileId decode_tile(const GemmDesc& d, int bid, int nb
     // 4 B panels (12 panel loads per k-step instead of 33 for a row of 32 tiles); measured 3-7 %
     // faster than row-major order on 4096 x 14336, and a little better than 4 x 8
     const int sup = t >> 5, within = t & 31;
-    const int sup_per_row = tiles_n >> 2;
-    const int sr = sup / sup_per_row, sc = sup - sr * sup_per_row;
+    const int sup_per_row = tiles_n >> 2, sup_rows = tiles_m >> 3;
+    int sr, sc;
+    // (dealt in turns, the eight XCDs then cover whole columns of super-tiles: a B panel is in use by all the XCDs
+    // that need it at the same time)
+    if (interleave) { sc = sup / sup_rows; sr = sup - sc * sup_rows; }
+    else { sr = sup / sup_per_row; sc = sup - sr * sup_per_row; }
     r.ti = sr * 8 + (within >> 2);
     r.tj = sc * 4 + (within & 3);
   } else if ((tiles_m % 4) == 0 && (tiles_n % 8) == 0) {
@@ -129,7 +146,7 @@ __global__ __launch_bounds__(C::NT) void gemm_bf16_kernel(GemmArgs args) {
   const int lane = tid & 63;
   const int wave = wave_uniform(tid >> 6);
   const int wm = wave / C::WGN, wn = wave % C::WGN;
-  const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0);
+  const TileId tile = decode_tile<BT, SYM>(d, (int)blockIdx.x - blk0, args.start[grp + 1] - blk0, (blk0 & 7) == 0, (args.interleave >> grp) & 1);
   const int ti = tile.ti, tj = tile.tj;
   // with K slices the tile index counts (slice, matrix) pairs: the slice's partial product is matrix tile.b of C
   int b = tile.b, dK = d.K;
@@ -248,6 +265,17 @@ int launch(const GemmDesc* d, int n, hipStream_t stream) {
   // rounds that shortens the tail (Llama-8B layer: X X^T 0.81 -> 0.77 ms); over many rounds of a long K the tiles
   // lose each other in the L2 (32 x 4096 x 14336: 1.7 x the fetched bytes, 6.93 -> 7.35 ms), so there only up to
   // K = 4096 (bA + cAA: 2 % faster with it).  DION_AMD_DIAG_K overrides the limit (0: never).
+  // With a contiguous eighth of the launch per XCD the eight XCDs work on eight different matrices.  A launch whose
+  // operands exceed the 256 MB Infinity Cache has the XCDs take turns at the tiles of one matrix instead: a panel then
+  // comes from HBM once and for the other XCDs from that cache (32 x 4096 x 14336: X' = aX + BX 13.5 -> 13.0 ms,
+  // X X^T 7.0 -> 6.8 ms; all Newton-Schulz products of Llama-3-8B 443 -> 437 ms per step; launches of a few matrices
+  // are up to 1 % faster without).  DION_AMD_XCD_INTERLEAVE=0|1 overrides the rule.
+  static const int il_env = [] { const char* e = getenv("DION_AMD_XCD_INTERLEAVE"); return e ? atoi(e) : -1; }();
+  args.interleave = 0;
+  for (int g = 0; g < n; ++g) {
+    const double bytes = 2.0 * d[g].batch * ((double)d[g].M * d[g].K + (SYM ? 0.0 : (double)d[g].N * d[g].K));
+    if (il_env >= 0 ? il_env != 0 : bytes > 512.0 * 1048576.0) args.interleave |= 1 << g;
+  }
   static const int diag_k_env = [] { const char* e = getenv("DION_AMD_DIAG_K"); return e ? atoi(e) : -1; }();
   args.diag_k = diag_k_env >= 0 ? diag_k_env : (blocks <= 4LL * da_cu_count() ? 0x7fffffff : 4096);
   for (int g = 0; g < n; ++g)   // the weight-update epilogue exists for interior tiles of plain bf16 AXPBY products
